@@ -1,0 +1,184 @@
+"""Compiles the native libraries in-tree and loads them through ctypes.
+
+Two kinds of library live under ``csrc/``: the host runtime (``host/*.cpp``, plain
+C++ built with g++: cache manager, scheduler, sampler) and the device kernels
+(``hip/*.hip``, built with hipcc for gfx950, one shared object per source file so
+that a run compiles only the groups it uses).  Built objects go to
+``glassbox_amd/_lib`` with a stamp of the hash of their sources and flags; a
+stale or missing object is rebuilt on first use, with a progress line every few
+seconds.  If the package folder cannot be written, a per-user folder under the
+temporary directory is used instead.
+"""
+from __future__ import annotations
+
+import ctypes
+import hashlib
+import os
+import shutil
+import subprocess
+import sys
+import tempfile
+import threading
+import time
+from concurrent.futures import ThreadPoolExecutor
+from typing import Dict, List, Optional
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+_CSRC = os.path.join(_HERE, "csrc")
+_ARCH = "gfx950"
+
+HIP_FLAGS = [
+    f"--offload-arch={_ARCH}", "-O3", "-std=c++17", "-fPIC", "-shared", "-fno-gpu-rdc",
+    # packed fp32 instructions off: some of their forms have given wrong results on these machines
+    "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+    "-Wno-unused-result", "-Wno-unknown-warning-option",
+]
+HOST_FLAGS = ["-O2", "-std=c++17", "-fPIC", "-shared", "-Wall"]
+
+#: name -> (compiler kind, sources relative to csrc, extra dependencies hashed with them)
+LIBRARIES: Dict[str, tuple] = {
+    "host": ("host", ["host/cache_manager.cpp", "host/scheduler.cpp", "host/c_api.cpp"],
+             ["host/cache_manager.h", "host/scheduler.h", "host/sampler.h"]),
+    "elementwise": ("hip", ["hip/elementwise.hip"], ["hip/common.h"]),
+    "gemm_f32": ("hip", ["hip/gemm_f32.hip"], ["hip/common.h"]),
+    "gemm_bf16": ("hip", ["hip/gemm_bf16.hip"], ["hip/common.h"]),
+    "attention_plain": ("hip", ["hip/attention_plain.hip"], ["hip/common.h"]),
+    "attention_bf16": ("hip", ["hip/attention_bf16.hip"], ["hip/common.h"]),
+    "sampling": ("hip", ["hip/sampling.hip"], ["hip/common.h"]),
+}
+
+_lock = threading.Lock()
+_loaded: Dict[str, ctypes.CDLL] = {}
+
+
+class BuildError(RuntimeError):
+    pass
+
+
+def _say(msg: str) -> None:
+    print(f"[glassbox_amd] {msg}", file=sys.stderr, flush=True)
+
+
+def _hipcc() -> str:
+    for cand in (os.environ.get("HIPCC"), shutil.which("hipcc"), "/opt/rocm/bin/hipcc"):
+        if cand and os.path.exists(cand):
+            return cand
+    raise BuildError("hipcc not found (looked at $HIPCC, PATH and /opt/rocm/bin): the device kernels cannot be built")
+
+
+def _lib_dir() -> str:
+    d = os.path.join(_HERE, "_lib")
+    try:
+        os.makedirs(d, exist_ok=True)
+        probe = os.path.join(d, f".w{os.getpid()}")
+        with open(probe, "w"):
+            pass
+        os.remove(probe)
+        return d
+    except OSError:
+        d = os.path.join(tempfile.gettempdir(), f"glassbox_amd-{os.getuid()}", "_lib")
+        os.makedirs(d, exist_ok=True)
+        return d
+
+
+def _digest(name: str) -> str:
+    kind, sources, deps = LIBRARIES[name]
+    h = hashlib.sha256()
+    h.update(" ".join(HIP_FLAGS if kind == "hip" else HOST_FLAGS).encode())
+    for rel in list(sources) + list(deps):
+        with open(os.path.join(_CSRC, rel), "rb") as fh:
+            h.update(rel.encode())
+            h.update(fh.read())
+    return h.hexdigest()[:16]
+
+
+def lib_path(name: str) -> str:
+    return os.path.join(_lib_dir(), f"libgb_{name}.so")
+
+
+def is_current(name: str) -> bool:
+    path = lib_path(name)
+    stamp = path + ".stamp"
+    if not (os.path.exists(path) and os.path.exists(stamp)):
+        return False
+    try:
+        with open(stamp) as fh:
+            return fh.read().strip() == _digest(name)
+    except OSError:
+        return False
+
+
+def compile_library(name: str, quiet: bool = False) -> str:
+    """Compile one library now, whatever is there.  Returns the path of the shared object."""
+    kind, sources, _ = LIBRARIES[name]
+    out = lib_path(name)
+    tmp = f"{out}.{os.getpid()}.{threading.get_ident()}.tmp"
+    srcs = [os.path.join(_CSRC, s) for s in sources]
+    if kind == "hip":
+        cmd = [_hipcc()] + HIP_FLAGS + srcs + ["-o", tmp]
+    else:
+        cxx = os.environ.get("CXX") or shutil.which("g++") or shutil.which("c++") or _hipcc()
+        cmd = [cxx] + HOST_FLAGS + srcs + ["-o", tmp]
+    env = dict(os.environ)
+    env.setdefault("TMPDIR", tempfile.gettempdir())
+    if not env.get("HOME") or not os.access(env.get("HOME", "/"), os.W_OK):
+        env["HOME"] = tempfile.gettempdir()  # the compiler driver wants a writable home for its caches
+    t0 = time.time()
+    if not quiet:
+        _say(f"compiling {name} ({', '.join(sources)}) ...")
+    proc = subprocess.Popen(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, env=env, cwd=_CSRC)
+    done = threading.Event()
+
+    def ticker():
+        while not done.wait(10.0):
+            _say(f"  still compiling {name}: {time.time() - t0:.0f} s")
+
+    th = threading.Thread(target=ticker, daemon=True)
+    th.start()
+    log = proc.communicate()[0].decode(errors="replace")
+    done.set()
+    if proc.returncode != 0:
+        try:
+            os.remove(tmp)
+        except OSError:
+            pass
+        lines = [l for l in log.splitlines() if "packed-fp32-ops" not in l]
+        raise BuildError(f"building {name} failed ({' '.join(cmd)}):\n" + "\n".join(lines[-60:]))
+    os.replace(tmp, out)
+    with open(out + ".stamp", "w") as fh:
+        fh.write(_digest(name))
+    if not quiet:
+        _say(f"built {name} in {time.time() - t0:.1f} s")
+    return out
+
+
+def build_all(force: bool = True, names: Optional[List[str]] = None, jobs: int = 8) -> None:
+    """Compile every library (or ``names``).  With ``force`` also those that are current."""
+    todo = [n for n in (names or list(LIBRARIES)) if force or not is_current(n)]
+    if not todo:
+        return
+    with ThreadPoolExecutor(max_workers=max(1, min(jobs, len(todo)))) as pool:
+        list(pool.map(compile_library, todo))
+
+
+def load(name: str) -> ctypes.CDLL:
+    """The library ``name``, compiled first if it is missing or older than its sources."""
+    with _lock:
+        lib = _loaded.get(name)
+        if lib is not None:
+            return lib
+        if name not in LIBRARIES:
+            raise BuildError(f"no native library called {name!r}")
+        if not is_current(name):
+            compile_library(name)
+        try:
+            lib = ctypes.CDLL(lib_path(name))
+        except OSError as e:
+            raise BuildError(f"cannot load {lib_path(name)}: {e}") from None
+        _loaded[name] = lib
+        return lib
+
+
+def ensure(names: List[str]) -> None:
+    """Compile, in parallel, those of ``names`` that are missing or stale (no loading)."""
+    build_all(force=False, names=names)

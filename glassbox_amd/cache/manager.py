@@ -1,0 +1,206 @@
+"""Python face of the host cache manager (csrc/host/cache_manager.cpp).
+
+The manager decides which pages of which pool belong to which request; it owns
+no device memory (``cache/pools.py`` does).  Requests are named by integers.
+"""
+from __future__ import annotations
+
+import ctypes as C
+from dataclasses import dataclass
+from typing import List, Sequence, Tuple
+
+from .. import build
+
+FULL, WINDOW = 0, 1
+
+
+class OutOfPages(RuntimeError):
+    """reserve() found too few free pages; nothing was changed."""
+
+
+class CacheError(RuntimeError):
+    pass
+
+
+@dataclass(frozen=True)
+class GroupSpec:
+    """One pool of pages: ``kind`` FULL keeps every key, WINDOW only the last ``window``."""
+    kind: int = FULL
+    window: int = 0
+    num_pages: int = 0
+
+
+_lib = None
+
+
+def _host():
+    global _lib
+    if _lib is None:
+        lib = build.load("host")
+        i32p, i64 = C.POINTER(C.c_int32), C.c_int64
+        lib.gbh_cache_create.restype = C.c_void_p
+        lib.gbh_cache_create.argtypes = [C.c_int, C.c_int, C.POINTER(C.c_int), C.POINTER(C.c_int),
+                                         C.POINTER(C.c_int), C.c_int, C.c_int]
+        lib.gbh_cache_destroy.argtypes = [C.c_void_p]
+        lib.gbh_cache_destroy.restype = None
+        for name, args in {
+            "add_seq": [i64, i32p, C.c_int], "reserve": [i64, C.c_int], "commit": [i64, i32p, C.c_int],
+            "truncate": [i64, C.c_int], "fork": [i64, i64], "remove_seq": [i64], "has_seq": [i64],
+            "seq_len": [i64], "state_slot": [i64], "free_pages": [C.c_int], "min_free_pages": [],
+            "num_pages": [C.c_int], "ref_count": [C.c_int, C.c_int], "free_state_slots": [],
+            "num_seqs": [], "share_prefixes": [], "pages_needed": [i64, C.c_int],
+            "table": [i64, C.c_int, i32p, C.c_int], "take_copies": [i32p, C.c_int],
+            "check": [C.c_char_p, C.c_int],
+        }.items():
+            fn = getattr(lib, "gbh_cache_" + name)
+            fn.argtypes = [C.c_void_p] + args
+            fn.restype = C.c_int
+        lib.gbh_chain_hash.restype = C.c_uint64
+        lib.gbh_chain_hash.argtypes = [C.c_uint64, i32p, C.c_int]
+        _lib = lib
+    return _lib
+
+
+def _ints(values: Sequence[int]):
+    arr = (C.c_int32 * max(1, len(values)))(*values)
+    return arr
+
+
+def chain_hash(prev: int, tokens: Sequence[int]) -> int:
+    return int(_host().gbh_chain_hash(prev, _ints(tokens), len(tokens)))
+
+
+class CacheManager:
+    def __init__(self, page_size: int, groups: Sequence[GroupSpec], num_state_slots: int = 0,
+                 share_prefixes: bool = True):
+        if page_size <= 0:
+            raise CacheError("page_size must be positive")
+        for g in groups:
+            if g.kind == WINDOW and g.window <= 0:
+                raise CacheError("a window group needs a positive window")
+            if g.num_pages <= 0:
+                raise CacheError("every page group needs at least one page")
+        self._lib = _host()
+        self.page_size = page_size
+        self.groups = list(groups)
+        self.num_state_slots = num_state_slots
+        n = len(groups)
+        mk = lambda vals: (C.c_int * max(1, n))(*vals)
+        self._h = C.c_void_p(self._lib.gbh_cache_create(
+            page_size, n, mk([g.kind for g in groups]), mk([g.window for g in groups]),
+            mk([g.num_pages for g in groups]), num_state_slots, 1 if share_prefixes else 0))
+        self._table_buf = (C.c_int32 * 64)()
+
+    def __del__(self):
+        h, self._h = getattr(self, "_h", None), None
+        if h:
+            self._lib.gbh_cache_destroy(h)
+
+    @property
+    def handle(self):
+        return self._h
+
+    # requests ---------------------------------------------------------------
+    def add_seq(self, seq_id: int, prompt: Sequence[int] = ()) -> int:
+        r = self._lib.gbh_cache_add_seq(self._h, seq_id, _ints(prompt), len(prompt))
+        if r == -1:
+            raise CacheError(f"request {seq_id} exists")
+        if r == -2:
+            raise CacheError("no state slot is free")
+        return r
+
+    def reserve(self, seq_id: int, n: int) -> None:
+        r = self._lib.gbh_cache_reserve(self._h, seq_id, n)
+        if r == 1:
+            raise OutOfPages(f"request {seq_id}: no room for {n} more tokens")
+        if r != 0:
+            raise CacheError(f"unknown request {seq_id}")
+
+    def commit(self, seq_id: int, tokens: Sequence[int]) -> None:
+        if self._lib.gbh_cache_commit(self._h, seq_id, _ints(tokens), len(tokens)) != 0:
+            raise CacheError(f"unknown request {seq_id}")
+
+    def truncate(self, seq_id: int, length: int) -> None:
+        r = self._lib.gbh_cache_truncate(self._h, seq_id, length)
+        if r == -1:
+            raise CacheError(f"unknown request {seq_id}")
+        if r == -2:
+            raise CacheError(f"request {seq_id}: cannot truncate to {length}")
+        if r == -3:
+            raise CacheError(f"request {seq_id}: a window's pages before {length} were already given back")
+
+    def fork(self, parent: int, child: int) -> None:
+        r = self._lib.gbh_cache_fork(self._h, parent, child)
+        if r != 0:
+            raise CacheError({-1: f"unknown request {parent}", -2: f"request {child} exists",
+                              -3: "no state slot is free"}.get(r, "fork failed"))
+
+    def remove_seq(self, seq_id: int) -> None:
+        self._lib.gbh_cache_remove_seq(self._h, seq_id)
+
+    # queries ----------------------------------------------------------------
+    def has_seq(self, seq_id: int) -> bool:
+        return bool(self._lib.gbh_cache_has_seq(self._h, seq_id))
+
+    def seq_len(self, seq_id: int) -> int:
+        r = self._lib.gbh_cache_seq_len(self._h, seq_id)
+        if r < 0:
+            raise CacheError(f"unknown request {seq_id}")
+        return r
+
+    def state_slot(self, seq_id: int) -> int:
+        return self._lib.gbh_cache_state_slot(self._h, seq_id)
+
+    def table(self, seq_id: int, group: int = 0) -> List[int]:
+        n = self._lib.gbh_cache_table(self._h, seq_id, group, self._table_buf, len(self._table_buf))
+        if n < 0:
+            raise CacheError(f"unknown request {seq_id} or group {group}")
+        if n > len(self._table_buf):
+            self._table_buf = (C.c_int32 * (2 * n))()
+            n = self._lib.gbh_cache_table(self._h, seq_id, group, self._table_buf, len(self._table_buf))
+        return self._table_buf[:n]
+
+    def slot(self, seq_id: int, pos: int, group: int = 0) -> int:
+        """Row of (request, position) in a layer's pages (kv.rs:199-201)."""
+        return self.table(seq_id, group)[pos // self.page_size] * self.page_size + pos % self.page_size
+
+    def free_pages(self, group: int = 0) -> int:
+        return self._lib.gbh_cache_free_pages(self._h, group)
+
+    def min_free_pages(self) -> int:
+        return self._lib.gbh_cache_min_free_pages(self._h)
+
+    def num_pages(self, group: int = 0) -> int:
+        return self._lib.gbh_cache_num_pages(self._h, group)
+
+    def used_pages(self, group: int = 0) -> int:
+        return self.num_pages(group) - self.free_pages(group)
+
+    def ref_count(self, page: int, group: int = 0) -> int:
+        return self._lib.gbh_cache_ref_count(self._h, group, page)
+
+    def free_state_slots(self) -> int:
+        return self._lib.gbh_cache_free_state_slots(self._h)
+
+    def num_seqs(self) -> int:
+        return self._lib.gbh_cache_num_seqs(self._h)
+
+    @property
+    def share_prefixes(self) -> bool:
+        return bool(self._lib.gbh_cache_share_prefixes(self._h))
+
+    def pages_needed(self, seq_id: int, n: int) -> int:
+        return self._lib.gbh_cache_pages_needed(self._h, seq_id, n)
+
+    def take_copies(self) -> List[Tuple[int, int, int]]:
+        """Pending device copies (group, src, dst); group -1 means a state slot."""
+        buf = (C.c_int32 * (3 * 64))()
+        n = self._lib.gbh_cache_take_copies(self._h, buf, 64)
+        if n > 64:
+            raise CacheError("more pending copies than the buffer holds")
+        return [(buf[3 * i], buf[3 * i + 1], buf[3 * i + 2]) for i in range(n)]
+
+    def check_invariants(self) -> None:
+        why = C.create_string_buffer(1024)
+        if not self._lib.gbh_cache_check(self._h, why, 1024):
+            raise AssertionError("cache invariants broken: " + why.value.decode())

@@ -1,0 +1,107 @@
+// Shared by every device library: element types, conversions, wave and block
+// reductions, and the error channel of the C entry points.
+//
+// Every entry point is `extern "C" int gb_*(...)`: it checks on the host that the
+// operand shapes fit what the kernel and its grid assume, launches on the given
+// stream and returns 0, or returns 1 after leaving a message for gb_last_error().
+#pragma once
+#include <hip/hip_runtime.h>
+
+#include <cstdarg>
+#include <cstdint>
+#include <cstdio>
+#include <string>
+
+namespace gb {
+
+typedef __bf16 bf16;
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef __bf16 bf16x4 __attribute__((ext_vector_type(4)));
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+typedef float f32x16 __attribute__((ext_vector_type(16)));
+
+constexpr int kWave = 64;
+
+// dtype codes shared with the Python side
+enum : int { kF32 = 0, kBF16 = 1 };
+
+__device__ __forceinline__ float to_f(float v) { return v; }
+__device__ __forceinline__ float to_f(bf16 v) { return (float)v; }
+template <typename T> __device__ __forceinline__ T from_f(float v);
+template <> __device__ __forceinline__ float from_f<float>(float v) { return v; }
+template <> __device__ __forceinline__ bf16 from_f<bf16>(float v) { return (bf16)v; }  // round to nearest even
+
+__device__ __forceinline__ float wave_sum(float v) {
+#pragma unroll
+  for (int o = kWave / 2; o > 0; o >>= 1) v += __shfl_xor(v, o, kWave);
+  return v;
+}
+__device__ __forceinline__ float wave_max(float v) {
+#pragma unroll
+  for (int o = kWave / 2; o > 0; o >>= 1) v = fmaxf(v, __shfl_xor(v, o, kWave));
+  return v;
+}
+
+// Sum over a block of up to 1024 threads; `scratch` holds at least 17 floats.  Every thread
+// gets the result.  The order of additions is fixed by the thread layout alone.
+__device__ __forceinline__ float block_sum(float v, float* scratch) {
+  const int lane = threadIdx.x % kWave, wave = threadIdx.x / kWave;
+  const int waves = (blockDim.x + kWave - 1) / kWave;
+  v = wave_sum(v);
+  __syncthreads();
+  if (lane == 0) scratch[wave] = v;
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    float t = 0.f;
+    for (int w = 0; w < waves; ++w) t += scratch[w];
+    scratch[16] = t;
+  }
+  __syncthreads();
+  return scratch[16];
+}
+__device__ __forceinline__ float block_max(float v, float* scratch) {
+  const int lane = threadIdx.x % kWave, wave = threadIdx.x / kWave;
+  const int waves = (blockDim.x + kWave - 1) / kWave;
+  v = wave_max(v);
+  __syncthreads();
+  if (lane == 0) scratch[wave] = v;
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    float t = scratch[0];
+    for (int w = 1; w < waves; ++w) t = fmaxf(t, scratch[w]);
+    scratch[16] = t;
+  }
+  __syncthreads();
+  return scratch[16];
+}
+
+inline std::string& last_error() {
+  static thread_local std::string msg;
+  return msg;
+}
+
+inline int fail(const char* fmt, ...) {
+  char buf[512];
+  va_list ap;
+  va_start(ap, fmt);
+  vsnprintf(buf, sizeof buf, fmt, ap);
+  va_end(ap);
+  last_error() = buf;
+  return 1;
+}
+
+inline int launched(const char* what) {
+  hipError_t e = hipGetLastError();
+  if (e != hipSuccess) return fail("%s: launch failed: %s", what, hipGetErrorString(e));
+  return 0;
+}
+
+}  // namespace gb
+
+#define GB_REQUIRE(cond, ...) \
+  do {                        \
+    if (!(cond)) return gb::fail(__VA_ARGS__); \
+  } while (0)
+
+#define GB_DEFINE_LAST_ERROR \
+  extern "C" const char* gb_last_error() { return gb::last_error().c_str(); }

@@ -1,0 +1,210 @@
+// Memory-bound parts of a decoder step, in 32-bit and bfloat16 storage: embedding
+// gather, RMS norm, rotary table, rotation fused with the cache write, SiLU-multiply,
+// and page copies.  All arithmetic is 32-bit; only loads and stores differ by type.
+#include "common.h"
+
+using namespace gb;
+
+GB_DEFINE_LAST_ERROR
+
+// ---------------------------------------------------------------- embedding gather
+// x[i, :] = table[ids[i], :]   (crates/glassbox-core/src/model.rs:228-231)
+template <typename T>
+__global__ void embed_kernel(const T* __restrict__ table, const int32_t* __restrict__ ids, float* __restrict__ x,
+                             int d, int vocab) {
+  const int i = blockIdx.x;
+  int id = ids[i];
+  const bool ok = id >= 0 && id < vocab;
+  const T* row = table + (size_t)(ok ? id : 0) * d;
+  for (int c = threadIdx.x; c < d; c += blockDim.x)
+    x[(size_t)i * d + c] = ok ? to_f(row[c]) : __builtin_nanf("");  // a bad id must not pass silently
+}
+
+extern "C" int gb_embed(const void* table, int table_dtype, const int32_t* ids, float* x, int n, int d, int vocab,
+                        hipStream_t stream) {
+  GB_REQUIRE(n >= 0 && d > 0 && vocab > 0, "embed: bad sizes n=%d d=%d vocab=%d", n, d, vocab);
+  if (n == 0) return 0;
+  const int threads = d >= 256 ? 256 : 64;
+  if (table_dtype == kF32)
+    hipLaunchKernelGGL(embed_kernel<float>, dim3(n), dim3(threads), 0, stream, (const float*)table, ids, x, d, vocab);
+  else if (table_dtype == kBF16)
+    hipLaunchKernelGGL(embed_kernel<bf16>, dim3(n), dim3(threads), 0, stream, (const bf16*)table, ids, x, d, vocab);
+  else
+    return fail("embed: unknown table dtype %d", table_dtype);
+  return launched("embed");
+}
+
+// ------------------------------------------------------------------------ RMS norm
+// ms = sum(x^2)/d ; s = 1/sqrt(ms + eps) ; out = g * (x * s)     (model.rs:94-100)
+// One block per output row; `rows` (optional) picks the input row of each output row.
+template <typename G, typename O>
+__global__ void rmsnorm_kernel(const float* __restrict__ x, const G* __restrict__ gamma, const int32_t* __restrict__ rows,
+                               O* __restrict__ out, int d, float eps) {
+  __shared__ float scratch[17];
+  const int r = blockIdx.x;
+  const float* xr = x + (size_t)(rows ? rows[r] : r) * d;
+  float ss = 0.f;
+  for (int c = threadIdx.x; c < d; c += blockDim.x) {
+    float v = xr[c];
+    ss += v * v;
+  }
+  ss = block_sum(ss, scratch);
+  const float s = 1.0f / sqrtf(ss / (float)d + eps);
+  for (int c = threadIdx.x; c < d; c += blockDim.x) out[(size_t)r * d + c] = from_f<O>(to_f(gamma[c]) * (xr[c] * s));
+}
+
+extern "C" int gb_rmsnorm(const float* x, const void* gamma, int gamma_dtype, const int32_t* rows, void* out,
+                          int out_dtype, int m, int d, float eps, hipStream_t stream) {
+  GB_REQUIRE(m >= 0 && d > 0, "rmsnorm: bad sizes m=%d d=%d", m, d);
+  if (m == 0) return 0;
+  const int threads = d >= 1024 ? 256 : (d >= 256 ? 128 : 64);
+#define GB_LAUNCH(G, O) \
+  hipLaunchKernelGGL((rmsnorm_kernel<G, O>), dim3(m), dim3(threads), 0, stream, x, (const G*)gamma, rows, (O*)out, d, eps)
+  if (gamma_dtype == kF32 && out_dtype == kF32) GB_LAUNCH(float, float);
+  else if (gamma_dtype == kF32 && out_dtype == kBF16) GB_LAUNCH(float, bf16);
+  else if (gamma_dtype == kBF16 && out_dtype == kF32) GB_LAUNCH(bf16, float);
+  else if (gamma_dtype == kBF16 && out_dtype == kBF16) GB_LAUNCH(bf16, bf16);
+  else return fail("rmsnorm: unknown dtypes gamma=%d out=%d", gamma_dtype, out_dtype);
+#undef GB_LAUNCH
+  return launched("rmsnorm");
+}
+
+// -------------------------------------------------------------------- rotary table
+// angle = f32(pos) * inv[i] as a 32-bit product; sin and cos of it evaluated in 64-bit and
+// rounded to 32-bit (model.rs:105-109).  inv comes from the host, computed as the reference does.
+__global__ void rope_table_kernel(const int32_t* __restrict__ pos, const float* __restrict__ inv,
+                                  float* __restrict__ cosv, float* __restrict__ sinv, int n, int half) {
+  const int idx = blockIdx.x * blockDim.x + threadIdx.x;
+  if (idx >= n * half) return;
+  const int t = idx / half, i = idx % half;
+  const float a = __fmul_rn((float)pos[t], inv[i]);
+  cosv[idx] = (float)cos((double)a);
+  sinv[idx] = (float)sin((double)a);
+}
+
+extern "C" int gb_rope_table(const int32_t* pos, const float* inv, float* cosv, float* sinv, int n, int half,
+                             hipStream_t stream) {
+  GB_REQUIRE(n >= 0 && half > 0, "rope_table: bad sizes n=%d half=%d", n, half);
+  if (n == 0) return 0;
+  const int total = n * half;
+  hipLaunchKernelGGL(rope_table_kernel, dim3((total + 255) / 256), dim3(256), 0, stream, pos, inv, cosv, sinv, n, half);
+  return launched("rope_table");
+}
+
+// ------------------------------------------------- rotation and cache write, fused
+// For token t: every query head and key head is rotated in half-split pairs (i, i + hd/2):
+//   x0' = x0 c - x1 s ; x1' = x1 c + x0 s                              (model.rs:110-113)
+// queries are rotated in place inside the stacked qkv row; rotated keys and plain values go to
+// the pages at slot[t] (model.rs:273-275).  Pages are [page][kv head][slot in page][hd].
+// With slots == nullptr nothing is stored (a layer that reads another layer's cache).
+// With n_rot_kv == 0 the row holds queries only.
+template <typename T>
+__global__ void rope_store_kernel(T* __restrict__ qkv, int row_stride, const float* __restrict__ cosv,
+                                  const float* __restrict__ sinv, const int32_t* __restrict__ slots,
+                                  T* __restrict__ k_pages, T* __restrict__ v_pages, int nh, int nkv, int hd,
+                                  int page_size, int rotate) {
+  const int t = blockIdx.x;
+  const int half = hd / 2;
+  T* row = qkv + (size_t)t * row_stride;
+  const float* c = cosv + (size_t)t * half;
+  const float* s = sinv + (size_t)t * half;
+  const int slot = slots ? slots[t] : -1;
+  const int page = slot >= 0 ? slot / page_size : 0, off = slot >= 0 ? slot % page_size : 0;
+  // queries, then keys: (nh + nkv) heads of `half` pairs
+  const int pairs = (nh + nkv) * half;
+  for (int p = threadIdx.x; p < pairs; p += blockDim.x) {
+    const int head = p / half, i = p % half;
+    T* h = row + (size_t)head * hd;
+    float x0 = to_f(h[i]), x1 = to_f(h[i + half]);
+    float y0 = x0, y1 = x1;
+    if (rotate) {
+      y0 = x0 * c[i] - x1 * s[i];
+      y1 = x1 * c[i] + x0 * s[i];
+    }
+    if (head < nh) {
+      h[i] = from_f<T>(y0);
+      h[i + half] = from_f<T>(y1);
+    } else {
+      h[i] = from_f<T>(y0);  // keep the rotated key in the row too: parts may read it back
+      h[i + half] = from_f<T>(y1);
+      if (slot >= 0) {
+        const int kvh = head - nh;
+        T* dst = k_pages + (((size_t)page * nkv + kvh) * page_size + off) * hd;
+        dst[i] = from_f<T>(y0);
+        dst[i + half] = from_f<T>(y1);
+      }
+    }
+  }
+  if (slot >= 0) {
+    const T* v = row + (size_t)(nh + nkv) * hd;
+    for (int e = threadIdx.x; e < nkv * hd; e += blockDim.x) {
+      const int kvh = e / hd, i = e % hd;
+      v_pages[(((size_t)page * nkv + kvh) * page_size + off) * hd + i] = v[e];
+    }
+  }
+}
+
+extern "C" int gb_rope_store(void* qkv, int dtype, int row_stride, const float* cosv, const float* sinv,
+                             const int32_t* slots, void* k_pages, void* v_pages, int n, int nh, int nkv, int hd,
+                             int page_size, int rotate, hipStream_t stream) {
+  GB_REQUIRE(n >= 0 && nh >= 0 && nkv >= 0 && hd > 0 && hd % 2 == 0, "rope_store: bad sizes n=%d nh=%d nkv=%d hd=%d", n, nh, nkv, hd);
+  GB_REQUIRE(row_stride >= (nh + 2 * nkv) * hd || (slots == nullptr && row_stride >= (nh + nkv) * hd),
+             "rope_store: row stride %d is shorter than the stacked heads", row_stride);
+  GB_REQUIRE(slots == nullptr || (k_pages && v_pages && page_size > 0), "rope_store: slots given without pages");
+  GB_REQUIRE(!rotate || (cosv && sinv), "rope_store: rotation asked without a table");
+  if (n == 0) return 0;
+  const int threads = (nh + nkv) * hd / 2 >= 256 ? 256 : 64;
+  if (dtype == kF32)
+    hipLaunchKernelGGL(rope_store_kernel<float>, dim3(n), dim3(threads), 0, stream, (float*)qkv, row_stride, cosv, sinv,
+                       slots, (float*)k_pages, (float*)v_pages, nh, nkv, hd, page_size, rotate);
+  else if (dtype == kBF16)
+    hipLaunchKernelGGL(rope_store_kernel<bf16>, dim3(n), dim3(threads), 0, stream, (bf16*)qkv, row_stride, cosv, sinv,
+                       slots, (bf16*)k_pages, (bf16*)v_pages, nh, nkv, hd, page_size, rotate);
+  else
+    return fail("rope_store: unknown dtype %d", dtype);
+  return launched("rope_store");
+}
+
+// ------------------------------------------------------------------- SiLU-multiply
+// act = g / (1 + exp(-g)) * u, gate in the first I columns, up in the last I (model.rs:336-340)
+template <typename T>
+__global__ void silu_mul_kernel(const T* __restrict__ gu, T* __restrict__ act, int n, int inter) {
+  const size_t idx = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (idx >= (size_t)n * inter) return;
+  const size_t t = idx / inter, c = idx % inter;
+  const float g = to_f(gu[t * 2 * inter + c]);
+  const float u = to_f(gu[t * 2 * inter + inter + c]);
+  act[idx] = from_f<T>(g / (1.0f + expf(-g)) * u);
+}
+
+extern "C" int gb_silu_mul(const void* gu, void* act, int dtype, int n, int inter, hipStream_t stream) {
+  GB_REQUIRE(n >= 0 && inter > 0, "silu_mul: bad sizes n=%d inter=%d", n, inter);
+  if (n == 0) return 0;
+  const size_t total = (size_t)n * inter;
+  const dim3 grid((unsigned)((total + 255) / 256));
+  if (dtype == kF32)
+    hipLaunchKernelGGL(silu_mul_kernel<float>, grid, dim3(256), 0, stream, (const float*)gu, (float*)act, n, inter);
+  else if (dtype == kBF16)
+    hipLaunchKernelGGL(silu_mul_kernel<bf16>, grid, dim3(256), 0, stream, (const bf16*)gu, (bf16*)act, n, inter);
+  else
+    return fail("silu_mul: unknown dtype %d", dtype);
+  return launched("silu_mul");
+}
+
+// ---------------------------------------------------------------------- row copies
+// base is [rows][row_bytes]; copies row src[i] onto row dst[i] (copy-on-write of a page in one
+// layer's pool, kv.rs:189-196, and copies of state slots).  row_bytes is a multiple of 4.
+__global__ void copy_rows_kernel(uint32_t* __restrict__ base, size_t row_words, const int32_t* __restrict__ src,
+                                 const int32_t* __restrict__ dst) {
+  const uint32_t* s = base + (size_t)src[blockIdx.x] * row_words;
+  uint32_t* d = base + (size_t)dst[blockIdx.x] * row_words;
+  for (size_t w = threadIdx.x; w < row_words; w += blockDim.x) d[w] = s[w];
+}
+
+extern "C" int gb_copy_rows(void* base, long long row_bytes, const int32_t* src, const int32_t* dst, int count,
+                            hipStream_t stream) {
+  GB_REQUIRE(row_bytes > 0 && row_bytes % 4 == 0, "copy_rows: row of %lld bytes is not a multiple of 4", row_bytes);
+  if (count <= 0) return 0;
+  hipLaunchKernelGGL(copy_rows_kernel, dim3(count), dim3(256), 0, stream, (uint32_t*)base, (size_t)(row_bytes / 4), src, dst);
+  return launched("copy_rows");
+}

@@ -1,0 +1,79 @@
+"""What one step carries to the parts: the batch's rows and their metadata on the device.
+
+A step is a flat batch of tokens from several requests, portions of prompts beside single
+decoded tokens (crates/glassbox-core/src/model.rs:203-215).  Per token: id, position, request
+index, and the cache row to write in each page group.  Per request: first row, row count,
+first position, state slot, and its block table in each group.  All integer metadata travels
+in one pinned host buffer and one copy.
+"""
+from __future__ import annotations
+
+from typing import Dict, List, Optional, Sequence, Tuple
+
+import torch
+
+from .. import ops
+
+
+class Workspace:
+    """Named device buffers that grow when a step needs more and are otherwise reused, so a step
+    allocates nothing once sizes have been seen (which also keeps graph capture simple)."""
+
+    def __init__(self, device):
+        self.device = device
+        self._flat: Dict[Tuple[str, torch.dtype], torch.Tensor] = {}
+
+    def buffer(self, name: str, shape: Sequence[int], dtype: torch.dtype) -> torch.Tensor:
+        count = 1
+        for s in shape:
+            count *= int(s)
+        key = (name, dtype)
+        flat = self._flat.get(key)
+        if flat is None or flat.numel() < count:
+            if torch.cuda.is_current_stream_capturing():
+                raise RuntimeError(f"workspace buffer {name!r} would have to grow during graph capture")
+            grow = max(count, int((flat.numel() if flat is not None else 0) * 1.5), 1)
+            flat = torch.empty(grow, dtype=dtype, device=self.device)
+            self._flat[key] = flat
+        return flat[:count].view(*shape)
+
+    def bytes(self) -> int:
+        return sum(t.numel() * t.element_size() for t in self._flat.values())
+
+
+class StepContext:
+    def __init__(self, *, device, dtype, page_size: int, workspace: Workspace, n: int, num_seqs: int,
+                 token_ids, positions, tok_seq, slots: List[torch.Tensor], tables: List[torch.Tensor],
+                 q_start, q_len, pos0, state_slots, want, host: dict, attention_impl: str = "auto"):
+        self.device, self.dtype, self.page_size, self.workspace = device, dtype, page_size, workspace
+        self.n, self.num_seqs = n, num_seqs
+        self.token_ids, self.positions, self.tok_seq = token_ids, positions, tok_seq
+        self.slots, self.tables = slots, tables          # one entry per page group
+        self.q_start, self.q_len, self.pos0, self.state_slots = q_start, q_len, pos0, state_slots
+        self.want = want
+        #: the same metadata as Python lists, for kernel selection and for parts written in Python
+        self.host = host
+        self.attention_impl = attention_impl
+        self.memo: dict = {}
+
+    def buffer(self, name: str, shape, dtype) -> torch.Tensor:
+        return self.workspace.buffer(name, shape, dtype)
+
+    # -------------------------------------------------------------------------------
+    def attention(self, q: torch.Tensor, out: torch.Tensor, cache, n_heads: int, scale: float, window: int) -> None:
+        """Paged attention of every row of the step over its request's cache.
+
+        float32 always takes the plain kernel.  bfloat16 takes the tuned kernels where they apply:
+        requests with one row go to the split-context decode kernel, longer portions to the
+        matrix-core prefill kernel; ``attention_impl='plain'`` forces the plain kernel."""
+        tables = self.tables[cache.group]
+        impl = self.attention_impl
+        if self.dtype == torch.float32 or impl == "plain" or not ops.tuned_attention_supports(cache.k_pages, n_heads, window):
+            ops.attention_plain(q, out, self.positions, self.tok_seq, tables, cache.k_pages, cache.v_pages,
+                                n_heads, scale, window)
+            return
+        h = self.host
+        if h["n_decode"] > 0:
+            ops.attention_decode(q, out, self, cache, n_heads, scale, window)
+        if h["n_decode"] < self.num_seqs:
+            ops.attention_prefill(q, out, self, cache, n_heads, scale, window)

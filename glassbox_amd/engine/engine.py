@@ -1,0 +1,254 @@
+"""The engine: a model, its cache (host bookkeeping and device pages) and the step function.
+
+``Engine.step`` is the one place where tokens become logits.  Generation, the scheduler, the
+benchmark and trace replay all go through it, as everything in the reference goes through
+``Model::forward`` (crates/glassbox-core/src/model.rs:207-362, docs/ARCHITECTURE.md:17).
+"""
+from __future__ import annotations
+
+import os
+from typing import Dict, Hashable, List, Optional, Sequence, Tuple
+
+import torch
+
+from .. import ops
+from ..cache.manager import FULL, CacheManager, GroupSpec, OutOfPages
+from ..parts.base import LayerCache
+from ..weights.loader import compute_dtype, load_model
+from .context import StepContext, Workspace
+
+Entry = Tuple[Hashable, Sequence[int], Sequence[int]]  # (request, its next tokens, wanted places among them)
+
+
+class EngineError(RuntimeError):
+    pass
+
+
+class Engine:
+    """model: a folder (config.json + model.safetensors) or a built and loaded model.
+
+    max_tokens: tokens the cache holds over all live requests (rounded up to whole pages).
+    max_seqs: most live requests (= state slots).  page_size: tokens per page (16 as in the
+    reference, crates/glassbox-core/src/kv.rs:11).
+    """
+
+    def __init__(self, model, dtype="bfloat16", max_tokens: int = 4096, max_seqs: int = 32, page_size: int = 16,
+                 prefix_caching: bool = False, device: str = "cuda:0", attention_impl: str = "auto"):
+        ops.require_gpu()
+        self.dtype = compute_dtype(dtype)
+        self.device = torch.device(device)
+        torch.cuda.set_device(self.device)
+        if isinstance(model, (str, os.PathLike)):
+            model = load_model(str(model), self.dtype, self.device)
+        self.model = model
+        self.page_size = int(page_size)
+        if self.page_size <= 0 or self.page_size % 16:
+            raise EngineError(f"page size {page_size} must be a positive multiple of 16")
+        self.max_seqs = int(max_seqs)
+        self.attention_impl = attention_impl
+        num_pages = max(1, -(-int(max_tokens) // self.page_size))
+
+        # page groups: cache layers whose mixers keep the same span of positions share page numbers
+        specs = model.cache_specs()
+        states = model.state_specs()
+        keys: List[Tuple[int, int]] = []
+        for spec in specs:
+            if spec is not None and spec.group_key not in keys:
+                keys.append(spec.group_key)
+        self.group_keys = keys
+        self.has_state = any(s is not None for s in states)
+        groups = [GroupSpec(kind, window, num_pages) for kind, window in keys]
+        share = prefix_caching and not self.has_state and all(kind == FULL for kind, _ in keys)
+        self.cache = CacheManager(self.page_size, groups, self.max_seqs, share)
+
+        self.layers: List[LayerCache] = []
+        for spec, state in zip(specs, states):
+            lc = LayerCache()
+            if spec is not None:
+                lc.group = keys.index(spec.group_key)
+                shape = (num_pages, spec.num_kv_heads, self.page_size, spec.head_dim)
+                lc.k_pages = torch.zeros(shape, dtype=self.dtype, device=self.device)
+                lc.v_pages = torch.zeros(shape, dtype=self.dtype, device=self.device)
+            if state is not None:
+                lc.state = torch.zeros((self.max_seqs,) + tuple(state.shape), dtype=state.dtype, device=self.device)
+            self.layers.append(lc)
+
+        self.workspace = Workspace(self.device)
+        self._ids: Dict[Hashable, int] = {}
+        self._next_id = 1
+        self._meta_dev: Optional[torch.Tensor] = None
+        self.steps = 0
+
+    # ---------------------------------------------------------------- requests
+    def has_request(self, request: Hashable) -> bool:
+        return request in self._ids
+
+    def add_request(self, request: Hashable, prompt: Sequence[int] = ()) -> int:
+        """Registers a request.  With prefix caching and a prompt, returns how many of its first
+        tokens are already in the cache and need not be run."""
+        if request in self._ids:
+            raise EngineError(f"request {request!r} is live already")
+        sid = self._next_id
+        self._next_id += 1
+        reused = self.cache.add_seq(sid, list(prompt))
+        self._ids[request] = sid
+        slot = self.cache.state_slot(sid)
+        for lc in self.layers:
+            if lc.state is not None:
+                lc.state[slot].zero_()   # a fresh request starts from empty state
+        return reused
+
+    def end_request(self, request: Hashable) -> None:
+        """Gives back everything the request holds."""
+        sid = self._ids.pop(request, None)
+        if sid is not None:
+            self.cache.remove_seq(sid)
+
+    def request_len(self, request: Hashable) -> int:
+        return self.cache.seq_len(self._ids[request])
+
+    def fork_request(self, parent: Hashable, child: Hashable) -> None:
+        if child in self._ids:
+            raise EngineError(f"request {child!r} is live already")
+        sid = self._next_id
+        self._next_id += 1
+        self.cache.fork(self._ids[parent], sid)
+        self._ids[child] = sid
+        self._apply_copies()
+
+    def free_tokens(self) -> int:
+        return self.cache.min_free_pages() * self.page_size
+
+    # -------------------------------------------------------------------- the step
+    def reserve(self, entries: Sequence[Entry]) -> None:
+        """Makes room for every entry's tokens; raises OutOfPages when the pool is too small
+        (entries reserved before the failing one keep their pages; nothing is written)."""
+        for request, tokens, _ in entries:
+            if request not in self._ids:
+                self.add_request(request)
+            self.cache.reserve(self._ids[request], len(tokens))
+        self._apply_copies()
+
+    def _apply_copies(self) -> None:
+        copies = self.cache.take_copies()
+        if not copies:
+            return
+        by_group: Dict[int, List[Tuple[int, int]]] = {}
+        for g, src, dst in copies:
+            by_group.setdefault(g, []).append((src, dst))
+        for g, pairs in by_group.items():
+            src = torch.tensor([p[0] for p in pairs], dtype=torch.int32, device=self.device)
+            dst = torch.tensor([p[1] for p in pairs], dtype=torch.int32, device=self.device)
+            for lc in self.layers:
+                if g == -1:
+                    if lc.state is not None:
+                        ops.copy_rows(lc.state, src, dst)
+                elif lc.k_pages is not None and lc.group == g:
+                    ops.copy_rows(lc.k_pages, src, dst)   # copy-on-write in every layer (kv.rs:189-196)
+                    ops.copy_rows(lc.v_pages, src, dst)
+
+    def step(self, entries: Sequence[Entry], commit: bool = True, reserved: bool = False) -> torch.Tensor:
+        """Runs exactly the given tokens, as one batch, from the cache that earlier steps left.
+
+        Returns float32 logits [wanted, vocab] in the order of the entries and of their wanted
+        places.  The tensor is a view of the engine's workspace: use it before the next step."""
+        entries = [(r, list(t), list(w)) for r, t, w in entries]
+        if not entries:
+            return torch.empty((0, self.model.vocab_size), dtype=torch.float32, device=self.device)
+        seen = set()
+        vocab = self.model.vocab_size
+        for request, tokens, want in entries:
+            if request in seen:
+                raise EngineError(f"request {request!r} appears twice in one step")
+            seen.add(request)
+            if not tokens:
+                raise EngineError(f"request {request!r} brings no tokens")
+            if min(tokens) < 0 or max(tokens) >= vocab:
+                raise EngineError(f"request {request!r}: token ids must lie in 0..{vocab - 1}")
+            if any(w < 0 or w >= len(tokens) for w in want):
+                raise EngineError(f"request {request!r}: wanted places must lie among its {len(tokens)} tokens")
+        if not reserved:
+            self.reserve(entries)
+        ctx = self._build_context(entries)
+        logits = self.model.forward(ctx, self.layers)
+        if commit:
+            for request, tokens, _ in entries:
+                self.cache.commit(self._ids[request], tokens)
+        self.steps += 1
+        return logits
+
+    # ---------------------------------------------------------------- metadata
+    def _build_context(self, entries) -> StepContext:
+        P = self.page_size
+        # single-token requests first: the tuned attention kernels take the two kinds in two launches
+        order = sorted(range(len(entries)), key=lambda i: len(entries[i][1]) > 1)
+        S = len(entries)
+        G = len(self.group_keys)
+        token_ids: List[int] = []
+        positions: List[int] = []
+        tok_seq: List[int] = []
+        q_start, q_len, pos0, state_slots = [], [], [], []
+        tables_host: List[List[List[int]]] = [[] for _ in range(G)]
+        slots_host: List[List[int]] = [[] for _ in range(G)]
+        want_flat: List[Tuple[int, int, int]] = []   # (entry index, place, flat row)
+        for s, ei in enumerate(order):
+            request, tokens, want = entries[ei]
+            sid = self._ids[request]
+            start = self.cache.seq_len(sid)
+            q_start.append(len(token_ids))
+            q_len.append(len(tokens))
+            pos0.append(start)
+            state_slots.append(self.cache.state_slot(sid))
+            for g in range(G):
+                table = self.cache.table(sid, g)
+                tables_host[g].append(table)
+                for j in range(len(tokens)):
+                    p = start + j
+                    slots_host[g].append(table[p // P] * P + p % P)
+            for k, w in enumerate(want):
+                want_flat.append((ei, k, len(token_ids) + w))
+            token_ids.extend(tokens)
+            positions.extend(range(start, start + len(tokens)))
+            tok_seq.extend([s] * len(tokens))
+        n = len(token_ids)
+        # logits come out in the order of the wanted rows: make that the order of the entries
+        want_flat.sort(key=lambda w: (w[0], w[1]))
+        want_rows = [w[2] for w in want_flat]
+        maxp = [max(1, max(len(t) for t in tables_host[g])) for g in range(G)]
+
+        pieces: List[List[int]] = [token_ids, positions, tok_seq, q_start, q_len, pos0, state_slots, want_rows]
+        for g in range(G):
+            pieces.append(slots_host[g])
+            flat: List[int] = []
+            for t in tables_host[g]:
+                flat.extend(t)
+                flat.extend([-1] * (maxp[g] - len(t)))
+            pieces.append(flat)
+        total = sum(len(p) for p in pieces)
+        if self._meta_dev is None or self._meta_dev.numel() < total:
+            self._meta_dev = torch.empty(max(total * 2, 4096), dtype=torch.int32, device=self.device)
+        flat_all: List[int] = []
+        for p in pieces:
+            flat_all.extend(p)
+        # a fresh pinned buffer per step: the host allocator hands it out again only after the copy ran
+        staged = torch.empty(total, dtype=torch.int32, pin_memory=True)
+        staged.copy_(torch.tensor(flat_all, dtype=torch.int32))
+        self._meta_dev[:total].copy_(staged, non_blocking=True)
+        views: List[torch.Tensor] = []
+        off = 0
+        for p in pieces:
+            views.append(self._meta_dev[off:off + len(p)])
+            off += len(p)
+        d_tok, d_pos, d_seq, d_qs, d_ql, d_p0, d_ss, d_want = views[:8]
+        slots = [views[8 + 2 * g] for g in range(G)]
+        tables = [views[9 + 2 * g].view(S, maxp[g]) for g in range(G)]
+        n_decode = sum(1 for l in q_len if l == 1)
+        host = {"q_start": q_start, "q_len": q_len, "pos0": pos0, "state_slots": state_slots,
+                "positions": positions, "tok_seq": tok_seq, "token_ids": token_ids, "tables": tables_host,
+                "n_decode": n_decode, "max_q_len": max(q_len),
+                "max_context": max(p + l for p, l in zip(pos0, q_len)), "want_rows": want_rows}
+        ctx = StepContext(device=self.device, dtype=self.dtype, page_size=P, workspace=self.workspace, n=n,
+                          num_seqs=S, token_ids=d_tok, positions=d_pos, tok_seq=d_seq, slots=slots, tables=tables,
+                          q_start=d_qs, q_len=d_ql, pos0=d_p0, state_slots=d_ss, want=d_want, host=host,
+                          attention_impl=self.attention_impl)
+        return ctx

@@ -1,0 +1,270 @@
+"""Python bindings of the device kernels (csrc/hip/*.hip), through ctypes.
+
+Each function checks devices, dtypes, contiguity and shapes, then passes raw
+pointers and the current HIP stream to the kernel's C entry point.  There is no
+CPU path and no library fallback: a missing GPU or a library that cannot be
+built raises.  Tensors are torch tensors only because torch is the allocator
+and stream owner; no torch operator computes anything here.
+"""
+from __future__ import annotations
+
+import ctypes as C
+from typing import Optional
+
+import torch
+
+from . import build
+
+F32, BF16 = 0, 1
+_vp, _i, _f = C.c_void_p, C.c_int, C.c_float
+
+
+class KernelError(RuntimeError):
+    pass
+
+
+def require_gpu() -> None:
+    if not torch.cuda.is_available():
+        raise KernelError("no GPU is visible: glassbox_amd runs on a gfx950 GPU only and has no CPU path")
+
+
+def dtype_code(t: torch.Tensor) -> int:
+    if t.dtype == torch.float32:
+        return F32
+    if t.dtype == torch.bfloat16:
+        return BF16
+    raise KernelError(f"unsupported element type {t.dtype}")
+
+
+_SIGS = {
+    "elementwise": {
+        "gb_embed": [_vp, _i, _vp, _vp, _i, _i, _i, _vp],
+        "gb_rmsnorm": [_vp, _vp, _i, _vp, _vp, _i, _i, _i, _f, _vp],
+        "gb_rope_table": [_vp, _vp, _vp, _vp, _i, _i, _vp],
+        "gb_rope_store": [_vp, _i, _i, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _vp],
+        "gb_silu_mul": [_vp, _vp, _i, _i, _i, _vp],
+        "gb_copy_rows": [_vp, C.c_longlong, _vp, _vp, _i, _vp],
+    },
+    "gemm_f32": {
+        "gb_gemm_f32": [_vp, _i, _vp, _i, _vp, _i, _i, _i, _i, _i, _vp],
+    },
+    "gemm_bf16": {
+        "gb_gemm_bf16": [_vp, _i, _vp, _i, _vp, _i, _i, _i, _i, _i, _i, _vp],
+    },
+    "attention_plain": {
+        "gb_attention_plain": [_vp, _i, _vp, _i, _i, _vp, _vp, _vp, _i, _vp, _vp, _i, _i, _i, _i, _i, _f, _i, _vp],
+    },
+    "attention_bf16": {
+        "gb_attention_decode_bf16": [_vp, _i, _vp, _i, _vp, _vp, _vp, _i, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i,
+                                     _f, _i, _i, _vp],
+        "gb_attention_prefill_bf16": [_vp, _i, _vp, _i, _vp, _vp, _vp, _vp, _i, _vp, _vp, _i, _i, _i, _i, _i, _i, _f,
+                                      _i, _vp],
+    },
+    "sampling": {
+        "gb_argmax": [_vp, _vp, _i, _i, _vp],
+        "gb_penalize": [_vp, _i, _vp, _vp, _vp, _vp, _i, _vp],
+        "gb_sample": [_vp, _i, _i, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp],
+    },
+}
+_libs = {}
+
+
+def _lib(name: str):
+    lib = _libs.get(name)
+    if lib is None:
+        require_gpu()
+        lib = build.load(name)
+        for fn, args in _SIGS[name].items():
+            f = getattr(lib, fn)
+            f.argtypes = args
+            f.restype = C.c_int
+        lib.gb_last_error.restype = C.c_char_p
+        _libs[name] = lib
+    return lib
+
+
+def _check(lib, rc: int) -> None:
+    if rc != 0:
+        raise KernelError(lib.gb_last_error().decode())
+
+
+def _stream():
+    return torch.cuda.current_stream().cuda_stream
+
+
+def _dev(*tensors: Optional[torch.Tensor]) -> None:
+    for t in tensors:
+        if t is not None and not t.is_cuda:
+            raise KernelError("operands must be on the GPU")
+
+
+def _p(t: Optional[torch.Tensor]):
+    return None if t is None else t.data_ptr()
+
+
+def _rows(t: torch.Tensor, what: str) -> int:
+    """Row stride of a 2-d tensor whose rows are dense."""
+    if t.dim() != 2 or t.stride(1) != 1:
+        raise KernelError(f"{what} must be 2-d with dense rows, got shape {tuple(t.shape)} strides {t.stride()}")
+    return t.stride(0)
+
+
+def _i32(t: Optional[torch.Tensor], what: str, n: Optional[int] = None) -> None:
+    if t is None:
+        return
+    if t.dtype != torch.int32 or not t.is_contiguous():
+        raise KernelError(f"{what} must be a contiguous int32 tensor")
+    if n is not None and t.numel() < n:
+        raise KernelError(f"{what} holds {t.numel()} entries, {n} are needed")
+
+
+# ------------------------------------------------------------------ elementwise
+def embed(table: torch.Tensor, ids: torch.Tensor, out: torch.Tensor) -> None:
+    """out[i, :] = table[ids[i], :] as 32-bit floats."""
+    _dev(table, ids, out)
+    n, d = out.shape
+    _i32(ids, "ids", n)
+    if out.dtype != torch.float32 or not out.is_contiguous() or not table.is_contiguous() or table.shape[1] != d:
+        raise KernelError("embed: out must be contiguous float32 [n, d] and table [vocab, d]")
+    lib = _lib("elementwise")
+    _check(lib, lib.gb_embed(_p(table), dtype_code(table), _p(ids), _p(out), n, d, table.shape[0], _stream()))
+
+
+def rmsnorm(x: torch.Tensor, gamma: torch.Tensor, eps: float, out: torch.Tensor,
+            rows: Optional[torch.Tensor] = None) -> None:
+    """out[r] = gamma * (x[rows[r] or r] / sqrt(mean(x^2) + eps)); x is float32."""
+    _dev(x, gamma, out, rows)
+    m, d = out.shape
+    if x.dtype != torch.float32 or not x.is_contiguous() or x.shape[1] != d or not out.is_contiguous():
+        raise KernelError("rmsnorm: x must be contiguous float32 [n, d] and out contiguous [m, d]")
+    if gamma.numel() != d or not gamma.is_contiguous():
+        raise KernelError(f"rmsnorm: gamma has {gamma.numel()} entries, the rows have {d}")
+    if rows is None and x.shape[0] < m:
+        raise KernelError("rmsnorm: fewer input rows than output rows")
+    _i32(rows, "rows", m)
+    lib = _lib("elementwise")
+    _check(lib, lib.gb_rmsnorm(_p(x), _p(gamma), dtype_code(gamma), _p(rows), _p(out), dtype_code(out), m, d,
+                               float(eps), _stream()))
+
+
+def rope_table(positions: torch.Tensor, inv_freq: torch.Tensor, cos: torch.Tensor, sin: torch.Tensor) -> None:
+    _dev(positions, inv_freq, cos, sin)
+    n, half = cos.shape
+    _i32(positions, "positions", n)
+    for t in (inv_freq, cos, sin):
+        if t.dtype != torch.float32 or not t.is_contiguous():
+            raise KernelError("rope_table: tables must be contiguous float32")
+    if inv_freq.numel() != half or sin.shape != cos.shape:
+        raise KernelError("rope_table: table shapes do not match")
+    lib = _lib("elementwise")
+    _check(lib, lib.gb_rope_table(_p(positions), _p(inv_freq), _p(cos), _p(sin), n, half, _stream()))
+
+
+def rope_store(qkv: torch.Tensor, cos: Optional[torch.Tensor], sin: Optional[torch.Tensor],
+               slots: Optional[torch.Tensor], k_pages: Optional[torch.Tensor], v_pages: Optional[torch.Tensor],
+               n_heads: int, n_kv_heads: int, head_dim: int, rotate: bool = True) -> None:
+    """Rotate the query and key heads of each stacked row in place and write keys and values
+    to the pages at ``slots``.  ``slots`` None: nothing is stored."""
+    _dev(qkv, cos, sin, slots, k_pages, v_pages)
+    n = qkv.shape[0]
+    stride = _rows(qkv, "qkv")
+    page_size = 0
+    if slots is not None:
+        _i32(slots, "slots", n)
+        want = (n_kv_heads, head_dim)
+        for pg in (k_pages, v_pages):
+            if pg is None or pg.dim() != 4 or (pg.shape[1], pg.shape[3]) != want or not pg.is_contiguous() \
+                    or pg.dtype != qkv.dtype:
+                raise KernelError("rope_store: pages must be contiguous [pages, kv heads, page size, head size] "
+                                  "of the activations' type")
+        page_size = k_pages.shape[2]
+        if v_pages.shape != k_pages.shape:
+            raise KernelError("rope_store: key and value pages differ in shape")
+    if rotate:
+        if cos is None or sin is None or cos.shape != (n, head_dim // 2) and cos.shape[0] < n:
+            raise KernelError("rope_store: rotation needs cos/sin tables of [n, head_dim/2]")
+        if cos.shape[1] != head_dim // 2 or cos.dtype != torch.float32 or not cos.is_contiguous() \
+                or not sin.is_contiguous():
+            raise KernelError("rope_store: cos/sin must be contiguous float32 [n, head_dim/2]")
+    lib = _lib("elementwise")
+    _check(lib, lib.gb_rope_store(_p(qkv), dtype_code(qkv), stride, _p(cos), _p(sin), _p(slots), _p(k_pages),
+                                  _p(v_pages), n, n_heads, n_kv_heads, head_dim, page_size, 1 if rotate else 0,
+                                  _stream()))
+
+
+def silu_mul(gate_up: torch.Tensor, out: torch.Tensor) -> None:
+    _dev(gate_up, out)
+    n, inter = out.shape
+    if gate_up.shape != (n, 2 * inter) or not gate_up.is_contiguous() or not out.is_contiguous() \
+            or gate_up.dtype != out.dtype:
+        raise KernelError("silu_mul: gate_up must be contiguous [n, 2I] and out [n, I] of one type")
+    lib = _lib("elementwise")
+    _check(lib, lib.gb_silu_mul(_p(gate_up), _p(out), dtype_code(out), n, inter, _stream()))
+
+
+def copy_rows(base: torch.Tensor, src: torch.Tensor, dst: torch.Tensor) -> None:
+    """base[dst[i]] = base[src[i]] along the first dimension."""
+    _dev(base, src, dst)
+    if not base.is_contiguous():
+        raise KernelError("copy_rows: base must be contiguous")
+    count = src.numel()
+    _i32(src, "src", count)
+    _i32(dst, "dst", count)
+    row_bytes = base[0].numel() * base.element_size()
+    lib = _lib("elementwise")
+    _check(lib, lib.gb_copy_rows(_p(base), row_bytes, _p(src), _p(dst), count, _stream()))
+
+
+# ------------------------------------------------------------------------ products
+def gemm(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor, accumulate: bool = False) -> None:
+    """out (+)= a . w^T with w in the [out features, in features] layout.
+    float32 operands take the true 32-bit kernel; bfloat16 operands the matrix-core kernels,
+    with out in bfloat16 or float32 (float32 when accumulating into the residual)."""
+    _dev(a, w, out)
+    M, K = a.shape
+    N = w.shape[0]
+    if w.shape[1] != K or out.shape != (M, N):
+        raise KernelError(f"gemm: shapes do not match: a {tuple(a.shape)}, w {tuple(w.shape)}, out {tuple(out.shape)}")
+    lda, ldw, ldc = _rows(a, "a"), _rows(w, "w"), _rows(out, "out")
+    if a.dtype == torch.float32 and w.dtype == torch.float32:
+        if out.dtype != torch.float32:
+            raise KernelError("gemm: 32-bit operands need a 32-bit result")
+        lib = _lib("gemm_f32")
+        _check(lib, lib.gb_gemm_f32(_p(a), lda, _p(w), ldw, _p(out), ldc, M, N, K, 1 if accumulate else 0, _stream()))
+    elif a.dtype == torch.bfloat16 and w.dtype == torch.bfloat16:
+        if accumulate and out.dtype != torch.float32:
+            raise KernelError("gemm: accumulation is into a 32-bit result")
+        lib = _lib("gemm_bf16")
+        _check(lib, lib.gb_gemm_bf16(_p(a), lda, _p(w), ldw, _p(out), ldc, dtype_code(out), M, N, K,
+                                     1 if accumulate else 0, _stream()))
+    else:
+        raise KernelError(f"gemm: operand types {a.dtype} and {w.dtype} do not match a kernel")
+
+
+# ----------------------------------------------------------------------- attention
+def attention_plain(q: torch.Tensor, out: torch.Tensor, positions: torch.Tensor, tok_seq: torch.Tensor,
+                    tables: torch.Tensor, k_pages: torch.Tensor, v_pages: torch.Tensor, n_heads: int,
+                    scale: float, window: int = 0) -> None:
+    """Paged attention, one block per (token, head); q may be a view into the stacked qkv rows."""
+    _dev(q, out, positions, tok_seq, tables, k_pages, v_pages)
+    n = q.shape[0]
+    _, nkv, page_size, hd = k_pages.shape
+    if q.shape[1] != n_heads * hd or out.shape != (n, n_heads * hd):
+        raise KernelError("attention: q and out must be [n, heads * head size]")
+    if not (q.dtype == out.dtype == k_pages.dtype == v_pages.dtype):
+        raise KernelError("attention: q, out and pages must share one element type")
+    if not k_pages.is_contiguous() or not v_pages.is_contiguous() or k_pages.shape != v_pages.shape:
+        raise KernelError("attention: pages must be contiguous and alike")
+    _i32(positions, "positions", n)
+    _i32(tok_seq, "tok_seq", n)
+    if tables.dtype != torch.int32 or tables.dim() != 2 or tables.stride(1) != 1:
+        raise KernelError("attention: block tables must be int32 [requests, pages]")
+    lib = _lib("attention_plain")
+    _check(lib, lib.gb_attention_plain(_p(q), _rows(q, "q"), _p(out), _rows(out, "out"), dtype_code(q), _p(positions),
+                                       _p(tok_seq), _p(tables), tables.stride(0), _p(k_pages), _p(v_pages), n,
+                                       n_heads, nkv, hd, page_size, float(scale), int(window), _stream()))
+
+
+def tuned_attention_supports(k_pages: torch.Tensor, n_heads: int, window: int) -> bool:
+    """Whether the tuned bfloat16 attention kernels take this layer's sizes."""
+    return False

@@ -1,0 +1,71 @@
+"""Grouped-query attention over the paged cache: the mixer of a Llama layer.
+
+qkv = h . Wqkv^T (query rows, then key rows, then value rows stacked, as the
+reference stacks them: crates/glassbox-core/src/model.rs:59-61,260-265);
+positions are encoded and keys/values written to the pages
+(model.rs:266-276); every token attends to its own request's positions up to
+its own through the block table (model.rs:285-312); the output projection is
+added into the residual (model.rs:322-325).
+"""
+from __future__ import annotations
+
+import math
+from typing import Dict, Optional
+
+import torch
+
+from .. import ops
+from .base import FULL, WINDOW, CacheSpec, LayerCache, Mixer, PositionEncoding, TensorSpec
+
+
+class PagedAttention(Mixer):
+    def __init__(self, width: int, n_heads: int, n_kv_heads: int, head_dim: int, position: PositionEncoding,
+                 window: int = 0, shares_kv: bool = False, scale: Optional[float] = None):
+        if n_heads % n_kv_heads:
+            raise ValueError(f"{n_heads} query heads are not a multiple of {n_kv_heads} key heads")
+        self.width, self.n_heads, self.n_kv_heads, self.head_dim = width, n_heads, n_kv_heads, head_dim
+        self.position = position
+        self.window = int(window)
+        self.shares_kv = shares_kv          # reads another layer's pages; has no key/value projections
+        self.scale = float(scale) if scale is not None else 1.0 / math.sqrt(head_dim)  # model.rs:244
+        self.q_dim = n_heads * head_dim
+        self.kv_dim = n_kv_heads * head_dim
+        self.cache_spec = None if shares_kv else CacheSpec(n_kv_heads, head_dim,
+                                                           WINDOW if window > 0 else FULL, self.window)
+        self.wqkv: Optional[torch.Tensor] = None
+        self.wo: Optional[torch.Tensor] = None
+
+    def tensor_specs(self) -> Dict[str, TensorSpec]:
+        specs = {"q_proj.weight": TensorSpec((self.q_dim, self.width))}
+        if not self.shares_kv:
+            specs["k_proj.weight"] = TensorSpec((self.kv_dim, self.width))
+            specs["v_proj.weight"] = TensorSpec((self.kv_dim, self.width))
+        specs["o_proj.weight"] = TensorSpec((self.width, self.q_dim))
+        return specs
+
+    def children(self):
+        return {"": self.position} if self.position.tensor_specs() else {}
+
+    def load(self, tensors):
+        if self.shares_kv:
+            self.wqkv = tensors["q_proj.weight"].contiguous()
+        else:
+            # one product computes all three (model.rs:59-61)
+            self.wqkv = torch.cat([tensors["q_proj.weight"], tensors["k_proj.weight"], tensors["v_proj.weight"]], 0)
+        self.wo = tensors["o_proj.weight"].contiguous()
+
+    def forward(self, ctx, h, residual, cache: Optional[LayerCache]):
+        if cache is None or cache.k_pages is None:
+            raise ValueError("PagedAttention needs a layer cache with pages")
+        n = h.shape[0]
+        rows = self.q_dim + (0 if self.shares_kv else 2 * self.kv_dim)
+        qkv = ctx.buffer("qkv", (n, rows), ctx.dtype)
+        ops.gemm(h, self.wqkv, qkv)
+        write = cache.writable and not self.shares_kv
+        self.position.apply_and_store(
+            ctx, qkv, self.n_heads, 0 if self.shares_kv else self.n_kv_heads, self.head_dim,
+            ctx.slots[cache.group] if write else None, cache.k_pages if write else None,
+            cache.v_pages if write else None)
+        att = ctx.buffer("att", (n, self.q_dim), ctx.dtype)
+        ctx.attention(qkv[:, :self.q_dim], att, cache, self.n_heads, self.scale, self.window)
+        ops.gemm(att, self.wo, residual, accumulate=True)

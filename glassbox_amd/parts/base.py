@@ -1,0 +1,116 @@
+"""What every part of a model is: something with named tensors and a forward.
+
+A part takes its sizes and constants as constructor arguments and never asks
+which model it is in.  It declares the tensors it needs (``tensor_specs``), is
+handed them on the device (``load``) and works on the rows of a step
+(``forward``).  Parts may nest (``children``); tensor names are the path of
+child names joined by dots, which is how checkpoint names come about.
+
+Interfaces (all activations are [tokens, width] tensors on the device;
+``ctx`` is an ``engine.context.StepContext``):
+
+  Norm.forward(ctx, x_f32, rows=None) -> h          normalised rows in the compute type
+  PositionEncoding.apply_and_store(ctx, qkv, n_heads, n_kv_heads, head_dim, slots, k_pages, v_pages)
+                                                    encodes positions into the query/key heads of the
+                                                    stacked rows in place and writes keys/values to pages
+  Mixer.forward(ctx, h, residual, cache)            adds the mixed rows into ``residual`` (float32)
+      .cache_spec  -> CacheSpec | None              paged keys/values it needs
+      .state_spec  -> StateSpec | None              fixed-size per-request state it needs
+  FeedForward.forward(ctx, h, residual)             adds its output into ``residual`` (float32)
+  Block.forward(ctx, x, cache)                      one layer: arrangement of the four above
+"""
+from __future__ import annotations
+
+from dataclasses import dataclass
+from typing import Dict, Iterator, Optional, Tuple
+
+import torch
+
+FULL, WINDOW = 0, 1
+
+
+@dataclass(frozen=True)
+class TensorSpec:
+    """A tensor a part needs.  ``kind`` decides its type on the device:
+    'matrix' follows the compute type (bfloat16 or float32); 'vector' keeps 32-bit storage if the
+    file has it and is bfloat16 otherwise (float32 in the 32-bit path); 'f32' is always float32;
+    'int' becomes int32.  ``init`` is what the random-weights mode draws: 'normal', 'ones', 'zeros'."""
+    shape: Tuple[int, ...]
+    kind: str = "matrix"
+    init: str = "normal"
+
+
+@dataclass(frozen=True)
+class CacheSpec:
+    """Paged keys and values of one layer.  kind FULL keeps every position, WINDOW the last ``window``."""
+    num_kv_heads: int
+    head_dim: int
+    kind: int = FULL
+    window: int = 0
+
+    @property
+    def group_key(self) -> Tuple[int, int]:
+        return (self.kind, self.window if self.kind == WINDOW else 0)
+
+
+@dataclass(frozen=True)
+class StateSpec:
+    """Fixed-size state of one layer for each live request (one slot per request)."""
+    shape: Tuple[int, ...]
+    dtype: torch.dtype = torch.float32
+
+
+@dataclass
+class LayerCache:
+    """What the engine hands a mixer: its layer's pages, the index of their page group, its state."""
+    k_pages: Optional[torch.Tensor] = None   # [pages, kv heads, page size, head size]
+    v_pages: Optional[torch.Tensor] = None
+    group: int = 0
+    state: Optional[torch.Tensor] = None     # [slots, *state shape]
+    writable: bool = True                    # False: the layer reads another layer's cache
+
+
+class Part:
+    def tensor_specs(self) -> Dict[str, TensorSpec]:
+        return {}
+
+    def children(self) -> Dict[str, "Part"]:
+        return {}
+
+    def load(self, tensors: Dict[str, torch.Tensor]) -> None:
+        """Receives the tensors of ``tensor_specs`` (own names only), already on the device."""
+
+    def named_specs(self, prefix: str = "") -> Iterator[Tuple[str, TensorSpec]]:
+        for name, spec in self.tensor_specs().items():
+            yield prefix + name, spec
+        for cname, child in self.children().items():
+            yield from child.named_specs(f"{prefix}{cname}." if cname else prefix)
+
+    def load_tree(self, tensors: Dict[str, torch.Tensor], prefix: str = "") -> None:
+        own = {name: tensors[prefix + name] for name in self.tensor_specs()}
+        self.load(own)
+        for cname, child in self.children().items():
+            child.load_tree(tensors, f"{prefix}{cname}." if cname else prefix)
+
+
+class Norm(Part):
+    def forward(self, ctx, x: torch.Tensor, rows: Optional[torch.Tensor] = None, out_name: str = "h") -> torch.Tensor:
+        raise NotImplementedError
+
+
+class PositionEncoding(Part):
+    def apply_and_store(self, ctx, qkv, n_heads, n_kv_heads, head_dim, slots, k_pages, v_pages) -> None:
+        raise NotImplementedError
+
+
+class Mixer(Part):
+    cache_spec: Optional[CacheSpec] = None
+    state_spec: Optional[StateSpec] = None
+
+    def forward(self, ctx, h: torch.Tensor, residual: torch.Tensor, cache: Optional[LayerCache]) -> None:
+        raise NotImplementedError
+
+
+class FeedForward(Part):
+    def forward(self, ctx, h: torch.Tensor, residual: torch.Tensor) -> None:
+        raise NotImplementedError

@@ -1,0 +1,110 @@
+"""A decoder assembled from parts, with the order of its layers as data.
+
+``blocks`` are the layers that own weights.  ``schedule`` is the list of calls
+that a step makes, in order: each names a block and the cache layer it writes
+(``cache``) or, instead, a cache layer that it only reads (``reads``).  A block
+may be named twice (shared weights, each call with a cache layer of its own),
+and a call may read the cache that an earlier call wrote.  For Llama the
+schedule is simply block i with cache layer i
+(crates/glassbox-core/src/model.rs:251).
+"""
+from __future__ import annotations
+
+from dataclasses import dataclass
+from typing import Dict, List, Optional, Sequence
+
+import torch
+
+from .base import CacheSpec, LayerCache, Norm, Part, StateSpec
+from .embedding import Embedding, LMHead
+
+
+@dataclass(frozen=True)
+class LayerCall:
+    block: int
+    cache: Optional[int] = None   # cache layer this call writes and reads
+    reads: Optional[int] = None   # or: cache layer of another call that this one only reads
+
+
+class DecoderModel(Part):
+    def __init__(self, config, embedding: Embedding, blocks: Sequence[Part], schedule: Sequence[LayerCall],
+                 final_norm: Norm, head: LMHead, names=("model.embed_tokens", "model.layers.{}", "model.norm", "lm_head"),
+                 ignorable: Sequence[str] = ()):
+        self.config = config
+        self.embedding, self.blocks, self.schedule = embedding, list(blocks), list(schedule)
+        self.final_norm, self.head = final_norm, head
+        self.names = tuple(names)
+        self.ignorable = tuple(ignorable)   # tensors a checkpoint may hold that the model does not use
+        self.vocab_size = embedding.vocab
+        self.width = embedding.width
+        self._check_schedule()
+
+    # structure ------------------------------------------------------------------
+    def children(self) -> Dict[str, Part]:
+        out: Dict[str, Part] = {self.names[0]: self.embedding}
+        for i, b in enumerate(self.blocks):
+            out[self.names[1].format(i)] = b
+        out[self.names[2]] = self.final_norm
+        out[self.names[3]] = self.head
+        return out
+
+    def _check_schedule(self) -> None:
+        owners: Dict[int, int] = {}
+        for pos, call in enumerate(self.schedule):
+            if not 0 <= call.block < len(self.blocks):
+                raise ValueError(f"schedule entry {pos} names block {call.block}, there are {len(self.blocks)}")
+            if call.cache is not None and call.reads is not None:
+                raise ValueError(f"schedule entry {pos} both owns and borrows a cache layer")
+            if call.cache is not None:
+                if call.cache in owners:
+                    raise ValueError(f"cache layer {call.cache} is written by schedule entries {owners[call.cache]} and {pos}")
+                owners[call.cache] = pos
+        for pos, call in enumerate(self.schedule):
+            if call.reads is not None and (call.reads not in owners or owners[call.reads] >= pos):
+                raise ValueError(f"schedule entry {pos} reads cache layer {call.reads}, which no earlier entry writes")
+        self.num_cache_layers = (max(owners) + 1) if owners else 0
+        if sorted(owners) != list(range(self.num_cache_layers)):
+            raise ValueError("cache layers must be numbered 0..n-1 without gaps")
+        self._owners = owners
+
+    def cache_specs(self) -> List[Optional[CacheSpec]]:
+        """What each cache layer holds, from the mixer of the block that writes it."""
+        return [getattr(self.blocks[self.schedule[self._owners[c]].block].mixer, "cache_spec", None)
+                for c in range(self.num_cache_layers)]
+
+    def state_specs(self) -> List[Optional[StateSpec]]:
+        return [getattr(self.blocks[self.schedule[self._owners[c]].block].mixer, "state_spec", None)
+                for c in range(self.num_cache_layers)]
+
+    # the step ---------------------------------------------------------------------
+    def forward(self, ctx, caches: Sequence[LayerCache]) -> torch.Tensor:
+        """Runs the tokens of ``ctx`` through every scheduled layer; logits [wanted, vocab] float32."""
+        x = ctx.buffer("x", (ctx.n, self.width), torch.float32)
+        self.embedding.forward(ctx, x)
+        for call in self.schedule:
+            if call.cache is not None:
+                cache = caches[call.cache]
+            elif call.reads is not None:
+                src = caches[call.reads]
+                cache = LayerCache(src.k_pages, src.v_pages, src.group, src.state, writable=False)
+            else:
+                cache = None
+            self.blocks[call.block].forward(ctx, x, cache)
+        if ctx.want.numel() == 0:
+            return ctx.buffer("logits", (0, self.vocab_size), torch.float32)
+        rows = self.final_norm.forward(ctx, x, rows=ctx.want, out_name="h_out")
+        return self.head.forward(ctx, rows)
+
+    def weight_bytes(self) -> int:
+        """Bytes of the matrices a decode step reads once (model.rs:175-184: norm vectors excluded)."""
+        seen, total = set(), 0
+        for call in self.schedule:
+            blk = self.blocks[call.block]
+            for part in (getattr(blk, "mixer", None), getattr(blk, "ffn", None)):
+                for t in vars(part).values() if part is not None else ():
+                    if isinstance(t, torch.Tensor) and t.dim() == 2 and t.data_ptr() not in seen:
+                        seen.add(t.data_ptr())
+                        total += t.numel() * t.element_size()
+        head = self.head.matrix()
+        total += head.numel() * head.element_size()
+        return total

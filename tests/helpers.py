@@ -1,0 +1,150 @@
+"""Shared by the tests: the tiny configurations, model folders, the plain oracle with a cache of
+its results, and replay schedules (ways of cutting requests into steps)."""
+from __future__ import annotations
+
+import functools
+import os
+import random
+from typing import Dict, List, Sequence, Tuple
+
+import numpy as np
+import torch
+
+from plain import llama as plain_llama
+
+# Two tiny configurations that differ in every size and option.
+TINY_A = dict(architectures=["LlamaForCausalLM"], hidden_size=64, intermediate_size=176, num_hidden_layers=2,
+              num_attention_heads=4, num_key_value_heads=2, vocab_size=256, rope_theta=10000.0,
+              rms_norm_eps=1e-5, tie_word_embeddings=True, max_position_embeddings=128)
+TINY_B = dict(architectures=["LlamaForCausalLM"], hidden_size=96, intermediate_size=256, num_hidden_layers=3,
+              num_attention_heads=3, num_key_value_heads=1, head_dim=32, vocab_size=384, rope_theta=500000.0,
+              rms_norm_eps=1e-6, tie_word_embeddings=False, max_position_embeddings=256)
+# sizes that are no power of two and a head size that hidden/heads does not give
+TINY_C = dict(architectures=["LlamaForCausalLM"], hidden_size=80, intermediate_size=144, num_hidden_layers=2,
+              num_attention_heads=6, num_key_value_heads=2, head_dim=48, vocab_size=331, rope_theta=130000.0,
+              rms_norm_eps=3e-5, tie_word_embeddings=True, max_position_embeddings=512)
+TINY = {"A": TINY_A, "B": TINY_B, "C": TINY_C}
+
+
+class ModelDirs:
+    def __init__(self, base: str):
+        self.base = base
+        self._made: Dict[Tuple, str] = {}
+
+    def get(self, name: str, seed: int = 0, norm_init: str = "uniform", dtype=torch.float32) -> str:
+        from glassbox_amd.config import config_from_dict
+        from glassbox_amd.weights import write_random_model
+        key = (name, seed, norm_init, str(dtype))
+        if key not in self._made:
+            folder = os.path.join(self.base, "_".join(str(k).replace(".", "_") for k in key))
+            write_random_model(config_from_dict(TINY[name]), folder, seed, norm_init=norm_init, dtype=dtype)
+            self._made[key] = folder
+        return self._made[key]
+
+
+@functools.lru_cache(maxsize=None)
+def _load(folder: str):
+    return plain_llama.load_folder(folder)
+
+
+@functools.lru_cache(maxsize=None)
+def plain_logits(folder: str, tokens: Tuple[int, ...]) -> np.ndarray:
+    """Logits at every position by the plain implementation in float64."""
+    cfg, w = _load(folder)
+    return plain_llama.forward(w, cfg, list(tokens), torch.float64).numpy()
+
+
+def random_tokens(vocab: int, n: int, seed: int) -> List[int]:
+    rng = random.Random(seed)
+    return [rng.randrange(vocab) for _ in range(n)]
+
+
+# ------------------------------------------------------------------ schedules
+Step = Dict  # {"entries": [(id, tokens, want)], "end": [ids]}
+
+
+def schedule_whole(requests: Dict[str, List[int]]) -> List[Step]:
+    return [{"entries": [(rid, toks, list(range(len(toks))))], "end": [rid]} for rid, toks in requests.items()]
+
+
+def schedule_tail(requests: Dict[str, List[int]], tail: int = 32) -> List[Step]:
+    steps = []
+    for rid, toks in requests.items():
+        head = max(0, len(toks) - tail)
+        if head:
+            steps.append({"entries": [(rid, toks[:head], list(range(head)))], "end": []})
+        for i in range(head, len(toks)):
+            steps.append({"entries": [(rid, [toks[i]], [0])], "end": [rid] if i == len(toks) - 1 else []})
+    return steps
+
+
+def schedule_chunks(requests: Dict[str, List[int]], sizes=(7, 2, 16, 3, 33, 5, 2, 64, 17)) -> List[Step]:
+    steps = []
+    for rid, toks in requests.items():
+        at, k = 0, 0
+        while at < len(toks):
+            n = min(sizes[k % len(sizes)], len(toks) - at)
+            k += 1
+            steps.append({"entries": [(rid, toks[at:at + n], list(range(n)))],
+                          "end": [rid] if at + n == len(toks) else []})
+            at += n
+    return steps
+
+
+def schedule_mixed(requests: Dict[str, List[int]], seed: int = 0, live: int = 4, tail: int = 32):
+    """Up to ``live`` requests at once: portions of some beside decoded tokens of others; a finished
+    request gives its pages back and the next one is admitted into them.  Returns (steps, the most
+    tokens live requests hold at any time, each rounded up to a multiple of 64)."""
+    rng = random.Random(seed)
+    waiting = list(requests.items())
+    running: List[List] = []   # [rid, tokens, done]
+    steps: List[Step] = []
+    peak = 0
+    while waiting or running:
+        while waiting and len(running) < live:
+            rid, toks = waiting.pop(0)
+            running.append([rid, toks, 0])
+        entries, end = [], []
+        for r in running:
+            rid, toks, done = r
+            if rng.random() < 0.2 and len(running) > 1:
+                continue   # left out of this step, goes on later
+            left = len(toks) - done
+            if left <= tail:
+                n = 1
+            else:
+                n = min(left - tail, rng.choice([2, 3, 5, 8, 13, 16, 21, 40]))
+                n = max(2, n) if left - tail >= 2 else 1
+            entries.append((rid, toks[done:done + n], list(range(n))))
+            r[2] = done + n
+            if r[2] == len(toks):
+                end.append(rid)
+        if not entries:
+            continue
+        peak = max(peak, sum(-(-r[2] // 64) * 64 for r in running))
+        steps.append({"entries": entries, "end": end})
+        running = [r for r in running if r[0] not in end]
+    return steps, peak
+
+
+def replay(engine, steps: Sequence[Step]) -> Dict[str, np.ndarray]:
+    """Drives engine.step through ``steps``; returns each request's logits at every wanted position,
+    in position order (the schedules above want every position exactly once)."""
+    got: Dict[str, List[np.ndarray]] = {}
+    for st in steps:
+        logits = engine.step(st["entries"]).float().cpu().numpy()
+        row = 0
+        for rid, toks, want in st["entries"]:
+            got.setdefault(rid, []).append(logits[row:row + len(want)].copy())
+            row += len(want)
+        assert row == logits.shape[0]
+        for rid in st["end"]:
+            engine.end_request(rid)
+    return {rid: np.concatenate(parts, 0) for rid, parts in got.items()}
+
+
+def first_bad(got: np.ndarray, want: np.ndarray, tol: float):
+    """Position of the first row beyond tolerance, or None."""
+    err = np.abs(got - want).max(axis=1)
+    bad = np.nonzero(err > tol)[0]
+    return (int(bad[0]), float(err[bad[0]])) if bad.size else None

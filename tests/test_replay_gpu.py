@@ -1,0 +1,139 @@
+"""The engine against the plain implementation under every way of cutting requests into steps:
+whole, last 32 tokens one by one, portions of changing size, and mixed batches with so few pages
+that they are used again; in 32-bit and in bfloat16."""
+import json
+import os
+import subprocess
+import sys
+
+import numpy as np
+import pytest
+import torch
+
+import helpers
+
+pytestmark = pytest.mark.gpu
+
+# 32-bit: the stated target of the engine.  bfloat16: operands carry 8 bits, about 4e-3 relative
+# per rounding; logits here are of order 0.3, a few dozen roundings deep.
+TOL = {"float32": 1e-4, "bfloat16": 2.5e-2}
+
+REQUESTS = {
+    "A": {"a0": 5, "a1": 17, "a2": 49, "a3": 128, "a4": 70, "a5": 33},
+    "B": {"b0": 1, "b1": 33, "b2": 64, "b3": 94, "b4": 200, "b5": 40},
+    "C": {"c0": 3, "c1": 47, "c2": 130, "c3": 65, "c4": 257},
+}
+# more requests than are live at once, so that finished requests' pages are handed out again
+MORE = {
+    "A": {"a6": 100, "a7": 60, "a8": 128, "a9": 20, "a10": 81},
+    "B": {"b6": 150, "b7": 17, "b8": 256, "b9": 77},
+    "C": {"c5": 90, "c6": 33, "c7": 200, "c8": 16, "c9": 129},
+}
+
+
+def make_requests_det(name, more=False):
+    vocab = helpers.TINY[name]["vocab_size"]
+    lengths = dict(REQUESTS[name], **(MORE[name] if more else {}))
+    return {rid: helpers.random_tokens(vocab, n, seed=100 * ord(name) + i)
+            for i, (rid, n) in enumerate(lengths.items())}
+
+
+def check(folder, requests, got, dtype, what):
+    for rid, toks in requests.items():
+        want = helpers.plain_logits(folder, tuple(toks))
+        assert got[rid].shape == want.shape, f"{what} {rid}: shape {got[rid].shape} vs {want.shape}"
+        bad = helpers.first_bad(got[rid], want, TOL[dtype])
+        assert bad is None, (f"{what}, request {rid} ({len(toks)} tokens), {dtype}: first wrong position {bad[0]} "
+                             f"(page offset {bad[0] % 16}), max abs error {bad[1]:.3e}")
+
+
+@pytest.fixture(scope="module")
+def engines(model_dirs):
+    from glassbox_amd.engine import Engine
+    made = {}
+
+    def get(name, dtype, max_tokens=1024):
+        key = (name, dtype, max_tokens)
+        if key not in made:
+            made[key] = Engine(model_dirs.get(name), dtype=dtype, max_tokens=max_tokens, max_seqs=8)
+        return made[key]
+    return get
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("name", ["A", "B", "C"])
+@pytest.mark.parametrize("mode", ["whole", "tail32", "chunks"])
+def test_single_request_splits(engines, model_dirs, name, dtype, mode):
+    folder = model_dirs.get(name)
+    requests = make_requests_det(name)
+    steps = {"whole": helpers.schedule_whole, "tail32": helpers.schedule_tail,
+             "chunks": helpers.schedule_chunks}[mode](requests)
+    eng = engines(name, dtype)
+    got = helpers.replay(eng, steps)
+    check(folder, requests, got, dtype, mode)
+    eng.cache.check_invariants()
+    assert eng.cache.used_pages() == 0
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("name", ["A", "B", "C"])
+def test_mixed_batches_with_page_reuse(model_dirs, name, dtype):
+    from glassbox_amd.engine import Engine
+    folder = model_dirs.get(name)
+    requests = make_requests_det(name, more=True)
+    for seed in (0, 1):
+        steps, peak = helpers.schedule_mixed(requests, seed=seed)
+        eng = Engine(folder, dtype=dtype, max_tokens=peak, max_seqs=4)   # exactly as many pages as are held at the peak
+        got = helpers.replay(eng, steps)
+        check(folder, requests, got, dtype, f"mixed(seed {seed}, pool {peak})")
+        eng.cache.check_invariants()
+        assert eng.cache.used_pages() == 0
+        assert sum(len(t) for t in requests.values()) > peak, "the schedule did not reuse pages"
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_long_decoding(engines, model_dirs, dtype):
+    folder = model_dirs.get("C")
+    toks = helpers.random_tokens(helpers.TINY["C"]["vocab_size"], 300, seed=9)
+    steps = helpers.schedule_tail({"long": toks}, tail=290)
+    got = helpers.replay(engines("C", dtype), steps)
+    check(folder, {"long": toks}, got, dtype, "long decoding")
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("name", ["A", "B"])
+def test_first_tokens(engines, model_dirs, name, dtype):
+    folder = model_dirs.get(name)
+    toks = helpers.random_tokens(helpers.TINY[name]["vocab_size"], 4, seed=3)
+    got = helpers.replay(engines(name, dtype), helpers.schedule_tail({"first": toks}, tail=4))
+    check(folder, {"first": toks}, got, dtype, "first tokens")
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_trace_run_program(model_dirs, tmp_path, dtype):
+    """The program itself, as a child process: mixed steps over a small pool, files and 'done' lines."""
+    folder = model_dirs.get("B")
+    requests = make_requests_det("B")
+    steps, peak = helpers.schedule_mixed(requests, seed=5)
+    out = tmp_path / "out"
+    lines = []
+    for i, st in enumerate(steps):
+        lines.append(json.dumps({"step": i, "end": st["end"],
+                                 "entries": [{"id": r, "tokens": t, "want": w} for r, t, w in st["entries"]]}))
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    proc = subprocess.run([sys.executable, os.path.join(root, "bin", "trace_run"), "--model", folder, "--dtype", dtype,
+                           "--out", str(out), "--max-tokens", str(peak)], input="\n".join(lines) + "\n",
+                          capture_output=True, text=True, timeout=600)
+    assert proc.returncode == 0, proc.stderr[-2000:]
+    assert proc.stdout.split() == [w for i in range(len(steps)) for w in ("done", str(i))]
+    vocab = helpers.TINY["B"]["vocab_size"]
+    got = {}
+    for i, st in enumerate(steps):
+        data = np.fromfile(out / f"{i}.f32", dtype="<f4").reshape(-1, vocab)
+        row = 0
+        for r, t, w in st["entries"]:
+            got.setdefault(r, []).append(data[row:row + len(w)])
+            row += len(w)
+        assert row == data.shape[0]
+    got = {r: np.concatenate(p, 0) for r, p in got.items()}
+    check(folder, requests, got, dtype, "trace_run")
