@@ -1,0 +1,250 @@
+"""Each kernel alone against a plain float64 formula, at sizes other than the engine's."""
+import math
+
+import numpy as np
+import pytest
+import torch
+
+pytestmark = pytest.mark.gpu
+
+DEV = "cuda:0"
+
+
+def rnd(*shape, seed=0, scale=1.0, dtype=torch.float32):
+    g = torch.Generator().manual_seed(seed)
+    return (torch.randn(*shape, generator=g, dtype=torch.float64) * scale).to(dtype)
+
+
+def to_dev(t, dtype=None):
+    return t.to(device=DEV, dtype=dtype or t.dtype).contiguous()
+
+
+# ----------------------------------------------------------------------- products
+# (rows of W, k, tokens): the awkward shapes of the reference's own matmul test
+# (crates/glassbox-core/src/kernels.rs:697) and larger ones that cross tile edges
+GEMM_SHAPES_F32 = [(1, 32, 1), (8, 64, 2), (17, 64, 3), (33, 96, 9), (50, 160, 17), (331, 100, 70), (130, 257, 129)]
+GEMM_SHAPES_BF16 = [(1, 32, 1), (8, 64, 2), (17, 64, 3), (33, 96, 9), (50, 160, 17), (331, 104, 64), (331, 104, 65),
+                    (130, 264, 129), (16, 2048, 8), (272, 72, 300), (49, 520, 33)]
+
+
+@pytest.mark.parametrize("N,K,M", GEMM_SHAPES_F32)
+@pytest.mark.parametrize("accumulate", [False, True])
+def test_gemm_f32(N, K, M, accumulate):
+    from glassbox_amd import ops
+    a, w, c0 = rnd(M, K, seed=1), rnd(N, K, seed=2), rnd(M, N, seed=3)
+    want = a.double() @ w.double().T + (c0.double() if accumulate else 0)
+    c = to_dev(c0.clone())
+    ops.gemm(to_dev(a), to_dev(w), c, accumulate=accumulate)
+    err = (c.cpu().double() - want).abs().max().item()
+    assert err <= 1e-4 * (1 + want.abs().max().item()), err   # kernels.rs:716 tolerance
+
+
+@pytest.mark.parametrize("N,K,M", GEMM_SHAPES_BF16)
+@pytest.mark.parametrize("out", ["bf16", "f32", "f32+"])
+def test_gemm_bf16(N, K, M, out):
+    from glassbox_amd import ops
+    a, w = rnd(M, K, seed=1).bfloat16(), rnd(N, K, seed=2).bfloat16()
+    c0 = rnd(M, N, seed=3)
+    want = a.double() @ w.double().T + (c0.double() if out == "f32+" else 0)
+    c = to_dev(c0.clone(), torch.bfloat16 if out == "bf16" else torch.float32)
+    ops.gemm(to_dev(a), to_dev(w), c, accumulate=(out == "f32+"))
+    got = c.cpu().double()
+    # products of bfloat16 numbers are exact in 32-bit; only the summation order and (for a
+    # bfloat16 result) the final rounding differ from the float64 sum
+    tol = 1e-4 * math.sqrt(K) + (2 ** -8) * want.abs().max().item() * (out == "bf16")
+    assert (got - want).abs().max().item() <= tol
+
+
+def test_gemm_bf16_one_hot_rows_and_columns():
+    """Every (row, column, k) lands where it should: W picks single columns of A."""
+    from glassbox_amd import ops
+    M, K, N = 150, 136, 200
+    a = rnd(M, K, seed=5).bfloat16()
+    w = torch.zeros(N, K)
+    for n in range(N):
+        w[n, (7 * n + 3) % K] = 1.0
+    c = torch.zeros(M, N, device=DEV)
+    ops.gemm(to_dev(a), to_dev(w.bfloat16()), c)
+    want = a.float()[:, [(7 * n + 3) % K for n in range(N)]]
+    assert torch.equal(c.cpu(), want)
+    c2 = torch.zeros(9, N, device=DEV)
+    ops.gemm(to_dev(a[:9]), to_dev(w.bfloat16()), c2)
+    assert torch.equal(c2.cpu(), want[:9])
+
+
+def test_gemm_refuses_bad_inner_size():
+    from glassbox_amd import ops
+    a, w = torch.zeros(4, 12, device=DEV, dtype=torch.bfloat16), torch.zeros(8, 12, device=DEV, dtype=torch.bfloat16)
+    with pytest.raises(ops.KernelError, match="multiple of 8"):
+        ops.gemm(a, w, torch.zeros(4, 8, device=DEV, dtype=torch.bfloat16))
+
+
+# -------------------------------------------------------------------- elementwise
+@pytest.mark.parametrize("n,d", [(1, 7), (3, 100), (5, 576), (2, 1537), (4, 2048)])
+@pytest.mark.parametrize("out_dtype", [torch.float32, torch.bfloat16])
+def test_rmsnorm(n, d, out_dtype):
+    from glassbox_amd import ops
+    x, g, eps = rnd(n, d, seed=1, scale=3.0), rnd(d, seed=2) + 1.0, 3e-5
+    want = g.double() * (x.double() * torch.rsqrt(x.double().pow(2).mean(-1, keepdim=True) + eps))
+    out = torch.empty(n, d, device=DEV, dtype=out_dtype)
+    ops.rmsnorm(to_dev(x), to_dev(g), eps, out)
+    tol = 1e-5 if out_dtype == torch.float32 else 2 ** -8
+    assert ((out.cpu().double() - want).abs() <= tol * (1 + want.abs())).all()
+    # picked rows
+    rows = torch.tensor([n - 1, 0], dtype=torch.int32, device=DEV)
+    out2 = torch.empty(2, d, device=DEV, dtype=out_dtype)
+    ops.rmsnorm(to_dev(x), to_dev(g), eps, out2, rows)
+    assert torch.equal(out2.cpu(), out.cpu()[[n - 1, 0]])
+
+
+def test_embed():
+    from glassbox_amd import ops
+    table = rnd(37, 50, seed=1)
+    ids = torch.tensor([5, 0, 36, 5], dtype=torch.int32, device=DEV)
+    for dt in (torch.float32, torch.bfloat16):
+        out = torch.empty(4, 50, device=DEV)
+        ops.embed(to_dev(table, dt), ids, out)
+        assert torch.equal(out.cpu(), table.to(dt).float()[[5, 0, 36, 5]])
+
+
+def test_silu_mul():
+    from glassbox_amd import ops
+    gu = rnd(6, 2 * 173, seed=4, scale=4.0)
+    g, u = gu[:, :173].double(), gu[:, 173:].double()
+    want = g / (1 + torch.exp(-g)) * u
+    out = torch.empty(6, 173, device=DEV)
+    ops.silu_mul(to_dev(gu), out)
+    assert (out.cpu().double() - want).abs().max().item() < 1e-5
+
+
+@pytest.mark.parametrize("hd,theta", [(16, 10000.0), (48, 500000.0), (128, 130000.0)])
+def test_rope_table_and_rotation(hd, theta):
+    """Against the plain implementation: pairing (i, i + hd/2), sign, 32-bit angle at long positions."""
+    from glassbox_amd import ops
+    from glassbox_amd.parts.rotary import Rotary
+    from plain import llama
+    pos = [0, 1, 17, 4095, 100003]
+    n, nh, nkv = len(pos), 3, 2
+    rot = Rotary(hd, theta)
+    cos = torch.empty(n, hd // 2, device=DEV)
+    sin = torch.empty_like(cos)
+    ops.rope_table(torch.tensor(pos, dtype=torch.int32, device=DEV), torch.from_numpy(rot.inv_host).to(DEV), cos, sin)
+    s_want, c_want = llama.rope_angles(pos, hd, theta)
+    assert np.abs(cos.cpu().numpy() - c_want).max() < 1e-7 and np.abs(sin.cpu().numpy() - s_want).max() < 1e-7
+    qkv = rnd(n, (nh + 2 * nkv) * hd, seed=3)
+    page = 16
+    k_pages = torch.zeros(4, nkv, page, hd, device=DEV)
+    v_pages = torch.zeros_like(k_pages)
+    slots = torch.tensor([3, 16 + 15, 32, 0, 63], dtype=torch.int32, device=DEV)
+    buf = to_dev(qkv.clone())
+    ops.rope_store(buf, cos, sin, slots, k_pages, v_pages, nh, nkv, hd)
+    q_want = llama.rope(qkv[:, :nh * hd].double().reshape(n, nh, hd), pos, theta)
+    k_want = llama.rope(qkv[:, nh * hd:(nh + nkv) * hd].double().reshape(n, nkv, hd), pos, theta)
+    got_q = buf.cpu()[:, :nh * hd].double().reshape(n, nh, hd)
+    assert (got_q - q_want).abs().max().item() < 1e-5
+    assert torch.equal(got_q[0], qkv[0, :nh * hd].double().reshape(nh, hd)), "position 0 must leave the vector as it is"
+    for i, s in enumerate(slots.tolist()):
+        got_k = k_pages[s // page, :, s % page, :].cpu().double()
+        got_v = v_pages[s // page, :, s % page, :].cpu()
+        assert (got_k - k_want[i]).abs().max().item() < 1e-5
+        assert torch.equal(got_v, qkv[i, (nh + nkv) * hd:].reshape(nkv, hd))
+
+
+# ---------------------------------------------------------------------- attention
+def paged_setup(ctx_lens, nkv, hd, page, seed, dtype, scatter=True):
+    """Keys and values of several requests scattered over pages in a shuffled order."""
+    g = torch.Generator().manual_seed(seed)
+    total_pages = sum(-(-c // page) for c in ctx_lens) + 3
+    perm = torch.randperm(total_pages, generator=g).tolist() if scatter else list(range(total_pages))
+    k_pages = torch.randn(total_pages, nkv, page, hd, generator=g).to(dtype)   # unowned slots hold junk
+    v_pages = torch.randn(total_pages, nkv, page, hd, generator=g).to(dtype)
+    tables, ks, vs = [], [], []
+    for c in ctx_lens:
+        np_ = -(-c // page)
+        t = [perm.pop() for _ in range(np_)]
+        tables.append(t)
+        k = torch.randn(c, nkv, hd, generator=g).to(dtype)
+        v = torch.randn(c, nkv, hd, generator=g).to(dtype)
+        for p in range(c):
+            k_pages[t[p // page], :, p % page, :] = k[p]
+            v_pages[t[p // page], :, p % page, :] = v[p]
+        ks.append(k)
+        vs.append(v)
+    maxp = max(len(t) for t in tables)
+    table_t = torch.tensor([t + [-1] * (maxp - len(t)) for t in tables], dtype=torch.int32)
+    return k_pages, v_pages, table_t, ks, vs
+
+
+def plain_attention_rows(q, ks, vs, tok_seq, positions, nh, scale, window):
+    out = torch.zeros_like(q, dtype=torch.float64)
+    n, _ = q.shape
+    hd = ks[0].shape[-1]
+    group = nh // ks[0].shape[1]
+    for i in range(n):
+        k, v, p = ks[tok_seq[i]].double(), vs[tok_seq[i]].double(), positions[i]
+        lo = max(0, p - window + 1) if window else 0
+        for h in range(nh):
+            s = (k[lo:p + 1, h // group] @ q[i, h * hd:(h + 1) * hd].double()) * scale
+            w = torch.softmax(s, 0)
+            out[i, h * hd:(h + 1) * hd] = w @ v[lo:p + 1, h // group]
+    return out
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("nh,nkv,hd,window", [(4, 2, 16, 0), (3, 1, 32, 0), (6, 2, 48, 0), (8, 8, 64, 0),
+                                              (8, 2, 128, 0), (5, 5, 80, 0), (4, 2, 32, 37), (2, 1, 256, 0)])
+def test_attention_plain_kernel(dtype, nh, nkv, hd, window):
+    from glassbox_amd import ops
+    page = 16
+    ctx_lens = [1, 300, 77, 16, 530]
+    k_pages, v_pages, tables, ks, vs = paged_setup(ctx_lens, nkv, hd, page, seed=hd + nh, dtype=dtype)
+    # rows: the last token of every request, plus a portion in the middle of request 1 and the first tokens of 4
+    tok_seq = [0, 1, 2, 3, 4] + [1] * 5 + [4] * 3
+    positions = [c - 1 for c in ctx_lens] + [100, 101, 102, 103, 104] + [0, 1, 2]
+    n = len(tok_seq)
+    q = rnd(n, nh * hd, seed=11).to(dtype)
+    scale = 1 / math.sqrt(hd)
+    out = torch.empty(n, nh * hd, device=DEV, dtype=dtype)
+    ops.attention_plain(to_dev(q), out, torch.tensor(positions, dtype=torch.int32, device=DEV),
+                        torch.tensor(tok_seq, dtype=torch.int32, device=DEV), to_dev(tables), to_dev(k_pages),
+                        to_dev(v_pages), nh, scale, window)
+    want = plain_attention_rows(q, ks, vs, tok_seq, positions, nh, scale, window)
+    tol = 2e-5 if dtype == torch.float32 else 2 ** -7
+    err = (out.cpu().double() - want).abs().max().item()
+    assert err < tol, err
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_attention_finds_one_far_key(dtype):
+    """One key among hundreds is made to stand out: the output must be its value, wherever it lies
+    (first or last slot of a page, first page, a page far away)."""
+    from glassbox_amd import ops
+    nh, nkv, hd, page, ctx = 4, 2, 32, 16, 700
+    k_pages, v_pages, tables, ks, vs = paged_setup([ctx], nkv, hd, page, seed=1, dtype=dtype)
+    q = rnd(1, nh * hd, seed=2).to(dtype)
+    for target in (0, 15, 16, 255, 256, 511, 683, 699):
+        kp = k_pages.clone()
+        for kvh in range(nkv):
+            # the key at `target` points along the mean query of its group, scaled up
+            qg = q[0].float().reshape(nh, hd)[kvh * 2:(kvh + 1) * 2]
+            key = torch.stack([qg[0], qg[1]]).mean(0)
+            # make both heads of the group agree on the direction: use head 0's query for both
+            kp[tables[0, target // page], kvh, target % page, :] = (qg[0] * 40).to(dtype)
+        qq = q.clone().float().reshape(nh, hd)
+        qq[1::2] = qq[0::2]   # both heads of a group ask the same
+        qq = qq.reshape(1, nh * hd).to(dtype)
+        out = torch.empty(1, nh * hd, device=DEV, dtype=dtype)
+        ops.attention_plain(to_dev(qq), out, torch.tensor([ctx - 1], dtype=torch.int32, device=DEV),
+                            torch.tensor([0], dtype=torch.int32, device=DEV), to_dev(tables), to_dev(kp),
+                            to_dev(v_pages), nh, 1 / math.sqrt(hd), 0)
+        want = vs[0][target].float().repeat_interleave(2, 0).reshape(-1)
+        assert (out.cpu().float()[0] - want).abs().max().item() < 2e-2, f"key at {target} was not found"
+
+
+def test_copy_rows():
+    from glassbox_amd import ops
+    base = rnd(6, 3, 10, seed=1).to(DEV)
+    want = base.clone()
+    want[4], want[0] = want[1].clone(), want[5].clone()
+    ops.copy_rows(base, torch.tensor([1, 5], dtype=torch.int32, device=DEV), torch.tensor([4, 0], dtype=torch.int32, device=DEV))
+    assert torch.equal(base, want)
