@@ -75,7 +75,7 @@ class Engine:
 
         self.workspace = Workspace(self.device)
         self._ids: Dict[Hashable, int] = {}
-        self._next_id = 1
+        self._next_id = 1 << 40   # the scheduler numbers its requests from 1 in the same cache manager
         self._meta_dev: Optional[torch.Tensor] = None
         self.steps = 0
 
@@ -147,35 +147,54 @@ class Engine:
                     ops.copy_rows(lc.k_pages, src, dst)   # copy-on-write in every layer (kv.rs:189-196)
                     ops.copy_rows(lc.v_pages, src, dst)
 
-    def step(self, entries: Sequence[Entry], commit: bool = True, reserved: bool = False) -> torch.Tensor:
+    def step(self, entries: Sequence[Entry]) -> torch.Tensor:
         """Runs exactly the given tokens, as one batch, from the cache that earlier steps left.
 
-        Returns float32 logits [wanted, vocab] in the order of the entries and of their wanted
-        places.  The tensor is a view of the engine's workspace: use it before the next step."""
+        Reserves pages (raising OutOfPages if the pool is too small), runs, commits.  Returns
+        float32 logits [wanted, vocab] in the order of the entries and of their wanted places.
+        The tensor is a view of the engine's workspace: use it before the next step."""
         entries = [(r, list(t), list(w)) for r, t, w in entries]
-        if not entries:
-            return torch.empty((0, self.model.vocab_size), dtype=torch.float32, device=self.device)
         seen = set()
-        vocab = self.model.vocab_size
-        for request, tokens, want in entries:
+        for request, _, _ in entries:
             if request in seen:
                 raise EngineError(f"request {request!r} appears twice in one step")
             seen.add(request)
+        self._validate(entries)
+        self.reserve(entries)
+        by_id = [(self._ids[r], t, w) for r, t, w in entries]
+        logits = self.run_reserved(by_id)
+        for sid, tokens, _ in by_id:
+            self.cache.commit(sid, tokens)
+        return logits
+
+    def _validate(self, entries) -> None:
+        vocab = self.model.vocab_size
+        for request, tokens, want in entries:
             if not tokens:
                 raise EngineError(f"request {request!r} brings no tokens")
             if min(tokens) < 0 or max(tokens) >= vocab:
                 raise EngineError(f"request {request!r}: token ids must lie in 0..{vocab - 1}")
             if any(w < 0 or w >= len(tokens) for w in want):
                 raise EngineError(f"request {request!r}: wanted places must lie among its {len(tokens)} tokens")
-        if not reserved:
-            self.reserve(entries)
+
+    def run_reserved(self, entries: Sequence[Tuple[int, List[int], List[int]]]) -> torch.Tensor:
+        """The step itself, on the cache manager's own request numbers: pages for the tokens are
+        reserved already and nothing is committed (the scheduler does both around this call)."""
+        if not entries:
+            return torch.empty((0, self.model.vocab_size), dtype=torch.float32, device=self.device)
+        self._validate(entries)
+        self._apply_copies()
         ctx = self._build_context(entries)
         logits = self.model.forward(ctx, self.layers)
-        if commit:
-            for request, tokens, _ in entries:
-                self.cache.commit(self._ids[request], tokens)
         self.steps += 1
         return logits
+
+    def reset_state(self, sid: int) -> None:
+        """Empties the state slot of a request that starts (again) from its first token."""
+        slot = self.cache.state_slot(sid)
+        for lc in self.layers:
+            if lc.state is not None and slot >= 0:
+                lc.state[slot].zero_()
 
     # ---------------------------------------------------------------- metadata
     def _build_context(self, entries) -> StepContext:
@@ -192,8 +211,7 @@ class Engine:
         slots_host: List[List[int]] = [[] for _ in range(G)]
         want_flat: List[Tuple[int, int, int]] = []   # (entry index, place, flat row)
         for s, ei in enumerate(order):
-            request, tokens, want = entries[ei]
-            sid = self._ids[request]
+            sid, tokens, want = entries[ei]
             start = self.cache.seq_len(sid)
             q_start.append(len(token_ids))
             q_len.append(len(tokens))

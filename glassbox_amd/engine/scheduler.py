@@ -1,0 +1,216 @@
+"""Continuous batching above Engine: the Python face of the host scheduler
+(csrc/host/scheduler.cpp), which follows the reference's Scheduler
+(crates/glassbox-server/src/scheduler.rs).
+
+One reference step() is plan -> forward -> sample -> finish.  The decisions (admission, token
+budget, preemption of the newest request when pages run out, stop and length rules) are taken
+by the C++ scheduler; this class runs the planned batch through ``Engine.run_reserved`` and the
+device sampler in between.
+"""
+from __future__ import annotations
+
+import ctypes as C
+import time
+from dataclasses import dataclass, field
+from typing import Dict, List, Optional, Sequence, Tuple
+
+from .. import build
+from ..sampling.sampler import SamplerConfig, sample_rows
+
+STOP, LENGTH, ABORTED = 0, 1, 2
+FINISH_NAMES = {STOP: "stop", LENGTH: "length", ABORTED: "aborted"}
+
+_lib = None
+
+
+def _host():
+    global _lib
+    if _lib is None:
+        lib = build.load("host")
+        vp, i64, i32p, i64p = C.c_void_p, C.c_int64, C.POINTER(C.c_int32), C.POINTER(C.c_int64)
+        ip, fp = C.POINTER(C.c_int), C.POINTER(C.c_float)
+        sig = {
+            "create": (vp, [vp, C.c_int, C.c_int, C.c_int]),
+            "destroy": (None, [vp]),
+            "submit": (i64, [vp, i32p, C.c_int, C.c_int, C.c_float, C.c_int, C.c_float, C.c_float, C.c_float,
+                             C.c_uint64, i32p, C.c_int]),
+            "abort": (C.c_int, [vp, i64]),
+            "is_idle": (C.c_int, [vp]), "waiting": (C.c_int, [vp]), "running": (C.c_int, [vp]),
+            "plan": (C.c_int, [vp]), "plan_size": (C.c_int, [vp]), "plan_tokens": (C.c_int, [vp]),
+            "plan_entry": (None, [vp, C.c_int, i64p, ip, ip, ip, ip]),
+            "plan_entry_tokens": (None, [vp, C.c_int, i32p]),
+            "row_params": (None, [vp, C.c_int, fp, ip, fp, fp, fp, fp, ip]),
+            "row_context": (C.c_int, [vp, C.c_int, i32p, C.c_int]),
+            "finish": (None, [vp, i32p, i32p, C.c_int]),
+            "take_events": (C.c_int, [vp, i64p, i32p, i32p, C.c_int]),
+            "request_counts": (C.c_int, [vp, i64, ip, ip]),
+            "metrics": (None, [vp, i64p]),
+            "last_preempted": (C.c_int, [vp, i64p, C.c_int]),
+        }
+        for name, (res, args) in sig.items():
+            fn = getattr(lib, "gbh_sched_" + name)
+            fn.restype, fn.argtypes = res, args
+        _lib = lib
+    return _lib
+
+
+@dataclass
+class SchedulerConfig:
+    """scheduler.rs:54-74.  The number of pages is the engine's (its ``max_tokens``)."""
+    token_budget: int = 256
+    max_seqs: int = 32
+
+
+@dataclass
+class RequestOutput:
+    tokens: List[int] = field(default_factory=list)
+    finish: Optional[str] = None
+    prompt_tokens: int = 0
+
+
+@dataclass
+class StepRecord:
+    """What one step did (scheduler.rs:104-115)."""
+    step: int
+    ms: float
+    batch: List[Tuple[int, str, int]]
+    preempted: List[int]
+    finished: List[int]
+    waiting: int
+    kv_used: int
+
+
+class Scheduler:
+    def __init__(self, engine, config: Optional[SchedulerConfig] = None, trace: bool = False, sample_fn=None):
+        self.engine = engine
+        #: (logits, configs, uniforms, contexts) -> (tokens, candidates); the device sampler by default
+        self.sample_fn = sample_fn or sample_rows
+        self.config = config or SchedulerConfig()
+        if self.config.max_seqs > engine.max_seqs:
+            raise ValueError(f"max_seqs {self.config.max_seqs} exceeds the engine's state slots ({engine.max_seqs})")
+        self._lib = _host()
+        max_pos = getattr(engine.model.config, "max_position_embeddings", 1 << 30)
+        self._h = C.c_void_p(self._lib.gbh_sched_create(engine.cache.handle, self.config.token_budget,
+                                                        self.config.max_seqs, max_pos))
+        self.outputs: Dict[int, RequestOutput] = {}
+        self.trace: Optional[List[StepRecord]] = [] if trace else None
+        self._steps = 0
+
+    def __del__(self):
+        h, self._h = getattr(self, "_h", None), None
+        if h:
+            self._lib.gbh_sched_destroy(h)
+
+    # ------------------------------------------------------------------ requests
+    def submit(self, prompt: Sequence[int], max_tokens: int, sampler: Optional[SamplerConfig] = None,
+               stop: Sequence[int] = ()) -> int:
+        if not prompt:
+            raise ValueError("a request needs at least one prompt token")
+        vocab = self.engine.model.vocab_size
+        if min(prompt) < 0 or max(prompt) >= vocab:
+            raise ValueError(f"prompt token ids must lie in 0..{vocab - 1}")
+        s = sampler or SamplerConfig()
+        p = (C.c_int32 * len(prompt))(*prompt)
+        st = (C.c_int32 * max(1, len(stop)))(*stop)
+        rid = self._lib.gbh_sched_submit(self._h, p, len(prompt), max_tokens, s.temperature, s.top_k, s.top_p,
+                                         s.min_p, s.repetition_penalty, s.seed, st, len(stop))
+        self.outputs[rid] = RequestOutput(prompt_tokens=len(prompt))
+        return rid
+
+    def abort(self, rid: int) -> None:
+        self._lib.gbh_sched_abort(self._h, rid)
+        self._drain_events()
+
+    def is_idle(self) -> bool:
+        return bool(self._lib.gbh_sched_is_idle(self._h))
+
+    def queue_depth(self) -> int:
+        return self._lib.gbh_sched_waiting(self._h)
+
+    def running(self) -> int:
+        return self._lib.gbh_sched_running(self._h)
+
+    # ---------------------------------------------------------------------- step
+    def step(self) -> bool:
+        """One batch through the model.  False when there was nothing to do (scheduler.rs:239)."""
+        t0 = time.perf_counter()
+        lib, h = self._lib, self._h
+        rc = lib.gbh_sched_plan(h)
+        if rc != 1:
+            finished = self._drain_events()
+            self._record(t0, [], finished)
+            return rc == 2
+        n = lib.gbh_sched_plan_size(h)
+        entries, batch_desc = [], []
+        rid, start, cnt, wants, dec = C.c_int64(), C.c_int(), C.c_int(), C.c_int(), C.c_int()
+        for i in range(n):
+            lib.gbh_sched_plan_entry(h, i, C.byref(rid), C.byref(start), C.byref(cnt), C.byref(wants), C.byref(dec))
+            buf = (C.c_int32 * cnt.value)()
+            lib.gbh_sched_plan_entry_tokens(h, i, buf)
+            if start.value == 0:
+                self.engine.reset_state(rid.value)
+            entries.append((rid.value, list(buf), [cnt.value - 1] if wants.value else []))
+            batch_desc.append((rid.value, "decode" if dec.value else "prefill", cnt.value))
+        logits = self.engine.run_reserved(entries)
+        rows = logits.shape[0]
+        configs, uniforms, contexts, skip = [], [], [], []
+        t, k, tp, mp, rp, u, sk = C.c_float(), C.c_int(), C.c_float(), C.c_float(), C.c_float(), C.c_float(), C.c_int()
+        for j in range(rows):
+            lib.gbh_sched_row_params(h, j, C.byref(t), C.byref(k), C.byref(tp), C.byref(mp), C.byref(rp), C.byref(u),
+                                     C.byref(sk))
+            configs.append(SamplerConfig(t.value, k.value, tp.value, mp.value, rp.value))
+            uniforms.append(u.value)
+            skip.append(sk.value)
+            if rp.value != 1.0:
+                m = lib.gbh_sched_row_context(h, j, None, 0)
+                cb = (C.c_int32 * max(1, m))()
+                lib.gbh_sched_row_context(h, j, cb, m)
+                contexts.append(list(cb[:m]))
+            else:
+                contexts.append([])
+        tokens, cands = self.sample_fn(logits, configs, uniforms, contexts) if rows else ([], [])
+        lib.gbh_sched_finish(h, (C.c_int32 * max(1, rows))(*tokens), (C.c_int32 * max(1, rows))(*cands), rows)
+        finished = self._drain_events()
+        self._steps += 1
+        self._record(t0, batch_desc, finished)
+        return True
+
+    def run(self, max_steps: int = 1 << 30) -> None:
+        steps = 0
+        while not self.is_idle() and steps < max_steps:
+            self.step()
+            steps += 1
+
+    def _drain_events(self) -> List[int]:
+        finished = []
+        cap = 4096
+        ids, kinds, vals = (C.c_int64 * cap)(), (C.c_int32 * cap)(), (C.c_int32 * cap)()
+        while True:
+            n = self._lib.gbh_sched_take_events(self._h, ids, kinds, vals, cap)
+            for i in range(min(n, cap)):
+                out = self.outputs.setdefault(ids[i], RequestOutput())
+                if kinds[i] == 0:
+                    out.tokens.append(vals[i])
+                else:
+                    out.finish = FINISH_NAMES[vals[i]]
+                    finished.append(ids[i])
+            if n <= cap:
+                return finished
+
+    def _record(self, t0: float, batch, finished) -> None:
+        if self.trace is None:
+            return
+        pre = (C.c_int64 * 64)()
+        npre = self._lib.gbh_sched_last_preempted(self._h, pre, 64)
+        self.trace.append(StepRecord(self._steps, (time.perf_counter() - t0) * 1e3, list(batch),
+                                     list(pre[:min(npre, 64)]), list(finished), self.queue_depth(),
+                                     self.engine.cache.used_pages() if self.engine.group_keys else 0))
+
+    @property
+    def metrics(self) -> Dict[str, int]:
+        """scheduler.rs:117-130 (the counters)."""
+        out = (C.c_int64 * 7)()
+        self._lib.gbh_sched_metrics(self._h, out)
+        names = ["requests_finished", "prompt_tokens", "generated_tokens", "prefix_hit_tokens", "preemptions",
+                 "steps", "batch_tokens"]
+        return dict(zip(names, out))

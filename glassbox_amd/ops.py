@@ -63,7 +63,7 @@ _SIGS = {
     "sampling": {
         "gb_argmax": [_vp, _vp, _i, _i, _vp],
         "gb_penalize": [_vp, _i, _vp, _vp, _vp, _vp, _i, _vp],
-        "gb_sample": [_vp, _i, _i, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp],
+        "gb_sample": [_vp, _i, _i, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp],
     },
 }
 _libs = {}
@@ -268,3 +268,47 @@ def attention_plain(q: torch.Tensor, out: torch.Tensor, positions: torch.Tensor,
 def tuned_attention_supports(k_pages: torch.Tensor, n_heads: int, window: int) -> bool:
     """Whether the tuned bfloat16 attention kernels take this layer's sizes."""
     return False
+
+
+# ------------------------------------------------------------------------ sampling
+def _logit_rows(logits: torch.Tensor):
+    if logits.dtype != torch.float32 or logits.dim() != 2 or not logits.is_contiguous() or not logits.is_cuda:
+        raise KernelError("sampling works on contiguous float32 logits [rows, vocab] on the GPU")
+    return logits.shape
+
+
+def argmax(logits: torch.Tensor, out: torch.Tensor) -> None:
+    """out[r] = index of the first maximum of row r."""
+    rows, vocab = _logit_rows(logits)
+    _i32(out, "out", rows)
+    lib = _lib("sampling")
+    _check(lib, lib.gb_argmax(_p(logits), _p(out), rows, vocab, _stream()))
+
+
+def penalize(logits: torch.Tensor, rows: torch.Tensor, tokens: torch.Tensor, counts: torch.Tensor,
+             penalties: torch.Tensor) -> None:
+    """In place, for every (row, token, count, penalty): count times v = v / pen if v > 0 else v * pen."""
+    _, vocab = _logit_rows(logits)
+    pairs = rows.numel()
+    for t, what in ((rows, "rows"), (tokens, "tokens"), (counts, "counts")):
+        _i32(t, what, pairs)
+    if penalties.dtype != torch.float32 or penalties.numel() < pairs:
+        raise KernelError("penalize: penalties must be float32, one per pair")
+    lib = _lib("sampling")
+    _check(lib, lib.gb_penalize(_p(logits), vocab, _p(rows), _p(tokens), _p(counts), _p(penalties), pairs, _stream()))
+
+
+def sample(logits: torch.Tensor, temperature: torch.Tensor, top_k: torch.Tensor, top_p: torch.Tensor,
+           min_p: torch.Tensor, uniform: torch.Tensor, out_token: torch.Tensor, out_candidates: torch.Tensor) -> None:
+    """The reference's sampler per row: temperature, top-k, min-p, top-p, then an inverse-CDF draw in
+    descending order of probability with the given uniform number; temperature <= 0 is greedy."""
+    rows, vocab = _logit_rows(logits)
+    for t, what in ((temperature, "temperature"), (top_p, "top_p"), (min_p, "min_p"), (uniform, "uniform")):
+        if t.dtype != torch.float32 or t.numel() < rows or not t.is_cuda:
+            raise KernelError(f"sample: {what} must be float32 on the GPU, one per row")
+    _i32(top_k, "top_k", rows)
+    _i32(out_token, "out_token", rows)
+    _i32(out_candidates, "out_candidates", rows)
+    lib = _lib("sampling")
+    _check(lib, lib.gb_sample(_p(logits), rows, vocab, _p(temperature), _p(top_k), _p(top_p), _p(min_p), _p(uniform),
+                              _p(out_token), _p(out_candidates), _stream()))

@@ -1,0 +1,187 @@
+"""Configuration, registry, safetensors reading and the weight errors (no GPU)."""
+import json
+import os
+
+import pytest
+import torch
+
+import helpers
+from glassbox_amd.config import (ConfigError, LlamaConfig, config_from_dict, config_from_dir, known_architectures,
+                                 register_architecture)
+from glassbox_amd.weights import (SafetensorsFile, WeightError, build_model, load_weights, save_file,
+                                  write_random_model)
+from plain import llama as plain
+
+
+def test_defaults_follow_the_reference():
+    # crates/glassbox-core/src/model.rs:15-35
+    cfg = config_from_dict(dict(architectures=["LlamaForCausalLM"], hidden_size=64, intermediate_size=128,
+                                num_hidden_layers=2, num_attention_heads=4, num_key_value_heads=2, vocab_size=97))
+    assert isinstance(cfg, LlamaConfig)
+    assert cfg.rms_norm_eps == 1e-5 and cfg.rope_theta == 10000.0 and cfg.tie_word_embeddings is False
+    assert cfg.max_position_embeddings == 2048 and cfg.head_dim is None
+    assert cfg.head_size == 16 and cfg.kv_dim == 32 and cfg.q_dim == 64
+
+
+def test_rope_theta_is_lifted_from_rope_parameters():
+    # model.rs:39-47
+    raw = dict(helpers.TINY_A)
+    del raw["rope_theta"]
+    raw["rope_parameters"] = {"rope_theta": 130000.0, "rope_type": "default"}
+    assert config_from_dict(raw).rope_theta == 130000.0
+
+
+def test_explicit_head_dim_and_every_key_is_read():
+    cfg = config_from_dict(helpers.TINY_B)
+    assert cfg.head_size == 32 and cfg.q_dim == 96 and cfg.kv_dim == 32
+    assert cfg.rms_norm_eps == 1e-6 and cfg.rope_theta == 500000.0 and not cfg.tie_word_embeddings
+    assert cfg.max_position_embeddings == 256 and cfg.vocab_size == 384 and cfg.intermediate_size == 256
+
+
+def test_missing_keys_are_listed_together():
+    with pytest.raises(ConfigError) as e:
+        config_from_dict(dict(architectures=["LlamaForCausalLM"], hidden_size=64))
+    for key in ("intermediate_size", "num_hidden_layers", "num_attention_heads", "num_key_value_heads", "vocab_size"):
+        assert key in str(e.value)
+
+
+@pytest.mark.parametrize("patch,word", [
+    ({"rope_scaling": {"rope_type": "llama3", "factor": 8.0}}, "rope_scaling"),
+    ({"attention_bias": True}, "attention_bias"),
+    ({"mlp_bias": True}, "mlp_bias"),
+    ({"hidden_act": "gelu"}, "hidden_act"),
+    ({"num_key_value_heads": 3}, "multiple"),
+    ({"head_dim": 15}, "odd"),
+    ({"hidden_size": "64"}, "integer"),
+    ({"vocab_size": 0}, "positive"),
+])
+def test_unsupported_options_are_refused(patch, word):
+    with pytest.raises(ConfigError, match=word):
+        config_from_dict(dict(helpers.TINY_A, **patch))
+
+
+def test_unknown_architecture_lists_the_known_ones():
+    with pytest.raises(ConfigError, match="LlamaForCausalLM"):
+        config_from_dict(dict(helpers.TINY_A, architectures=["NopeForCausalLM"]))
+    assert "LlamaForCausalLM" in known_architectures()
+    raw = dict(helpers.TINY_A)
+    del raw["architectures"]
+    raw["model_type"] = "llama"
+    assert isinstance(config_from_dict(raw), LlamaConfig)
+
+
+def test_a_new_architecture_registers_without_touching_the_package():
+    class Toy(LlamaConfig):
+        architecture = "ToyForCausalLM"
+    register_architecture("ToyForCausalLM", Toy, lambda cfg: ("built", cfg))
+    cfg = config_from_dict(dict(helpers.TINY_A, architectures=["ToyForCausalLM"]))
+    assert type(cfg) is Toy and build_model(cfg)[0] == "built"
+
+
+def test_config_round_trip_through_a_folder(tmp_path):
+    cfg = config_from_dict(helpers.TINY_B)
+    cfg.save(str(tmp_path))
+    assert config_from_dir(str(tmp_path)) == cfg
+    with pytest.raises(ConfigError, match="no such file"):
+        config_from_dir(str(tmp_path / "nope"))
+
+
+def test_random_model_folder_and_names(tmp_path):
+    folder = write_random_model(config_from_dict(helpers.TINY_B), str(tmp_path / "b"), seed=3)
+    f = SafetensorsFile(os.path.join(folder, "model.safetensors"))
+    names = set(f.names())
+    # crates/glassbox-core/src/load.rs:52-78
+    for i in range(3):
+        for leaf in ("input_layernorm.weight", "self_attn.q_proj.weight", "self_attn.k_proj.weight",
+                     "self_attn.v_proj.weight", "self_attn.o_proj.weight", "post_attention_layernorm.weight",
+                     "mlp.gate_proj.weight", "mlp.up_proj.weight", "mlp.down_proj.weight"):
+            assert f"model.layers.{i}.{leaf}" in names
+    assert {"model.embed_tokens.weight", "model.norm.weight", "lm_head.weight"} <= names
+    assert len(names) == 3 * 9 + 3
+    assert f.shape("model.layers.0.self_attn.k_proj.weight") == (32, 96)
+    assert f.shape("lm_head.weight") == (384, 96)
+    w = f.tensor("model.layers.1.mlp.down_proj.weight")
+    assert abs(w.std().item() - 0.02) < 0.002 and torch.all(f.tensor("model.norm.weight") == 1.0)
+    # the same seed gives the same file, another seed another
+    again = write_random_model(config_from_dict(helpers.TINY_B), str(tmp_path / "b2"), seed=3)
+    other = write_random_model(config_from_dict(helpers.TINY_B), str(tmp_path / "b3"), seed=4)
+    rd = lambda d: open(os.path.join(d, "model.safetensors"), "rb").read()
+    assert rd(folder) == rd(again) and rd(folder) != rd(other)
+    # tied model: no head in the file
+    tied = write_random_model(config_from_dict(helpers.TINY_A), str(tmp_path / "a"), seed=3)
+    assert "lm_head.weight" not in set(SafetensorsFile(os.path.join(tied, "model.safetensors")).names())
+
+
+def test_safetensors_reader_agrees_with_the_plain_reader_and_keeps_bfloat16(tmp_path):
+    t = {"a": torch.randn(3, 5), "b": torch.randn(7).bfloat16(), "c": torch.arange(6, dtype=torch.int32).reshape(2, 3)}
+    path = str(tmp_path / "x.safetensors")
+    save_file(t, path)
+    f = SafetensorsFile(path)
+    assert f.tensor("b").dtype == torch.bfloat16 and torch.equal(f.tensor("b"), t["b"])
+    assert torch.equal(f.tensor("a"), t["a"]) and torch.equal(f.tensor("c"), t["c"])
+    mine = plain.read_safetensors(path) if False else None  # the plain reader knows float types only
+    del t["c"]
+    save_file(t, path)
+    got = plain.read_safetensors(path)
+    assert torch.equal(got["a"], t["a"]) and torch.equal(got["b"], t["b"].float())
+
+
+def test_one_error_lists_missing_unexpected_and_wrong_shapes(tmp_path):
+    cfg = config_from_dict(helpers.TINY_B)
+    folder = write_random_model(cfg, str(tmp_path / "b"), seed=0)
+    path = os.path.join(folder, "model.safetensors")
+    f = SafetensorsFile(path)
+    tensors = {n: f.tensor(n).clone() for n in f.names()}
+    del tensors["model.layers.1.mlp.up_proj.weight"]
+    del tensors["lm_head.weight"]                                   # untied model without a head: an error here
+    tensors["model.layers.0.self_attn.rotary_emb.inv_freq"] = torch.zeros(16)
+    tensors["model.layers.2.self_attn.q_proj.weight"] = torch.zeros(96, 95)
+    tensors["model.norm.weight"] = torch.zeros(97)
+    save_file(tensors, path)
+    with pytest.raises(WeightError) as e:
+        load_weights(build_model(cfg), path, torch.float32, "cpu")
+    msg = str(e.value)
+    assert "missing tensors (2)" in msg and "model.layers.1.mlp.up_proj.weight" in msg and "lm_head.weight" in msg
+    assert "unexpected tensors (1)" in msg and "rotary_emb.inv_freq" in msg
+    assert "wrong shapes (2)" in msg and "model.layers.2.self_attn.q_proj.weight is [96, 95], expected [96, 96]" in msg
+    assert "model.norm.weight is [97], expected [96]" in msg
+
+
+def test_a_tied_checkpoint_may_carry_a_head(tmp_path):
+    cfg = config_from_dict(helpers.TINY_A)
+    folder = write_random_model(cfg, str(tmp_path / "a"), seed=0)
+    path = os.path.join(folder, "model.safetensors")
+    f = SafetensorsFile(path)
+    tensors = {n: f.tensor(n).clone() for n in f.names()}
+    tensors["lm_head.weight"] = torch.zeros(256, 64)   # ignored, as the reference does (load.rs:70-75)
+    save_file(tensors, path)
+    model = build_model(cfg)
+    load_weights(model, path, torch.float32, "cpu")
+    assert model.head.matrix() is model.embedding.table
+
+
+def test_types_on_the_device(tmp_path):
+    """Matrices follow the compute type; a vector stored in 32-bit stays so; 16-bit stays bfloat16."""
+    cfg = config_from_dict(helpers.TINY_A)
+    for stored in (torch.float32, torch.bfloat16):
+        folder = write_random_model(cfg, str(tmp_path / str(stored)), seed=0, dtype=stored)
+        path = os.path.join(folder, "model.safetensors")
+        m = build_model(cfg)
+        load_weights(m, path, torch.bfloat16, "cpu")
+        assert m.blocks[0].mixer.wqkv.dtype == torch.bfloat16 and m.embedding.table.dtype == torch.bfloat16
+        assert m.final_norm.weight.dtype == stored
+        assert m.blocks[0].mixer.wqkv.shape == (64 + 2 * 32, 64)          # q, k, v stacked (model.rs:59-61)
+        assert m.blocks[1].ffn.w_gate_up.shape == (2 * 176, 64)
+        m = build_model(cfg)
+        load_weights(m, path, torch.float32, "cpu")
+        assert m.blocks[0].mixer.wqkv.dtype == torch.float32 and m.final_norm.weight.dtype == torch.float32
+
+
+def test_bad_files(tmp_path):
+    cfg = config_from_dict(helpers.TINY_A)
+    with pytest.raises(WeightError, match="no such file"):
+        load_weights(build_model(cfg), str(tmp_path / "none.safetensors"), torch.float32, "cpu")
+    p = tmp_path / "short.safetensors"
+    p.write_bytes(b"abc")
+    with pytest.raises(WeightError, match="too short"):
+        load_weights(build_model(cfg), str(p), torch.float32, "cpu")

@@ -1,0 +1,217 @@
+"""Sampling kernels, the Python entry points and the scheduler on the GPU."""
+import math
+import random
+
+import numpy as np
+import pytest
+import torch
+
+import helpers
+from plain import llama as plain
+from plain import sampler as psampler
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda:0"
+
+
+# ------------------------------------------------------------------ sampling kernels
+def test_argmax_first_maximum_wins():
+    from glassbox_amd import ops
+    g = torch.Generator().manual_seed(0)
+    for vocab in (5, 331, 49152):
+        logits = torch.randn(6, vocab, generator=g)
+        logits[1, 3] = logits[1, vocab - 1] = 9.0            # a tie: the first one
+        logits[2, vocab - 1] = 10.0
+        logits[3, :] = -1.5                                  # all equal: token 0
+        logits[4, 0] = 11.0
+        out = torch.empty(6, dtype=torch.int32, device=DEV)
+        ops.argmax(logits.to(DEV), out)
+        assert out.tolist() == [psampler.argmax(r) for r in logits.tolist()]
+        assert out.tolist()[1:5] == [3, vocab - 1, 0, 0]
+
+
+def test_sampler_vectors_of_the_reference_on_the_device():
+    # crates/glassbox-core/src/sampler.rs:188-218
+    from glassbox_amd.sampling import SamplerConfig, sample_rows
+    logits = torch.tensor([[1.0, 3.0, 2.0, 0.0, -1.0]] * 4, device=DEV)
+    cfgs = [SamplerConfig(), SamplerConfig(temperature=1.0, top_k=2), SamplerConfig(temperature=1.0, top_p=0.5),
+            SamplerConfig(temperature=1.0, min_p=0.3)]
+    toks, cands = sample_rows(logits.clone(), cfgs, [0.99] * 4)
+    assert cands == [1, 2, 1, 2]
+    assert toks == [1, 2, 1, 2]            # u = 0.99 falls on the last candidate of each distribution
+    toks, _ = sample_rows(logits.clone(), cfgs, [0.0] * 4)
+    assert toks == [1, 1, 1, 1]
+    # p0 = 1 / (1 + e^-1) = 0.731 with top_k = 2: the draw turns at that value
+    assert sample_rows(logits[:1].clone(), [cfgs[1]], [0.73])[0] == [1]
+    assert sample_rows(logits[:1].clone(), [cfgs[1]], [0.7320])[0] == [2]
+    # repetition penalty 4 on token 1 makes token 2 the maximum (sampler.rs:213-217)
+    toks, _ = sample_rows(logits[:1].clone(), [SamplerConfig(repetition_penalty=4.0)], [0.0], [[1]])
+    assert toks == [2]
+
+
+@pytest.mark.parametrize("vocab", [97, 331, 49152])
+def test_sampling_kernel_agrees_with_the_plain_sampler(vocab):
+    from glassbox_amd.sampling import SamplerConfig, sample_rows
+    g = torch.Generator().manual_seed(vocab)
+    rng = random.Random(vocab)
+    rows = 24 if vocab < 1000 else 6
+    logits = torch.randn(rows, vocab, generator=g) * 3
+    logits[0, 5] = logits[0, 9] = logits[0].max() + 1         # ties at the top go by token id
+    logits[1, :] = 0.25                                        # every logit equal
+    cfgs, ctxs, us = [], [], []
+    for r in range(rows):
+        cfgs.append(SamplerConfig(temperature=rng.choice([0.0, 0.6, 1.0, 2.0]), top_k=rng.choice([0, 0, 1, 7, 50]),
+                                  top_p=rng.choice([1.0, 1.0, 0.95, 0.6, 0.1]), min_p=rng.choice([0.0, 0.0, 0.02, 0.3]),
+                                  repetition_penalty=rng.choice([1.0, 1.0, 1.2, 3.0])))
+        ctxs.append([rng.randrange(vocab) for _ in range(rng.randrange(0, 30))] + [5, 5])
+        us.append(rng.random())
+    toks, cands = sample_rows(logits.to(DEV), cfgs, us, ctxs)
+    for r in range(rows):
+        c = cfgs[r]
+        dist = psampler.distribution(logits[r].tolist(), ctxs[r], c.temperature, c.top_k, c.top_p, c.min_p,
+                                     c.repetition_penalty)
+        assert cands[r] == len(dist), (r, c)
+        acc, want = np.float32(0), dist[-1][0]
+        near_edge = False
+        for t, p in dist:
+            acc = np.float32(acc + np.float32(p))
+            near_edge |= abs(float(acc) - us[r]) < 1e-5       # a draw this close to a boundary may round either way
+            if us[r] < acc:
+                want = t
+                break
+        if len(dist) == 1:
+            want = dist[0][0]
+        assert toks[r] == want or near_edge, (r, c, toks[r], want)
+
+
+def test_temperature_draws_follow_the_softmax():
+    from glassbox_amd.sampling import Rng, SamplerConfig, sample_rows
+    logits = torch.tensor([[0.0, math.log(2.0), math.log(5.0), -30.0]], device=DEV).repeat(64, 1)
+    rng, counts = Rng(3), np.zeros(4)
+    cfg = [SamplerConfig(temperature=1.0)] * 64
+    for _ in range(60):
+        toks, _ = sample_rows(logits.clone(), cfg, [rng.next_f32() for _ in range(64)])
+        for t in toks:
+            counts[t] += 1
+    assert np.abs(counts / counts.sum() - np.array([1, 2, 5, 0]) / 8).max() < 0.03
+    # temperature 2 flattens: p ~ (1, sqrt 2, sqrt 5)
+    counts = np.zeros(4)
+    for _ in range(60):
+        toks, _ = sample_rows(logits.clone(), [SamplerConfig(temperature=2.0)] * 64, [rng.next_f32() for _ in range(64)])
+        for t in toks:
+            counts[t] += 1
+    want = np.array([1, math.sqrt(2), math.sqrt(5), 0])
+    assert np.abs(counts / counts.sum() - want / want.sum()).max() < 0.03
+
+
+# ------------------------------------------------------------------- entry points
+@pytest.mark.parametrize("name", ["A", "B"])
+def test_greedy_generation_through_the_entry_point(model_dirs, name):
+    """generate() against the plain implementation's greedy decoding.  With random weights two
+    logits can lie within rounding of each other; a step whose plain margin is that small may go
+    either way, and the comparison ends there."""
+    from glassbox_amd import Engine, generate
+    folder = model_dirs.get(name)
+    cfg, w = plain.load_folder(folder)
+    vocab = cfg["vocab_size"]
+    prompts = [helpers.random_tokens(vocab, n, seed=n) for n in ((5, 17, 33) if name == "A" else (1, 9, 40, 70))]
+    steps = 16 if name == "A" else 24
+    for dtype, margin in (("float32", 1e-4), ("bfloat16", 3e-2)):
+        eng = Engine(folder, dtype=dtype, max_tokens=1024, max_seqs=8)
+        outs = generate(eng, prompts, max_tokens=steps, token_budget=16 if name == "B" else 256)
+        for p, out in zip(prompts, outs):
+            assert len(out) == steps
+            toks = list(p)
+            for i, t in enumerate(out):
+                logits = plain.forward(w, cfg, toks)[-1]
+                top2 = torch.topk(logits, 2).values
+                if t != int(torch.argmax(logits)):
+                    assert (top2[0] - top2[1]).item() < margin, f"{dtype} prompt {len(p)} step {i}: wrong token"
+                    break
+                toks.append(t)
+        eng.cache.check_invariants()
+        assert eng.cache.used_pages() == 0
+
+
+def test_batched_equals_unbatched_on_the_device(model_dirs):
+    """crates/glassbox-server/tests/scheduler.rs:84-123 with the real model in 32-bit, where every
+    output cell is summed in an order that does not depend on the batch: exact equality."""
+    from glassbox_amd import Engine, generate, greedy
+    folder = model_dirs.get("A")
+    rng = random.Random(4)
+    jobs = [([rng.randrange(256) for _ in range(1 + rng.randrange(60))], 1 + rng.randrange(24)) for _ in range(10)]
+    eng = Engine(folder, dtype="float32", max_tokens=14 * 16, max_seqs=12, prefix_caching=True)
+    alone = [greedy(eng, p, n) for p, n in jobs]
+    assert eng.cache.used_pages() == 0
+    outs, sched = generate(eng, [p for p, _ in jobs], max_tokens=24, token_budget=16, return_scheduler=True)
+    for (p, n), out, ref in zip(jobs, outs, alone):
+        assert out[:n] == ref
+    assert sched.metrics["preemptions"] > 0, "14 pages for 10 requests should force preemption"
+    eng.cache.check_invariants()
+    assert eng.cache.used_pages() == 0
+
+
+def test_prefix_sharing_on_the_device(model_dirs):
+    """A shared 70-token prefix is computed once; outputs equal those without sharing
+    (tests/scheduler.rs:165-186), in 32-bit exactly."""
+    from glassbox_amd import Engine, generate
+    folder = model_dirs.get("A")
+    rng = random.Random(11)
+    system = [(i * 13) % 256 for i in range(70)]
+    prompts = [system + [rng.randrange(256) for _ in range(1 + rng.randrange(40))] for _ in range(8)]
+    res = {}
+    for share in (True, False):
+        eng = Engine(folder, dtype="float32", max_tokens=128 * 16, max_seqs=4, prefix_caching=share)
+        res[share] = generate(eng, prompts, max_tokens=12, token_budget=48, max_seqs=4, return_scheduler=True)
+        assert eng.cache.used_pages() == 0
+    assert res[True][0] == res[False][0]
+    assert res[True][1].metrics["prefix_hit_tokens"] >= 64 and res[False][1].metrics["prefix_hit_tokens"] == 0
+
+
+def test_fork_copies_the_shared_page_on_the_device(model_dirs):
+    """kv.rs:336-349 end to end: a forked request continues from its parent's cache, and the parent's
+    partial page is copied before the child writes into it."""
+    from glassbox_amd import Engine
+    folder = model_dirs.get("B")
+    toks = helpers.random_tokens(384, 41, seed=8)
+    eng = Engine(folder, dtype="float32", max_tokens=512, max_seqs=4)
+    eng.step([("p", toks[:20], [])])
+    eng.fork_request("p", "c")
+    a = eng.step([("c", [7, 8, 9], [0, 1, 2])]).cpu().numpy().copy()
+    b = eng.step([("p", toks[20:], list(range(21)))]).cpu().numpy().copy()
+    assert np.abs(a - helpers.plain_logits(folder, tuple(toks[:20] + [7, 8, 9]))[20:]).max() < 1e-4
+    assert np.abs(b - helpers.plain_logits(folder, tuple(toks))[20:]).max() < 1e-4
+    eng.end_request("p"); eng.end_request("c")
+    eng.cache.check_invariants()
+    assert eng.cache.used_pages() == 0
+
+
+def test_seeded_temperature_generation_repeats(model_dirs):
+    from glassbox_amd import Engine, SamplerConfig, generate
+    eng = Engine(model_dirs.get("B"), dtype="bfloat16", max_tokens=2048, max_seqs=8)
+    prompts = [helpers.random_tokens(384, n, seed=n) for n in (1, 9, 40, 70)]
+    cfgs = [SamplerConfig(temperature=0.8, seed=s) for s in (1, 2, 3, 4)]
+    a = generate(eng, prompts, 24, cfgs, token_budget=16)
+    b = generate(eng, prompts, 24, cfgs, token_budget=16)
+    c = generate(eng, prompts, 24, [SamplerConfig(temperature=0.8, seed=s + 10) for s in (1, 2, 3, 4)], token_budget=16)
+    assert a == b and a != c and all(len(o) == 24 for o in a)
+
+
+def test_the_command_line(model_dirs, tmp_path):
+    import json
+    import os
+    import subprocess
+    import sys
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    cfg = tmp_path / "cfg.json"
+    cfg.write_text(json.dumps(helpers.TINY_A))
+    out = tmp_path / "model"
+    run = lambda *a: subprocess.run([sys.executable, os.path.join(root, "bin", "glassbox"), *a], capture_output=True,
+                                    text=True, timeout=300)
+    r = run("random", "--config", str(cfg), "--out", str(out), "--seed", "5")
+    assert r.returncode == 0, r.stderr
+    r = run("generate", "--model", str(out), "--prompt", "5,17,3", "-n", "8", "--dtype", "float32")
+    assert r.returncode == 0, r.stderr
+    toks = [int(t) for t in r.stdout.split()]
+    c, w = plain.load_folder(str(out))
+    assert toks == plain.greedy(w, c, [5, 17, 3], 8) and "prefill 3 tokens" in r.stderr
