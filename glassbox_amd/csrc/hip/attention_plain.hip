@@ -62,7 +62,7 @@ __global__ __launch_bounds__(kChunk) void attention_plain_kernel(
       for (int j = 0; j < cnt; ++j) {
         const int pj = c0 + j;
         const int page = table[pj / page_size];
-        acc = fmaf(es[j], to_f(v_pages[(((size_t)page * nkv + kvh) * page_size + pj % page_size) * hd + tid]), acc);
+        acc = fmaf(es[j], to_f(v_pages[(((size_t)page * nkv + kvh) * hd + tid) * page_size + pj % page_size]), acc);
       }
     }
     m = m_new;

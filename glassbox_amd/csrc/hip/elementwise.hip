@@ -95,9 +95,11 @@ extern "C" int gb_rope_table(const int32_t* pos, const float* inv, float* cosv, 
 // For token t: every query head and key head is rotated in half-split pairs (i, i + hd/2):
 //   x0' = x0 c - x1 s ; x1' = x1 c + x0 s                              (model.rs:110-113)
 // queries are rotated in place inside the stacked qkv row; rotated keys and plain values go to
-// the pages at slot[t] (model.rs:273-275).  Pages are [page][kv head][slot in page][hd].
+// the pages at slot[t] (model.rs:273-275).  Key pages are [page][kv head][slot in page][hd]; value
+// pages are transposed, [page][kv head][hd][slot in page], so that the attention kernels find
+// consecutive keys of one value dimension side by side (the matrix cores' operand layout).
 // With slots == nullptr nothing is stored (a layer that reads another layer's cache).
-// With n_rot_kv == 0 the row holds queries only.
+// With nkv == 0 the row holds queries only.
 template <typename T>
 __global__ void rope_store_kernel(T* __restrict__ qkv, int row_stride, const float* __restrict__ cosv,
                                   const float* __restrict__ sinv, const int32_t* __restrict__ slots,
@@ -139,7 +141,7 @@ __global__ void rope_store_kernel(T* __restrict__ qkv, int row_stride, const flo
     const T* v = row + (size_t)(nh + nkv) * hd;
     for (int e = threadIdx.x; e < nkv * hd; e += blockDim.x) {
       const int kvh = e / hd, i = e % hd;
-      v_pages[(((size_t)page * nkv + kvh) * page_size + off) * hd + i] = v[e];
+      v_pages[(((size_t)page * nkv + kvh) * hd + i) * page_size + off] = v[e];
     }
   }
 }

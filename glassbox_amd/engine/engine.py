@@ -68,7 +68,8 @@ class Engine:
                 lc.group = keys.index(spec.group_key)
                 shape = (num_pages, spec.num_kv_heads, self.page_size, spec.head_dim)
                 lc.k_pages = torch.zeros(shape, dtype=self.dtype, device=self.device)
-                lc.v_pages = torch.zeros(shape, dtype=self.dtype, device=self.device)
+                lc.v_pages = torch.zeros((num_pages, spec.num_kv_heads, spec.head_dim, self.page_size),
+                                         dtype=self.dtype, device=self.device)   # transposed: see ops._check_pages
             if state is not None:
                 lc.state = torch.zeros((self.max_seqs,) + tuple(state.shape), dtype=state.dtype, device=self.device)
             self.layers.append(lc)

@@ -55,10 +55,14 @@ _SIGS = {
         "gb_attention_plain": [_vp, _i, _vp, _i, _i, _vp, _vp, _vp, _i, _vp, _vp, _i, _i, _i, _i, _i, _f, _i, _vp],
     },
     "attention_bf16": {
-        "gb_attention_decode_bf16": [_vp, _i, _vp, _i, _vp, _vp, _vp, _i, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i,
-                                     _f, _i, _i, _vp],
-        "gb_attention_prefill_bf16": [_vp, _i, _vp, _i, _vp, _vp, _vp, _vp, _i, _vp, _vp, _i, _i, _i, _i, _i, _i, _f,
-                                      _i, _vp],
+        # q, q_stride, out, out_stride, ws_acc, ws_ml, positions, tables, table_stride, k, v,
+        # n_decode, nh, nkv, hd, page, scale, window, chunk, max_context, stream
+        "gb_attention_decode_bf16": [_vp, _i, _vp, _i, _vp, _vp, _vp, _vp, _i, _vp, _vp, _i, _i, _i, _i, _i, _f, _i,
+                                     _i, _i, _vp],
+        # q, q_stride, out, out_stride, q_start, q_len, pos0, seq_base, n_seqs, max_q_len, tables, table_stride,
+        # k, v, nh, nkv, hd, page, scale, window, stream
+        "gb_attention_prefill_bf16": [_vp, _i, _vp, _i, _vp, _vp, _vp, _i, _i, _i, _vp, _i, _vp, _vp, _i, _i, _i, _i,
+                                      _f, _i, _vp],
     },
     "sampling": {
         "gb_argmax": [_vp, _vp, _i, _i, _vp],
@@ -118,6 +122,19 @@ def _i32(t: Optional[torch.Tensor], what: str, n: Optional[int] = None) -> None:
         raise KernelError(f"{what} holds {t.numel()} entries, {n} are needed")
 
 
+def _check_pages(k_pages, v_pages, dtype, what: str) -> None:
+    """Key pages [pages, kv heads, page size, head size]; value pages transposed [pages, kv heads, head size,
+    page size]; both contiguous and of the activations' type."""
+    if k_pages is None or v_pages is None or k_pages.dim() != 4 or v_pages.dim() != 4:
+        raise KernelError(f"{what}: key and value pages must be 4-d tensors")
+    p, h, s, d = k_pages.shape
+    if tuple(v_pages.shape) != (p, h, d, s):
+        raise KernelError(f"{what}: value pages must be [pages, kv heads, head size, page size] = "
+                          f"{(p, h, d, s)}, got {tuple(v_pages.shape)}")
+    if not k_pages.is_contiguous() or not v_pages.is_contiguous() or k_pages.dtype != dtype or v_pages.dtype != dtype:
+        raise KernelError(f"{what}: pages must be contiguous and of the activations' type")
+
+
 # ------------------------------------------------------------------ elementwise
 def embed(table: torch.Tensor, ids: torch.Tensor, out: torch.Tensor) -> None:
     """out[i, :] = table[ids[i], :] as 32-bit floats."""
@@ -171,15 +188,10 @@ def rope_store(qkv: torch.Tensor, cos: Optional[torch.Tensor], sin: Optional[tor
     page_size = 0
     if slots is not None:
         _i32(slots, "slots", n)
-        want = (n_kv_heads, head_dim)
-        for pg in (k_pages, v_pages):
-            if pg is None or pg.dim() != 4 or (pg.shape[1], pg.shape[3]) != want or not pg.is_contiguous() \
-                    or pg.dtype != qkv.dtype:
-                raise KernelError("rope_store: pages must be contiguous [pages, kv heads, page size, head size] "
-                                  "of the activations' type")
+        _check_pages(k_pages, v_pages, qkv.dtype, "rope_store")
+        if (k_pages.shape[1], k_pages.shape[3]) != (n_kv_heads, head_dim):
+            raise KernelError("rope_store: pages do not have this layer's kv heads and head size")
         page_size = k_pages.shape[2]
-        if v_pages.shape != k_pages.shape:
-            raise KernelError("rope_store: key and value pages differ in shape")
     if rotate:
         if cos is None or sin is None or cos.shape != (n, head_dim // 2) and cos.shape[0] < n:
             raise KernelError("rope_store: rotation needs cos/sin tables of [n, head_dim/2]")
@@ -251,10 +263,9 @@ def attention_plain(q: torch.Tensor, out: torch.Tensor, positions: torch.Tensor,
     _, nkv, page_size, hd = k_pages.shape
     if q.shape[1] != n_heads * hd or out.shape != (n, n_heads * hd):
         raise KernelError("attention: q and out must be [n, heads * head size]")
-    if not (q.dtype == out.dtype == k_pages.dtype == v_pages.dtype):
-        raise KernelError("attention: q, out and pages must share one element type")
-    if not k_pages.is_contiguous() or not v_pages.is_contiguous() or k_pages.shape != v_pages.shape:
-        raise KernelError("attention: pages must be contiguous and alike")
+    if q.dtype != out.dtype:
+        raise KernelError("attention: q and out must share one element type")
+    _check_pages(k_pages, v_pages, q.dtype, "attention")
     _i32(positions, "positions", n)
     _i32(tok_seq, "tok_seq", n)
     if tables.dtype != torch.int32 or tables.dim() != 2 or tables.stride(1) != 1:
@@ -266,8 +277,58 @@ def attention_plain(q: torch.Tensor, out: torch.Tensor, positions: torch.Tensor,
 
 
 def tuned_attention_supports(k_pages: torch.Tensor, n_heads: int, window: int) -> bool:
-    """Whether the tuned bfloat16 attention kernels take this layer's sizes."""
-    return False
+    """Whether the matrix-core attention kernels take this layer: bfloat16 pages, a head size that is
+    a multiple of 16 up to 128, at most 16 query heads per kv head, pages of a multiple of 16."""
+    _, nkv, page, hd = k_pages.shape
+    return (k_pages.dtype == torch.bfloat16 and hd % 16 == 0 and 16 <= hd <= 128 and n_heads % nkv == 0
+            and n_heads // nkv <= 16 and page % 16 == 0)
+
+
+def decode_chunk(n_decode: int, n_kv_heads: int, max_context: int) -> int:
+    """Keys per workgroup of the decode kernel: a multiple of 256, small enough that the launch has
+    about a thousand workgroups, large enough that a workgroup's fixed costs are spread."""
+    want_splits = max(1, 1024 // max(1, n_decode * n_kv_heads))
+    chunk = -(-max_context // want_splits)
+    return max(256, -(-chunk // 256) * 256)
+
+
+def attention_decode(q: torch.Tensor, out: torch.Tensor, ctx, cache, n_heads: int, scale: float, window: int) -> None:
+    """Rows 0..n_decode-1 of the step (requests with a single token), split over their context."""
+    n_dec = ctx.host["n_decode"]
+    k_pages, v_pages = cache.k_pages, cache.v_pages
+    _dev(q, out, k_pages, v_pages)
+    _check_pages(k_pages, v_pages, torch.bfloat16, "attention_decode")
+    _, nkv, page, hd = k_pages.shape
+    if q.dtype != torch.bfloat16 or out.dtype != torch.bfloat16 or q.shape[1] != n_heads * hd:
+        raise KernelError("attention_decode: q and out must be bfloat16 [n, heads * head size]")
+    tables = ctx.tables[cache.group]
+    max_context = int(ctx.host["max_context"])
+    chunk = decode_chunk(n_dec, nkv, max_context)
+    splits = -(-max_context // chunk)
+    ws_acc = ctx.buffer("attn_ws_acc", (n_dec * n_heads * splits * hd,), torch.float32)
+    ws_ml = ctx.buffer("attn_ws_ml", (n_dec * n_heads * splits * 2,), torch.float32)
+    lib = _lib("attention_bf16")
+    _check(lib, lib.gb_attention_decode_bf16(_p(q), _rows(q, "q"), _p(out), _rows(out, "out"), _p(ws_acc), _p(ws_ml),
+                                             _p(ctx.positions), _p(tables), tables.stride(0), _p(k_pages), _p(v_pages),
+                                             n_dec, n_heads, nkv, hd, page, float(scale), int(window), chunk,
+                                             max_context, _stream()))
+
+
+def attention_prefill(q: torch.Tensor, out: torch.Tensor, ctx, cache, n_heads: int, scale: float, window: int) -> None:
+    """The requests of the step that bring more than one token (they follow the single-token ones)."""
+    n_dec, S = ctx.host["n_decode"], ctx.num_seqs
+    k_pages, v_pages = cache.k_pages, cache.v_pages
+    _dev(q, out, k_pages, v_pages)
+    _check_pages(k_pages, v_pages, torch.bfloat16, "attention_prefill")
+    _, nkv, page, hd = k_pages.shape
+    if q.dtype != torch.bfloat16 or out.dtype != torch.bfloat16 or q.shape[1] != n_heads * hd:
+        raise KernelError("attention_prefill: q and out must be bfloat16 [n, heads * head size]")
+    tables = ctx.tables[cache.group]
+    lib = _lib("attention_bf16")
+    _check(lib, lib.gb_attention_prefill_bf16(_p(q), _rows(q, "q"), _p(out), _rows(out, "out"), _p(ctx.q_start),
+                                              _p(ctx.q_len), _p(ctx.pos0), n_dec, S - n_dec, int(ctx.host["max_q_len"]),
+                                              _p(tables), tables.stride(0), _p(k_pages), _p(v_pages), n_heads, nkv, hd,
+                                              page, float(scale), int(window), _stream()))
 
 
 # ------------------------------------------------------------------------ sampling

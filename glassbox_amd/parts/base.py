@@ -64,7 +64,7 @@ class StateSpec:
 class LayerCache:
     """What the engine hands a mixer: its layer's pages, the index of their page group, its state."""
     k_pages: Optional[torch.Tensor] = None   # [pages, kv heads, page size, head size]
-    v_pages: Optional[torch.Tensor] = None
+    v_pages: Optional[torch.Tensor] = None   # [pages, kv heads, head size, page size] (transposed)
     group: int = 0
     state: Optional[torch.Tensor] = None     # [slots, *state shape]
     writable: bool = True                    # False: the layer reads another layer's cache

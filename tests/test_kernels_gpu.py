@@ -134,7 +134,7 @@ def test_rope_table_and_rotation(hd, theta):
     qkv = rnd(n, (nh + 2 * nkv) * hd, seed=3)
     page = 16
     k_pages = torch.zeros(4, nkv, page, hd, device=DEV)
-    v_pages = torch.zeros_like(k_pages)
+    v_pages = torch.zeros(4, nkv, hd, page, device=DEV)
     slots = torch.tensor([3, 16 + 15, 32, 0, 63], dtype=torch.int32, device=DEV)
     buf = to_dev(qkv.clone())
     ops.rope_store(buf, cos, sin, slots, k_pages, v_pages, nh, nkv, hd)
@@ -145,7 +145,7 @@ def test_rope_table_and_rotation(hd, theta):
     assert torch.equal(got_q[0], qkv[0, :nh * hd].double().reshape(nh, hd)), "position 0 must leave the vector as it is"
     for i, s in enumerate(slots.tolist()):
         got_k = k_pages[s // page, :, s % page, :].cpu().double()
-        got_v = v_pages[s // page, :, s % page, :].cpu()
+        got_v = v_pages[s // page, :, :, s % page].cpu()
         assert (got_k - k_want[i]).abs().max().item() < 1e-5
         assert torch.equal(got_v, qkv[i, (nh + nkv) * hd:].reshape(nkv, hd))
 
@@ -157,7 +157,7 @@ def paged_setup(ctx_lens, nkv, hd, page, seed, dtype, scatter=True):
     total_pages = sum(-(-c // page) for c in ctx_lens) + 3
     perm = torch.randperm(total_pages, generator=g).tolist() if scatter else list(range(total_pages))
     k_pages = torch.randn(total_pages, nkv, page, hd, generator=g).to(dtype)   # unowned slots hold junk
-    v_pages = torch.randn(total_pages, nkv, page, hd, generator=g).to(dtype)
+    v_pages = torch.randn(total_pages, nkv, hd, page, generator=g).to(dtype)   # values are kept transposed
     tables, ks, vs = [], [], []
     for c in ctx_lens:
         np_ = -(-c // page)
@@ -167,7 +167,7 @@ def paged_setup(ctx_lens, nkv, hd, page, seed, dtype, scatter=True):
         v = torch.randn(c, nkv, hd, generator=g).to(dtype)
         for p in range(c):
             k_pages[t[p // page], :, p % page, :] = k[p]
-            v_pages[t[p // page], :, p % page, :] = v[p]
+            v_pages[t[p // page], :, :, p % page] = v[p]
         ks.append(k)
         vs.append(v)
     maxp = max(len(t) for t in tables)
@@ -239,6 +239,108 @@ def test_attention_finds_one_far_key(dtype):
                             to_dev(v_pages), nh, 1 / math.sqrt(hd), 0)
         want = vs[0][target].float().repeat_interleave(2, 0).reshape(-1)
         assert (out.cpu().float()[0] - want).abs().max().item() < 2e-2, f"key at {target} was not found"
+
+
+class BareContext:
+    """What the tuned attention bindings read from a step's context, for a hand-made batch: single-token
+    requests first, then portions."""
+
+    def __init__(self, q_lens, ctx_lens, tables, max_context=None):
+        from types import SimpleNamespace
+        self.num_seqs = len(q_lens)
+        n_dec = sum(1 for l in q_lens if l == 1)
+        assert all(l == 1 for l in q_lens[:n_dec]) and all(l > 1 for l in q_lens[n_dec:])
+        q_start = np.concatenate([[0], np.cumsum(q_lens)[:-1]]).tolist()
+        pos0 = [c - l for c, l in zip(ctx_lens, q_lens)]
+        self.tok_seq = [s for s, l in enumerate(q_lens) for _ in range(l)]
+        self.pos_list = [pos0[s] + j for s, l in enumerate(q_lens) for j in range(l)]
+        i32 = lambda v: torch.tensor(v, dtype=torch.int32, device=DEV)
+        self.positions, self.q_start, self.q_len, self.pos0 = i32(self.pos_list), i32(q_start), i32(q_lens), i32(pos0)
+        self.tables = [to_dev(tables)]
+        self.host = {"n_decode": n_dec, "max_q_len": max(q_lens), "max_context": max_context or max(ctx_lens)}
+        self._bufs = {}
+
+    def buffer(self, name, shape, dtype):
+        return self._bufs.setdefault((name, tuple(shape)), torch.empty(shape, dtype=dtype, device=DEV))
+
+
+@pytest.mark.parametrize("nh,nkv,hd,window", [(4, 2, 16, 0), (3, 1, 32, 0), (6, 2, 48, 0), (8, 8, 64, 0), (8, 2, 128, 0),
+                                              (16, 1, 64, 0), (5, 5, 80, 0), (4, 2, 64, 37), (4, 4, 64, 300), (2, 1, 112, 0)])
+@pytest.mark.parametrize("page", [16, 64])
+def test_tuned_attention_against_the_plain_kernel(nh, nkv, hd, window, page):
+    """The matrix-core kernels for decoding and for prompt portions against their plain twin and the
+    float64 formula: contexts that end at every offset of a page, chunks that split, windows."""
+    from types import SimpleNamespace
+    from glassbox_amd import ops
+    q_lens = [1, 1, 1, 1, 1, 5, 70, 16, 130]
+    ctx_lens = [1, 17, 256, 700, 1025, 5, 300, 16, 530]      # portions 5/5, 70 ending at 300, 16/16, 130 ending at 530
+    k_pages, v_pages, tables, ks, vs = paged_setup(ctx_lens, nkv, hd, page, seed=hd + nh, dtype=torch.bfloat16)
+    ctx = BareContext(q_lens, ctx_lens, tables, max_context=1100)
+    n = sum(q_lens)
+    q = (rnd(n, nh * hd, seed=11) * 0.7).bfloat16()
+    scale = 1 / math.sqrt(hd)
+    cache = SimpleNamespace(k_pages=to_dev(k_pages), v_pages=to_dev(v_pages), group=0)
+    assert ops.tuned_attention_supports(cache.k_pages, nh, window)
+    out = torch.zeros(n, nh * hd, device=DEV, dtype=torch.bfloat16)
+    qd = to_dev(q)
+    ops.attention_decode(qd, out, ctx, cache, nh, scale, window)
+    ops.attention_prefill(qd, out, ctx, cache, nh, scale, window)
+    twin = torch.zeros_like(out)
+    ops.attention_plain(qd, twin, ctx.positions, torch.tensor(ctx.tok_seq, dtype=torch.int32, device=DEV), ctx.tables[0],
+                        cache.k_pages, cache.v_pages, nh, scale, window)
+    want = plain_attention_rows(q, ks, vs, ctx.tok_seq, ctx.pos_list, nh, scale, window)
+    err = (out.cpu().double() - want).abs().max(dim=1).values
+    bad = torch.nonzero(err > 2 ** -6).flatten().tolist()
+    assert not bad, f"rows {bad[:8]} (request, position) {[(ctx.tok_seq[i], ctx.pos_list[i]) for i in bad[:8]]}: {err[bad[:8]]}"
+    # both are roundings to bfloat16 of nearly equal 32-bit results: at most a unit or two in the last place apart
+    assert ((out.float() - twin.float()).abs() <= 2 ** -7 * (1 + twin.float().abs())).all()
+
+
+def test_tuned_decode_finds_one_far_key_in_every_chunk_position():
+    """One key is made to stand out: first and last slot of a page, chunk edges, the last position."""
+    from types import SimpleNamespace
+    from glassbox_amd import ops
+    nh, nkv, hd, page, ctxlen = 4, 2, 64, 16, 1500
+    k_pages, v_pages, tables, ks, vs = paged_setup([ctxlen], nkv, hd, page, seed=1, dtype=torch.bfloat16)
+    q = rnd(1, nh * hd, seed=2).float().reshape(nh, hd)
+    q[1::2] = q[0::2]
+    q = q.reshape(1, nh * hd).bfloat16()
+    for target in (0, 15, 16, 63, 64, 255, 256, 257, 511, 512, 1023, 1024, 1279, 1280, 1498, 1499):
+        kp = k_pages.clone()
+        for kvh in range(nkv):
+            kp[tables[0, target // page], kvh, target % page, :] = (q[0].float().reshape(nh, hd)[2 * kvh] * 40).bfloat16()
+        for max_context in (1500, 4096):                       # one and several chunks per workgroup
+            ctx = BareContext([1], [ctxlen], tables, max_context=max_context)
+            out = torch.zeros(1, nh * hd, device=DEV, dtype=torch.bfloat16)
+            cache = SimpleNamespace(k_pages=to_dev(kp), v_pages=to_dev(v_pages), group=0)
+            ops.attention_decode(to_dev(q), out, ctx, cache, nh, 1 / math.sqrt(hd), 0)
+            want = vs[0][target].float().repeat_interleave(2, 0).reshape(-1)
+            assert (out.cpu().float()[0] - want).abs().max().item() < 2e-2, f"key at {target} was not found"
+
+
+def test_tuned_prefill_sees_exactly_the_causal_keys():
+    """A portion in the middle of a request: token t must find a marked key at its own position and
+    must not see the one after it."""
+    from types import SimpleNamespace
+    from glassbox_amd import ops
+    nh, nkv, hd, page = 2, 2, 64, 16
+    ctxlen, qlen = 200, 90                                     # the portion covers positions 110..199
+    k_pages, v_pages, tables, ks, vs = paged_setup([ctxlen], nkv, hd, page, seed=3, dtype=torch.bfloat16)
+    ctx = BareContext([qlen], [ctxlen], tables)
+    g = torch.Generator().manual_seed(5)
+    direction = torch.randn(hd, generator=g)
+    direction /= direction.norm()
+    # every key points along `direction` with a length that grows with its position: the newest visible key wins
+    kp = k_pages.clone()
+    for p in range(ctxlen):
+        kp[tables[0, p // page], :, p % page, :] = (direction * (1 + p)).bfloat16()
+    q = (direction * 120).repeat(qlen, nh).bfloat16()
+    out = torch.zeros(qlen, nh * hd, device=DEV, dtype=torch.bfloat16)
+    cache = SimpleNamespace(k_pages=to_dev(kp), v_pages=to_dev(v_pages), group=0)
+    ops.attention_prefill(to_dev(q), out, ctx, cache, nh, 1 / math.sqrt(hd), 0)
+    for t in range(qlen):
+        want = vs[0][110 + t].float().reshape(-1)             # not the value of position 111 + t
+        assert (out.cpu().float()[t] - want).abs().max().item() < 3e-2, f"token {t} of the portion"
 
 
 def test_copy_rows():

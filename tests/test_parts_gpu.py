@@ -89,7 +89,7 @@ def test_attention_part_with_rotary(model_dirs, window):
     lengths = [19, 7]
     ctx, _ = context_for(eng, lengths)
     pages = 512 // 16
-    cache = LayerCache(torch.zeros(pages, nkv, 16, hd, device=DEV), torch.zeros(pages, nkv, 16, hd, device=DEV), 0)
+    cache = LayerCache(torch.zeros(pages, nkv, 16, hd, device=DEV), torch.zeros(pages, nkv, hd, 16, device=DEV), 0)
     h = rnd(sum(lengths), d, seed=5).float()
     x = torch.zeros(sum(lengths), d, device=DEV)
     part.forward(ctx, h.to(DEV), x, cache)
