@@ -31,6 +31,8 @@ def main() -> int:
     ap.add_argument("--layers", type=int, default=MODEL["num_hidden_layers"])
     ap.add_argument("--dtype", default="bfloat16", choices=["bfloat16", "float32"])
     ap.add_argument("--no-points", action="store_true", help="skip the batch 1 and 64 points")
+    ap.add_argument("--only", choices=["decode", "prefill"], default=None,
+                    help="for profiling: run only the decode steps (after their prefill) or only the 2,048-token prefill")
     ap.add_argument("--no-graph", action="store_true", help="run decode steps without HIP graph replay")
     a = ap.parse_args()
     if a.gpus != 1:
@@ -68,8 +70,14 @@ def main() -> int:
         dt = time.perf_counter() - t0
         eng.end_request(name)
         return dt
-    prefill_once("warm")
-    pf = min(prefill_once(f"pf{i}") for i in range(3))
+    if a.only == "decode":
+        pf = float("nan")
+    else:
+        prefill_once("warm")
+        pf = min(prefill_once(f"pf{i}") for i in range(3))
+    if a.only == "prefill":
+        print(json.dumps({"prefill_ms": round(pf * 1e3, 3), "tokens": PREFILL_TOKENS}))
+        return 0
     T = PREFILL_TOKENS
     pf_flops = 2 * T * layer_params * L + L * 4 * qd * (T * (T + 1) // 2) + 2 * d * vocab
     peak = PEAK["bf16_tflops"] if a.dtype == "bfloat16" else PEAK["fp32_tflops"]

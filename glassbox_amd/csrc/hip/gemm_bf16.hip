@@ -114,87 +114,231 @@ __global__ __launch_bounds__(256) void gemm_tiled_kernel(const bf16* __restrict_
 }
 
 // ------------------------------------------------------------------------ skinny
-// MT = number of 16-wide column blocks of A's rows (M <= 16*MT).
-template <int MT, typename CT>
-__global__ __launch_bounds__(256) void gemm_skinny_kernel(const bf16* __restrict__ a, int lda, const bf16* __restrict__ w,
-                                                          int ldw, CT* __restrict__ c, int ldc, int M, int N, int K,
-                                                          int accumulate) {
-  __shared__ float part[4][MT][64][4];
+// grid (row tiles of W).  A workgroup of WAVES waves owns 16 rows of W and walks all of k in slices
+// of ITERS*WAVES*64: wave w takes the 64-wide k blocks w, w+WAVES, ... of a slice; inside a block
+// lane group q holds k = 16q..16q+15 as two operands of 8 (the same split for W and for A, so the
+// products pair up).  All loads of a slice are issued before its first MFMA.  The waves combine
+// through LDS in wave order.  Few rows of W (a small N) are given many waves each, so that the
+// launch still keeps enough loads in flight to use the memory system; no partial result ever
+// leaves the workgroup, so no pass over memory is needed to combine them.
+//
+// EPI_STORE / EPI_ACCUMULATE: C[m, n] = or += the product.  EPI_SILU_MUL: W holds gate rows
+// [0, N/2) and up rows [N/2, N); a tile takes 8 gate rows and the 8 up rows that belong to them
+// and writes act[m, j] = gate / (1 + exp(-gate)) * up (crates/glassbox-core/src/model.rs:336-340)
+// to C[M, N/2].
+enum : int { EPI_STORE = 0, EPI_ACCUMULATE = 1, EPI_SILU_MUL = 2 };
+
+template <int MT, int WAVES, int ITERS, int RT, int EPI, typename CT>
+__global__ __launch_bounds__(WAVES * 64) void gemm_skinny_kernel(const bf16* __restrict__ a, int lda,
+                                                                 const bf16* __restrict__ w, int ldw, CT* __restrict__ c,
+                                                                 int ldc, int M, int N, int K) {
+  __shared__ float part[WAVES][RT][MT][64][4];
   const int tid = threadIdx.x, lane = tid % 64, wave = tid / 64;
   const int r = lane % 16, q = lane / 16;
-  const int n0 = blockIdx.x * 16;
-  const int row = n0 + r;
-  const bool row_ok = row < N;
-  const bf16* wrow = w + (size_t)(row_ok ? row : 0) * ldw;
+  const bf16* wrow[RT];
+  bool row_ok[RT];
+#pragma unroll
+  for (int rt = 0; rt < RT; ++rt) {
+    const int tile = blockIdx.x * RT + rt;
+    int row;
+    if (EPI == EPI_SILU_MUL) row = r < 8 ? tile * 8 + r : N / 2 + tile * 8 + (r - 8);
+    else row = tile * 16 + r;
+    row_ok[rt] = EPI == EPI_SILU_MUL ? (tile * 8 + (r & 7) < N / 2) : row < N;
+    wrow[rt] = w + (size_t)(row_ok[rt] ? row : 0) * ldw;
+  }
 
-  f32x4 acc[MT];
+  f32x4 acc[RT][MT];
 #pragma unroll
-  for (int t = 0; t < MT; ++t)
+  for (int rt = 0; rt < RT; ++rt)
 #pragma unroll
-    for (int e = 0; e < 4; ++e) acc[t][e] = 0.f;
+    for (int t = 0; t < MT; ++t)
+#pragma unroll
+      for (int e = 0; e < 4; ++e) acc[rt][t][e] = 0.f;
 
-  // wave `wave` takes the 64-wide k blocks wave, wave+4, ...; inside a block lane group q holds
-  // k = 16q .. 16q+15 as two operands of 8 (the same split for W and for A, so the products pair up)
-#pragma unroll 4
-  for (int kb = wave * 64; kb < K; kb += 256) {
-    const int k = kb + q * 16;
-    bf16x8 w0 = (row_ok && k < K) ? load8(wrow + k) : zero8();
-    bf16x8 w1 = (row_ok && k + 8 < K) ? load8(wrow + k + 8) : zero8();
+  // a 64-wide k block is two MFMA steps of 32: lane group q holds k = 8q..8q+7 of each
+  for (int kbeg = 0; kbeg < K; kbeg += ITERS * WAVES * 64) {
+    bf16x8 wf[RT][ITERS][2];
 #pragma unroll
-    for (int t = 0; t < MT; ++t) {
-      const int m = t * 16 + r;
-      const bf16* arow = a + (size_t)(m < M ? m : 0) * lda;
-      bf16x8 x0 = (m < M && k < K) ? load8(arow + k) : zero8();
-      bf16x8 x1 = (m < M && k + 8 < K) ? load8(arow + k + 8) : zero8();
-      acc[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(w0, x0, acc[t], 0, 0, 0);
-      acc[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(w1, x1, acc[t], 0, 0, 0);
+    for (int rt = 0; rt < RT; ++rt)
+#pragma unroll
+      for (int it = 0; it < ITERS; ++it) {
+        const int k = kbeg + (wave + WAVES * it) * 64 + q * 8;
+        wf[rt][it][0] = (row_ok[rt] && k < K) ? load8(wrow[rt] + k) : zero8();
+        wf[rt][it][1] = (row_ok[rt] && k + 32 < K) ? load8(wrow[rt] + k + 32) : zero8();
+      }
+    if (MT == 1) {
+      const bf16* arow = a + (size_t)(r < M ? r : 0) * lda;
+      bf16x8 xf[ITERS][2];
+#pragma unroll
+      for (int it = 0; it < ITERS; ++it) {
+        const int k = kbeg + (wave + WAVES * it) * 64 + q * 8;
+        xf[it][0] = (r < M && k < K) ? load8(arow + k) : zero8();
+        xf[it][1] = (r < M && k + 32 < K) ? load8(arow + k + 32) : zero8();
+      }
+#pragma unroll
+      for (int it = 0; it < ITERS; ++it)
+#pragma unroll
+        for (int rt = 0; rt < RT; ++rt) {
+          acc[rt][0] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wf[rt][it][0], xf[it][0], acc[rt][0], 0, 0, 0);
+          acc[rt][0] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wf[rt][it][1], xf[it][1], acc[rt][0], 0, 0, 0);
+        }
+    } else {
+#pragma unroll
+      for (int it = 0; it < ITERS; ++it) {
+        const int k = kbeg + (wave + WAVES * it) * 64 + q * 8;
+#pragma unroll
+        for (int t = 0; t < MT; ++t) {
+          const int m = t * 16 + r;
+          const bf16* arow = a + (size_t)(m < M ? m : 0) * lda;
+          const bf16x8 x0 = (m < M && k < K) ? load8(arow + k) : zero8();
+          const bf16x8 x1 = (m < M && k + 32 < K) ? load8(arow + k + 32) : zero8();
+#pragma unroll
+          for (int rt = 0; rt < RT; ++rt) {
+            acc[rt][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wf[rt][it][0], x0, acc[rt][t], 0, 0, 0);
+            acc[rt][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wf[rt][it][1], x1, acc[rt][t], 0, 0, 0);
+          }
+        }
+      }
     }
   }
 #pragma unroll
-  for (int t = 0; t < MT; ++t)
+  for (int rt = 0; rt < RT; ++rt)
 #pragma unroll
-    for (int e = 0; e < 4; ++e) part[wave][t][lane][e] = acc[t][e];
+    for (int t = 0; t < MT; ++t)
+#pragma unroll
+      for (int e = 0; e < 4; ++e) part[wave][rt][t][lane][e] = acc[rt][t][e];
   __syncthreads();
-  // D[n, m]: lane holds column m = lane%16 and rows n = 4*(lane/16) + e.  256 threads share the
-  // MT*64*4 cells; the four waves' partial sums are added in wave order.
-  for (int cell = tid; cell < MT * 64 * 4; cell += 256) {
-    const int t = cell / 256, l = (cell / 4) % 64, e = cell % 4;
-    const float v = ((part[0][t][l][e] + part[1][t][l][e]) + part[2][t][l][e]) + part[3][t][l][e];
-    const int m = t * 16 + l % 16, n = n0 + 4 * (l / 16) + e;
-    if (m < M && n < N) store_c<CT>(c + (size_t)m * ldc + n, v, accumulate);
+  if (tid >= 256) return;
+
+  // D[n, m]: lane l holds column m = l%16 and rows n = 4*(l/16) + e.  The first 256 threads own the
+  // cells of the tiles: thread tid owns cell (l = tid/4, e = tid%4) of every row tile and column block.
+  const int l = tid / 4, e = tid % 4;
+  float v[RT][MT];
+#pragma unroll
+  for (int rt = 0; rt < RT; ++rt)
+#pragma unroll
+    for (int t = 0; t < MT; ++t) {
+      float s = part[0][rt][t][l][e];
+#pragma unroll
+      for (int wv = 1; wv < WAVES; ++wv) s += part[wv][rt][t][l][e];
+      v[rt][t] = s;
+    }
+  const int nrow = 4 * (l / 16) + e;  // row of the tile, 0..15
+  if (EPI == EPI_SILU_MUL) {
+    // rows 0..7 are gate, 8..15 the matching up rows: the up values travel through LDS.  Only the
+    // first four waves are here; the slice of the last wave is free once every sum above is done.
+    float* up = &part[WAVES - 1][0][0][0][0];
+    __syncthreads();
+#pragma unroll
+    for (int rt = 0; rt < RT; ++rt)
+#pragma unroll
+      for (int t = 0; t < MT; ++t) up[(rt * MT + t) * 256 + tid] = v[rt][t];
+    __syncthreads();
+    if (nrow < 8) {
+#pragma unroll
+      for (int rt = 0; rt < RT; ++rt) {
+        const int j = (blockIdx.x * RT + rt) * 8 + nrow;
+#pragma unroll
+        for (int t = 0; t < MT; ++t) {
+          const int m = t * 16 + l % 16;
+          const float g = v[rt][t], u = up[(rt * MT + t) * 256 + tid + 128];
+          if (m < M && j < N / 2) c[(size_t)m * ldc + j] = (CT)(g / (1.0f + __expf(-g)) * u);
+        }
+      }
+    }
+  } else {
+#pragma unroll
+    for (int rt = 0; rt < RT; ++rt) {
+      const int n = (blockIdx.x * RT + rt) * 16 + nrow;
+#pragma unroll
+      for (int t = 0; t < MT; ++t) {
+        const int m = t * 16 + l % 16;
+        if (m < M && n < N) store_c<CT>(c + (size_t)m * ldc + n, v[rt][t], EPI == EPI_ACCUMULATE);
+      }
+    }
   }
 }
 
-template <typename CT>
-int launch(const bf16* a, int lda, const bf16* w, int ldw, CT* c, int ldc, int M, int N, int K, int accumulate,
-           hipStream_t stream) {
-  if (M <= 64) {
-    const dim3 grid((N + 15) / 16), block(256);
-    const int mt = (M + 15) / 16;
-    if (mt == 1) hipLaunchKernelGGL((gemm_skinny_kernel<1, CT>), grid, block, 0, stream, a, lda, w, ldw, c, ldc, M, N, K, accumulate);
-    else if (mt == 2) hipLaunchKernelGGL((gemm_skinny_kernel<2, CT>), grid, block, 0, stream, a, lda, w, ldw, c, ldc, M, N, K, accumulate);
-    else if (mt == 3) hipLaunchKernelGGL((gemm_skinny_kernel<3, CT>), grid, block, 0, stream, a, lda, w, ldw, c, ldc, M, N, K, accumulate);
-    else hipLaunchKernelGGL((gemm_skinny_kernel<4, CT>), grid, block, 0, stream, a, lda, w, ldw, c, ldc, M, N, K, accumulate);
-  } else {
-    const dim3 grid((N + TBN - 1) / TBN, (M + TBM - 1) / TBM), block(256);
-    if (grid.y > 65535) return fail("gemm_bf16: M=%d needs more than 65535 row tiles", M);
-    hipLaunchKernelGGL(gemm_tiled_kernel<CT>, grid, block, 0, stream, a, lda, w, ldw, c, ldc, M, N, K, accumulate);
+// Waves per workgroup, loads in flight per wave and row tiles per workgroup.
+// GB_SKINNY="waves,iters,rowtiles" overrides (for measurements).
+inline void skinny_plan(int tiles, int K, int mt, int* waves, int* iters, int* rt) {
+  // measured on SmolLM2-1.7B and Llama-3-8B shapes: sixteen waves a workgroup keep the most loads in
+  // flight; two row tiles a workgroup halve the re-reading of A once there are tiles enough
+  const int blocks = (K + 63) / 64;               // 64-wide k blocks
+  *waves = blocks >= 16 ? 16 : 4;
+  *rt = tiles >= 256 ? 2 : 1;
+  const int per_wave = (blocks + *waves - 1) / *waves;
+  *iters = (mt == 1 && per_wave >= 2) ? 2 : 1;
+  if (const char* env = getenv("GB_SKINNY")) {
+    int wv = 0, it = 0, r = 0;
+    if (sscanf(env, "%d,%d,%d", &wv, &it, &r) == 3 && (wv == 4 || wv == 16) && (it == 1 || it == 2 || it == 4 || it == 8) &&
+        (r == 1 || r == 2) && !(r == 2 && it == 8)) {
+      *waves = wv;
+      *iters = it;
+      *rt = r;
+    }
   }
-  return launched("gemm_bf16");
+}
+
+template <int MT, int EPI, typename CT>
+int launch_skinny_mt(int tiles, const bf16* a, int lda, const bf16* w, int ldw, CT* c, int ldc, int M, int N, int K,
+                     hipStream_t stream) {
+  int waves, iters, rt;
+  skinny_plan(tiles, K, MT, &waves, &iters, &rt);
+#define GB_CFG(WV, IT, RT)                                                                                                \
+  if (waves == WV && iters == IT && rt == RT)                                                                             \
+    hipLaunchKernelGGL((gemm_skinny_kernel<MT, WV, IT, RT, EPI, CT>), dim3((tiles + RT - 1) / RT), dim3(WV * 64), 0, stream, \
+                       a, lda, w, ldw, c, ldc, M, N, K);
+  GB_CFG(4, 1, 1) GB_CFG(4, 2, 1) GB_CFG(4, 4, 1) GB_CFG(4, 8, 1) GB_CFG(16, 1, 1) GB_CFG(16, 2, 1) GB_CFG(16, 4, 1)
+  GB_CFG(16, 8, 1) GB_CFG(4, 1, 2) GB_CFG(4, 2, 2) GB_CFG(4, 4, 2) GB_CFG(16, 1, 2) GB_CFG(16, 2, 2) GB_CFG(16, 4, 2)
+#undef GB_CFG
+  return launched("gemm_bf16 (skinny)");
+}
+
+template <int EPI, typename CT>
+int launch_skinny(const bf16* a, int lda, const bf16* w, int ldw, CT* c, int ldc, int M, int N, int K, hipStream_t stream) {
+  const int tiles = EPI == EPI_SILU_MUL ? (N / 2 + 7) / 8 : (N + 15) / 16;
+  const int mt = (M + 15) / 16;
+  if (mt == 1) return launch_skinny_mt<1, EPI, CT>(tiles, a, lda, w, ldw, c, ldc, M, N, K, stream);
+  if (mt == 2) return launch_skinny_mt<2, EPI, CT>(tiles, a, lda, w, ldw, c, ldc, M, N, K, stream);
+  if (mt == 3) return launch_skinny_mt<3, EPI, CT>(tiles, a, lda, w, ldw, c, ldc, M, N, K, stream);
+  return launch_skinny_mt<4, EPI, CT>(tiles, a, lda, w, ldw, c, ldc, M, N, K, stream);
 }
 
 }  // namespace
 
+// epilogue: 0 store, 1 accumulate (float32 C), 2 SiLU-multiply of stacked gate/up rows (C is [M, N/2]).
 extern "C" int gb_gemm_bf16(const void* a, int lda, const void* w, int ldw, void* c, int ldc, int c_dtype, int M, int N,
-                            int K, int accumulate, hipStream_t stream) {
+                            int K, int epilogue, hipStream_t stream) {
   GB_REQUIRE(M >= 0 && N > 0 && K > 0, "gemm_bf16: bad sizes M=%d N=%d K=%d", M, N, K);
   GB_REQUIRE(K % 8 == 0, "gemm_bf16: the inner size K=%d must be a multiple of 8 (16-byte operand loads)", K);
   GB_REQUIRE(lda % 8 == 0 && ldw % 8 == 0, "gemm_bf16: row strides (%d, %d) must be multiples of 8 elements", lda, ldw);
-  GB_REQUIRE(lda >= K && ldw >= K && ldc >= N, "gemm_bf16: a leading dimension is shorter than its row");
+  GB_REQUIRE(epilogue >= 0 && epilogue <= 2, "gemm_bf16: unknown epilogue %d", epilogue);
+  const int ncols = epilogue == EPI_SILU_MUL ? N / 2 : N;
+  GB_REQUIRE(epilogue != EPI_SILU_MUL || N % 2 == 0, "gemm_bf16: stacked gate/up rows need an even N, got %d", N);
+  GB_REQUIRE(lda >= K && ldw >= K && ldc >= ncols, "gemm_bf16: a leading dimension is shorter than its row");
   GB_REQUIRE(((uintptr_t)a % 16 == 0) && ((uintptr_t)w % 16 == 0), "gemm_bf16: operands must be 16-byte aligned");
-  GB_REQUIRE(!accumulate || c_dtype == kF32, "gemm_bf16: accumulation is into a float32 result");
+  GB_REQUIRE(epilogue != EPI_ACCUMULATE || c_dtype == kF32, "gemm_bf16: accumulation is into a float32 result");
+  GB_REQUIRE(epilogue != EPI_SILU_MUL || M <= 64, "gemm_bf16: the fused SiLU-multiply serves up to 64 rows, got %d", M);
+  GB_REQUIRE(c_dtype == kF32 || c_dtype == kBF16, "gemm_bf16: unknown result dtype %d", c_dtype);
   if (M == 0) return 0;
-  if (c_dtype == kF32) return launch<float>((const bf16*)a, lda, (const bf16*)w, ldw, (float*)c, ldc, M, N, K, accumulate, stream);
-  if (c_dtype == kBF16) return launch<bf16>((const bf16*)a, lda, (const bf16*)w, ldw, (bf16*)c, ldc, M, N, K, accumulate, stream);
-  return fail("gemm_bf16: unknown result dtype %d", c_dtype);
+  const bf16* A = (const bf16*)a;
+  const bf16* W = (const bf16*)w;
+  if (M <= 64) {
+#define GB_SK(EPI, CT) return launch_skinny<EPI, CT>(A, lda, W, ldw, (CT*)c, ldc, M, N, K, stream)
+    if (epilogue == EPI_STORE && c_dtype == kF32) GB_SK(EPI_STORE, float);
+    if (epilogue == EPI_STORE && c_dtype == kBF16) GB_SK(EPI_STORE, bf16);
+    if (epilogue == EPI_ACCUMULATE) GB_SK(EPI_ACCUMULATE, float);
+    if (epilogue == EPI_SILU_MUL && c_dtype == kF32) GB_SK(EPI_SILU_MUL, float);
+    GB_SK(EPI_SILU_MUL, bf16);
+#undef GB_SK
+  }
+  const dim3 grid((N + TBN - 1) / TBN, (M + TBM - 1) / TBM), block(256);
+  GB_REQUIRE(grid.y <= 65535, "gemm_bf16: M=%d needs more than 65535 row tiles", M);
+  if (c_dtype == kF32)
+    hipLaunchKernelGGL(gemm_tiled_kernel<float>, grid, block, 0, stream, A, lda, W, ldw, (float*)c, ldc, M, N, K,
+                       epilogue == EPI_ACCUMULATE);
+  else
+    hipLaunchKernelGGL(gemm_tiled_kernel<bf16>, grid, block, 0, stream, A, lda, W, ldw, (bf16*)c, ldc, M, N, K, 0);
+  return launched("gemm_bf16 (tiled)");
 }

@@ -35,6 +35,7 @@ class DecodeLoop:
         cap = max_context or (max(lens) + 4096)
         if G:
             cap = min(cap, cache.num_pages(0) * P)
+        self.cap = cap
         self.maxp = max(1, -(-cap // P))
         # layout: 8 per-request arrays, then per group the rows and the tables
         total = 8 * S + G * (S + S * self.maxp)
@@ -71,7 +72,8 @@ class DecodeLoop:
                                host=host, attention_impl=engine.attention_impl)
         self.out = torch.zeros(S, dtype=torch.int32, device=engine.device)
         self.use_graph = use_graph
-        self.graph: Optional[torch.cuda.CUDAGraph] = None
+        self.graphs = {}          # context bucket -> captured graph
+        self.warm = set()         # buckets that have run once without a graph
         self.steps = 0
 
     def _run(self) -> None:
@@ -97,19 +99,24 @@ class DecodeLoop:
                 self.h_slots[g][i] = self.h_tables[g][i, pos // P] * P + pos % P
         eng._apply_copies()
         self.dev.copy_(self.host, non_blocking=True)
+        # the attention kernel's split of the context is fixed per launch: one graph per bucket of 1,024 tokens
+        bucket = min(self.cap, -(-(max(self.lens) + 1) // 1024) * 1024)
+        self.ctx.host["max_context"] = bucket
+        graph = self.graphs.get(bucket)
         if not self.use_graph:
             self._run()
-        elif self.graph is None and self.steps == 0:
-            self._run()                      # the first step runs plainly: buffers reach their sizes
-        elif self.graph is None:
+        elif graph is not None:
+            graph.replay()
+        elif bucket not in self.warm:
+            self._run()                      # the first step of a bucket runs plainly: buffers reach their sizes
+            self.warm.add(bucket)
+        else:
             torch.cuda.synchronize()
             graph = torch.cuda.CUDAGraph()
             with torch.cuda.graph(graph):
                 self._run()
-            self.graph = graph
+            self.graphs[bucket] = graph
             graph.replay()                   # capture does not execute
-        else:
-            self.graph.replay()
         nxt = self.out.tolist()              # waits for the step
         for i, sid in enumerate(self.sids):
             cache.commit(sid, [self.tokens[i]])
@@ -120,4 +127,4 @@ class DecodeLoop:
         return nxt
 
     def close(self) -> None:
-        self.graph = None
+        self.graphs.clear()

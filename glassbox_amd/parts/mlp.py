@@ -27,8 +27,12 @@ class SwiGLU(FeedForward):
 
     def forward(self, ctx, h, residual):
         n = h.shape[0]
-        gate_up = ctx.buffer("gate_up", (n, 2 * self.intermediate), ctx.dtype)
-        ops.gemm(h, self.w_gate_up, gate_up)
         act = ctx.buffer("act", (n, self.intermediate), ctx.dtype)
-        ops.silu_mul(gate_up, act)
+        if h.dtype == torch.bfloat16 and n <= ops.SILU_MUL_MAX_ROWS and self.intermediate % 8 == 0:
+            # few rows (decoding): the activation is applied where the product's tile is finished
+            ops.gemm(h, self.w_gate_up, act, silu_mul=True)
+        else:
+            gate_up = ctx.buffer("gate_up", (n, 2 * self.intermediate), ctx.dtype)
+            ops.gemm(h, self.w_gate_up, gate_up)
+            ops.silu_mul(gate_up, act)
         ops.gemm(act, self.w_down, residual, accumulate=True)

@@ -24,7 +24,9 @@ def to_dev(t, dtype=None):
 # (crates/glassbox-core/src/kernels.rs:697) and larger ones that cross tile edges
 GEMM_SHAPES_F32 = [(1, 32, 1), (8, 64, 2), (17, 64, 3), (33, 96, 9), (50, 160, 17), (331, 100, 70), (130, 257, 129)]
 GEMM_SHAPES_BF16 = [(1, 32, 1), (8, 64, 2), (17, 64, 3), (33, 96, 9), (50, 160, 17), (331, 104, 64), (331, 104, 65),
-                    (130, 264, 129), (16, 2048, 8), (272, 72, 300), (49, 520, 33)]
+                    (130, 264, 129), (16, 2048, 8), (272, 72, 300), (49, 520, 33),
+                    # few rows of W and a long k: the skinny kernel splits k over workgroups
+                    (2048, 2048, 8), (2048, 8192, 8), (64, 2056, 1), (100, 4104, 33), (2048, 2048, 64), (48, 8192, 17)]
 
 
 @pytest.mark.parametrize("N,K,M", GEMM_SHAPES_F32)
@@ -53,6 +55,37 @@ def test_gemm_bf16(N, K, M, out):
     # bfloat16 result) the final rounding differ from the float64 sum
     tol = 1e-4 * math.sqrt(K) + (2 ** -8) * want.abs().max().item() * (out == "bf16")
     assert (got - want).abs().max().item() <= tol
+
+
+@pytest.mark.parametrize("I,K,M", [(8, 32, 1), (176, 64, 5), (144, 80, 16), (200, 2048, 17), (8192, 2048, 8), (88, 4104, 64)])
+def test_gemm_bf16_fused_silu_mul(I, K, M):
+    """Stacked gate/up rows with the activation applied in the product's epilogue
+    (crates/glassbox-core/src/model.rs:335-340), against the formula in float64."""
+    from glassbox_amd import ops
+    a, w = rnd(M, K, seed=1).bfloat16(), (rnd(2 * I, K, seed=2) / math.sqrt(K)).bfloat16()
+    gu = a.double() @ w.double().T
+    g, u = gu[:, :I], gu[:, I:]
+    want = g / (1 + torch.exp(-g)) * u
+    for dt in (torch.bfloat16, torch.float32):
+        out = torch.full((M, I), 7.0, device=DEV, dtype=dt)
+        ops.gemm(to_dev(a), to_dev(w), out, silu_mul=True)
+        tol = 1e-4 + (2 ** -8) * want.abs().max().item() * (dt == torch.bfloat16)
+        assert (out.cpu().double() - want).abs().max().item() <= tol
+    # twice in a row: the tile counters were left at zero
+    out2 = torch.empty(M, I, device=DEV, dtype=torch.float32)
+    ops.gemm(to_dev(a), to_dev(w), out2, silu_mul=True)
+    assert torch.equal(out2, out)
+
+
+def test_gemm_bf16_split_k_is_the_same_on_every_run():
+    from glassbox_amd import ops
+    a, w = to_dev(rnd(8, 8192, seed=1).bfloat16()), to_dev(rnd(2048, 8192, seed=2).bfloat16())
+    base = torch.zeros(8, 2048, device=DEV)
+    ops.gemm(a, w, base, accumulate=True)
+    for _ in range(5):
+        again = torch.zeros(8, 2048, device=DEV)
+        ops.gemm(a, w, again, accumulate=True)
+        assert torch.equal(again, base)
 
 
 def test_gemm_bf16_one_hot_rows_and_columns():
