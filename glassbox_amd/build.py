@@ -66,19 +66,27 @@ def _hipcc() -> str:
     raise BuildError("hipcc not found (looked at $HIPCC, PATH and /opt/rocm/bin): the device kernels cannot be built")
 
 
+_dir_lock = threading.Lock()
+_dir: Optional[str] = None
+
+
 def _lib_dir() -> str:
-    d = os.path.join(_HERE, "_lib")
-    try:
-        os.makedirs(d, exist_ok=True)
-        probe = os.path.join(d, f".w{os.getpid()}")
-        with open(probe, "w"):
-            pass
-        os.remove(probe)
-        return d
-    except OSError:
-        d = os.path.join(tempfile.gettempdir(), f"glassbox_amd-{os.getuid()}", "_lib")
-        os.makedirs(d, exist_ok=True)
-        return d
+    """Where built objects live: decided once per process (in-tree if writable)."""
+    global _dir
+    with _dir_lock:
+        if _dir is None:
+            d = os.path.join(_HERE, "_lib")
+            try:
+                os.makedirs(d, exist_ok=True)
+                probe = os.path.join(d, f".w{os.getpid()}.{threading.get_ident()}")
+                with open(probe, "w"):
+                    pass
+                os.remove(probe)
+            except OSError:
+                d = os.path.join(tempfile.gettempdir(), f"glassbox_amd-{os.getuid()}", "_lib")
+                os.makedirs(d, exist_ok=True)
+            _dir = d
+        return _dir
 
 
 def _digest(name: str) -> str:
@@ -96,8 +104,7 @@ def lib_path(name: str) -> str:
     return os.path.join(_lib_dir(), f"libgb_{name}.so")
 
 
-def is_current(name: str) -> bool:
-    path = lib_path(name)
+def _current_at(path: str, name: str) -> bool:
     stamp = path + ".stamp"
     if not (os.path.exists(path) and os.path.exists(stamp)):
         return False
@@ -106,6 +113,20 @@ def is_current(name: str) -> bool:
             return fh.read().strip() == _digest(name)
     except OSError:
         return False
+
+
+def find_current(name: str) -> Optional[str]:
+    """Path of a built library that matches its sources: the package folder first (also when it
+    cannot be written, as in a read-only checkout that ships built objects), then the fallback."""
+    for d in (os.path.join(_HERE, "_lib"), _lib_dir()):
+        path = os.path.join(d, f"libgb_{name}.so")
+        if _current_at(path, name):
+            return path
+    return None
+
+
+def is_current(name: str) -> bool:
+    return find_current(name) is not None
 
 
 def compile_library(name: str, quiet: bool = False) -> str:
@@ -169,12 +190,11 @@ def load(name: str) -> ctypes.CDLL:
             return lib
         if name not in LIBRARIES:
             raise BuildError(f"no native library called {name!r}")
-        if not is_current(name):
-            compile_library(name)
+        path = find_current(name) or compile_library(name)
         try:
-            lib = ctypes.CDLL(lib_path(name))
+            lib = ctypes.CDLL(path)
         except OSError as e:
-            raise BuildError(f"cannot load {lib_path(name)}: {e}") from None
+            raise BuildError(f"cannot load {path}: {e}") from None
         _loaded[name] = lib
         return lib
 
