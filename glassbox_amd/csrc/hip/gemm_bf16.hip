@@ -271,8 +271,8 @@ inline void skinny_plan(int tiles, int K, int mt, int* waves, int* iters, int* r
   *iters = (mt == 1 && per_wave >= 2) ? 2 : 1;
   if (const char* env = getenv("GB_SKINNY")) {
     int wv = 0, it = 0, r = 0;
-    if (sscanf(env, "%d,%d,%d", &wv, &it, &r) == 3 && (wv == 4 || wv == 16) && (it == 1 || it == 2 || it == 4 || it == 8) &&
-        (r == 1 || r == 2) && !(r == 2 && it == 8)) {
+    if (sscanf(env, "%d,%d,%d", &wv, &it, &r) == 3 && (wv == 4 || wv == 16) && (it == 1 || (it == 2 && mt == 1)) &&
+        (r == 1 || r == 2)) {
       *waves = wv;
       *iters = it;
       *rt = r;
@@ -286,11 +286,14 @@ int launch_skinny_mt(int tiles, const bf16* a, int lda, const bf16* w, int ldw, 
   int waves, iters, rt;
   skinny_plan(tiles, K, MT, &waves, &iters, &rt);
 #define GB_CFG(WV, IT, RT)                                                                                                \
-  if (waves == WV && iters == IT && rt == RT)                                                                             \
-    hipLaunchKernelGGL((gemm_skinny_kernel<MT, WV, IT, RT, EPI, CT>), dim3((tiles + RT - 1) / RT), dim3(WV * 64), 0, stream, \
+  if (waves == WV && iters == (IT) && rt == RT)                                                                           \
+    hipLaunchKernelGGL((gemm_skinny_kernel<MT, WV, (IT), RT, EPI, CT>), dim3((tiles + RT - 1) / RT), dim3(WV * 64), 0, stream, \
                        a, lda, w, ldw, c, ldc, M, N, K);
-  GB_CFG(4, 1, 1) GB_CFG(4, 2, 1) GB_CFG(4, 4, 1) GB_CFG(4, 8, 1) GB_CFG(16, 1, 1) GB_CFG(16, 2, 1) GB_CFG(16, 4, 1)
-  GB_CFG(16, 8, 1) GB_CFG(4, 1, 2) GB_CFG(4, 2, 2) GB_CFG(4, 4, 2) GB_CFG(16, 1, 2) GB_CFG(16, 2, 2) GB_CFG(16, 4, 2)
+  // the configurations skinny_plan can ask for: two loads in flight only with one column block
+  GB_CFG(4, 1, 1) GB_CFG(4, 1, 2) GB_CFG(16, 1, 1) GB_CFG(16, 1, 2)
+  if (MT == 1) {
+    GB_CFG(4, MT == 1 ? 2 : 1, 1) GB_CFG(4, MT == 1 ? 2 : 1, 2) GB_CFG(16, MT == 1 ? 2 : 1, 1) GB_CFG(16, MT == 1 ? 2 : 1, 2)
+  }
 #undef GB_CFG
   return launched("gemm_bf16 (skinny)");
 }
