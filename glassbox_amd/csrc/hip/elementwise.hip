@@ -37,20 +37,42 @@ extern "C" int gb_embed(const void* table, int table_dtype, const int32_t* ids, 
 // ------------------------------------------------------------------------ RMS norm
 // ms = sum(x^2)/d ; s = 1/sqrt(ms + eps) ; out = g * (x * s)     (model.rs:94-100)
 // One block per output row; `rows` (optional) picks the input row of each output row.
-template <typename G, typename O>
+// A thread keeps its VPT values of the row (and of gamma) in registers across the reduction, so the
+// row is read once and the loads of gamma overlap the sum; rows longer than VPT * threads are read
+// a second time.  The sum's order is fixed by the thread layout.
+template <typename G, typename O, int VPT>
 __global__ void rmsnorm_kernel(const float* __restrict__ x, const G* __restrict__ gamma, const int32_t* __restrict__ rows,
                                O* __restrict__ out, int d, float eps) {
-  __shared__ float scratch[17];
-  const int r = blockIdx.x;
+  __shared__ float partial[16];
+  const int r = blockIdx.x, tid = threadIdx.x, nt = blockDim.x;
   const float* xr = x + (size_t)(rows ? rows[r] : r) * d;
+  float v[VPT], g[VPT];
   float ss = 0.f;
-  for (int c = threadIdx.x; c < d; c += blockDim.x) {
-    float v = xr[c];
-    ss += v * v;
+#pragma unroll
+  for (int j = 0; j < VPT; ++j) {
+    const int c = tid + j * nt;
+    v[j] = c < d ? xr[c] : 0.f;
+    g[j] = c < d ? to_f(gamma[c]) : 0.f;
   }
-  ss = block_sum(ss, scratch);
-  const float s = 1.0f / sqrtf(ss / (float)d + eps);
-  for (int c = threadIdx.x; c < d; c += blockDim.x) out[(size_t)r * d + c] = from_f<O>(to_f(gamma[c]) * (xr[c] * s));
+#pragma unroll
+  for (int j = 0; j < VPT; ++j) ss += v[j] * v[j];
+  for (int c = tid + VPT * nt; c < d; c += nt) {
+    const float t = xr[c];
+    ss += t * t;
+  }
+  ss = wave_sum(ss);
+  if (tid % kWave == 0) partial[tid / kWave] = ss;
+  __syncthreads();
+  float total = 0.f;
+  for (int w = 0; w < (nt + kWave - 1) / kWave; ++w) total += partial[w];
+  const float s = 1.0f / sqrtf(total / (float)d + eps);
+  O* orow = out + (size_t)r * d;
+#pragma unroll
+  for (int j = 0; j < VPT; ++j) {
+    const int c = tid + j * nt;
+    if (c < d) orow[c] = from_f<O>(g[j] * (v[j] * s));
+  }
+  for (int c = tid + VPT * nt; c < d; c += nt) orow[c] = from_f<O>(to_f(gamma[c]) * (xr[c] * s));
 }
 
 extern "C" int gb_rmsnorm(const float* x, const void* gamma, int gamma_dtype, const int32_t* rows, void* out,
@@ -58,8 +80,14 @@ extern "C" int gb_rmsnorm(const float* x, const void* gamma, int gamma_dtype, co
   GB_REQUIRE(m >= 0 && d > 0, "rmsnorm: bad sizes m=%d d=%d", m, d);
   if (m == 0) return 0;
   const int threads = d >= 1024 ? 256 : (d >= 256 ? 128 : 64);
-#define GB_LAUNCH(G, O) \
-  hipLaunchKernelGGL((rmsnorm_kernel<G, O>), dim3(m), dim3(threads), 0, stream, x, (const G*)gamma, rows, (O*)out, d, eps)
+  const int per_thread = (d + threads - 1) / threads;
+#define GB_LAUNCH(G, O)                                                                                                     \
+  do {                                                                                                                      \
+    if (per_thread <= 4)                                                                                                    \
+      hipLaunchKernelGGL((rmsnorm_kernel<G, O, 4>), dim3(m), dim3(threads), 0, stream, x, (const G*)gamma, rows, (O*)out, d, eps); \
+    else                                                                                                                    \
+      hipLaunchKernelGGL((rmsnorm_kernel<G, O, 16>), dim3(m), dim3(threads), 0, stream, x, (const G*)gamma, rows, (O*)out, d, eps); \
+  } while (0)
   if (gamma_dtype == kF32 && out_dtype == kF32) GB_LAUNCH(float, float);
   else if (gamma_dtype == kF32 && out_dtype == kBF16) GB_LAUNCH(float, bf16);
   else if (gamma_dtype == kBF16 && out_dtype == kF32) GB_LAUNCH(bf16, float);
@@ -114,26 +142,38 @@ __global__ void rope_store_kernel(T* __restrict__ qkv, int row_stride, const flo
   const int page = slot >= 0 ? slot / page_size : 0, off = slot >= 0 ? slot % page_size : 0;
   // queries, then keys: (nh + nkv) heads of `half` pairs
   const int pairs = (nh + nkv) * half;
-  for (int p = threadIdx.x; p < pairs; p += blockDim.x) {
-    const int head = p / half, i = p % half;
-    T* h = row + (size_t)head * hd;
-    float x0 = to_f(h[i]), x1 = to_f(h[i + half]);
-    float y0 = x0, y1 = x1;
-    if (rotate) {
-      y0 = x0 * c[i] - x1 * s[i];
-      y1 = x1 * c[i] + x0 * s[i];
+  // eight pairs a thread at a time: all loads first, so that they are in flight together (the
+  // stores into the row would otherwise order every later load behind them)
+  constexpr int B = 8;
+  for (int base = threadIdx.x; base < pairs; base += blockDim.x * B) {
+    float x0[B], x1[B], cc[B], sn[B];
+#pragma unroll
+    for (int j = 0; j < B; ++j) {
+      const int p = base + j * blockDim.x;
+      if (p < pairs) {
+        const int head = p / half, i = p % half;
+        const T* h = row + (size_t)head * hd;
+        x0[j] = to_f(h[i]);
+        x1[j] = to_f(h[i + half]);
+        cc[j] = rotate ? c[i] : 1.f;
+        sn[j] = rotate ? s[i] : 0.f;
+      }
     }
-    if (head < nh) {
-      h[i] = from_f<T>(y0);
-      h[i + half] = from_f<T>(y1);
-    } else {
-      h[i] = from_f<T>(y0);  // keep the rotated key in the row too: parts may read it back
-      h[i + half] = from_f<T>(y1);
-      if (slot >= 0) {
-        const int kvh = head - nh;
-        T* dst = k_pages + (((size_t)page * nkv + kvh) * page_size + off) * hd;
-        dst[i] = from_f<T>(y0);
-        dst[i + half] = from_f<T>(y1);
+#pragma unroll
+    for (int j = 0; j < B; ++j) {
+      const int p = base + j * blockDim.x;
+      if (p < pairs) {
+        const int head = p / half, i = p % half;
+        T* h = row + (size_t)head * hd;
+        const T y0 = from_f<T>(rotate ? x0[j] * cc[j] - x1[j] * sn[j] : x0[j]);
+        const T y1 = from_f<T>(rotate ? x1[j] * cc[j] + x0[j] * sn[j] : x1[j]);
+        h[i] = y0;  // rotated keys stay in the row too: parts may read them back
+        h[i + half] = y1;
+        if (head >= nh && slot >= 0) {
+          T* dst = k_pages + (((size_t)page * nkv + (head - nh)) * page_size + off) * hd;
+          dst[i] = y0;
+          dst[i + half] = y1;
+        }
       }
     }
   }

@@ -34,13 +34,22 @@ __device__ __forceinline__ uint64_t composite(float v, int idx) {
 
 // ---------------------------------------------------------------------------- argmax
 // first maximum wins (sampler.rs:49-57) = the largest composite key
-__global__ __launch_bounds__(TPB) void argmax_kernel(const float* __restrict__ logits, int32_t* __restrict__ out, int V) {
-  __shared__ uint64_t best[TPB / kWave];
+constexpr int ARGMAX_TPB = 1024;
+__global__ __launch_bounds__(ARGMAX_TPB) void argmax_kernel(const float* __restrict__ logits, int32_t* __restrict__ out, int V) {
+  __shared__ uint64_t best[ARGMAX_TPB / kWave];
   const float* row = logits + (size_t)blockIdx.x * V;
   uint64_t b = 0;
-  for (int i = threadIdx.x; i < V; i += TPB) {
-    const uint64_t c = composite(row[i], i);
-    b = c > b ? c : b;
+  // four loads in flight per thread
+  for (int i0 = threadIdx.x; i0 < V; i0 += 4 * ARGMAX_TPB) {
+    float v[4];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) v[j] = i0 + j * ARGMAX_TPB < V ? row[i0 + j * ARGMAX_TPB] : 0.f;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const int i = i0 + j * ARGMAX_TPB;
+      const uint64_t c = i < V ? composite(v[j], i) : 0;
+      b = c > b ? c : b;
+    }
   }
 #pragma unroll
   for (int o = kWave / 2; o > 0; o >>= 1) {
@@ -50,7 +59,7 @@ __global__ __launch_bounds__(TPB) void argmax_kernel(const float* __restrict__ l
   if (threadIdx.x % kWave == 0) best[threadIdx.x / kWave] = b;
   __syncthreads();
   if (threadIdx.x == 0) {
-    for (int w = 1; w < TPB / kWave; ++w) b = best[w] > b ? best[w] : b;
+    for (int w = 1; w < ARGMAX_TPB / kWave; ++w) b = best[w] > b ? best[w] : b;
     out[blockIdx.x] = (int32_t)(((1u << IDX_BITS) - 1u) - (uint32_t)(b & ((1u << IDX_BITS) - 1u)));
   }
 }
@@ -307,7 +316,7 @@ __global__ __launch_bounds__(TPB) void sample_kernel(const float* __restrict__ l
 extern "C" int gb_argmax(const float* logits, int32_t* out, int rows, int V, hipStream_t stream) {
   GB_REQUIRE(rows >= 0 && V > 0 && V <= (1 << IDX_BITS), "argmax: vocabulary %d is outside 1..%d", V, 1 << IDX_BITS);
   if (rows == 0) return 0;
-  hipLaunchKernelGGL(argmax_kernel, dim3(rows), dim3(TPB), 0, stream, logits, out, V);
+  hipLaunchKernelGGL(argmax_kernel, dim3(rows), dim3(ARGMAX_TPB), 0, stream, logits, out, V);
   return launched("argmax");
 }
 
