@@ -4,13 +4,13 @@
 // is the layout MFMA operands want: every lane loads 8 consecutive k as one 16-byte word.
 //
 // Two kernels:
-//  * tiled  (M > 64, prompt portions): 128x128 tile per workgroup of 4 waves, each wave a 64x64
-//    block of 2x2 v_mfma_f32_32x32x16_bf16 tiles, operands staged through LDS in k-steps of 32
-//    with two buffers.
-//  * skinny (M <= 64, decoding): bound by reading W once.  A workgroup owns 16 rows of W; its 4
+//  * tiled  (M > 64, prompt portions): a workgroup of 2x2 waves, each wave a block of up to 4x2
+//    v_mfma_f32_32x32x16_bf16 tiles (workgroup tile up to 256x128), operands staged through LDS in
+//    k-steps of 32 with two buffers; the SiLU-multiply of stacked gate/up rows can be its epilogue.
+//  * skinny (M <= 64, decoding): bound by reading W once.  A workgroup owns 16 or 32 rows of W; its
 //    waves take interleaved 64-wide k blocks, stream W straight from memory into MFMA operands
 //    (v_mfma_f32_16x16x32_bf16, W as the A operand so that the 16 rows fill the tile) and combine
-//    through LDS in a fixed order.
+//    through LDS in a fixed order; it can norm float32 rows on the way and apply the SiLU-multiply.
 // In both, every output cell is summed in an order fixed by (K, kernel) alone, not by M or by
 // the cell's neighbours.  C is bfloat16 or float32; accumulation (+=) is into float32.
 #include "common.h"
@@ -34,43 +34,84 @@ template <> __device__ __forceinline__ void store_c<float>(float* c, float v, in
 template <> __device__ __forceinline__ void store_c<bf16>(bf16* c, float v, int) { *c = (bf16)v; }
 
 // ------------------------------------------------------------------------- tiled
-constexpr int TBM = 128, TBN = 128, TBK = 32, TLD = TBK + 8;  // LDS row stride in elements (80 bytes)
+// A workgroup of 2 x 2 waves; a wave owns WM x WN tiles of 32 x 32, so the workgroup's tile is
+// (64 WM) x (64 WN).  Operands are staged through LDS in k-steps of 32, two buffers; rows are padded
+// to 80 bytes so that the 16-byte operand reads of a wave spread over the banks.
+//
+// EPI_SILU_MUL (WN = 2): W stacks gate rows [0, N/2) over up rows [N/2, N).  Of a wave's two column
+// tiles the first holds 32 gate columns and the second the 32 up columns that belong to them, so
+// act = gate / (1 + exp(-gate)) * up (crates/glassbox-core/src/model.rs:336-340) is formed in
+// registers and C is [M, N/2].
+enum : int { EPI_STORE = 0, EPI_ACCUMULATE = 1, EPI_SILU_MUL = 2 };
+constexpr int TBK = 64, TLD = TBK + 8;  // k-step; LDS row stride in elements (144 bytes)
+constexpr int TCPR = TBK / 8;           // 16-byte chunks per row of a k-step
+constexpr int TKS = TBK / 16;           // MFMA k-steps per LDS k-step
 
-template <typename CT>
+template <int WM, int WN, int EPI, typename CT>
 __global__ __launch_bounds__(256) void gemm_tiled_kernel(const bf16* __restrict__ a, int lda, const bf16* __restrict__ w,
-                                                         int ldw, CT* __restrict__ c, int ldc, int M, int N, int K,
-                                                         int accumulate) {
-  __shared__ __attribute__((aligned(16))) bf16 As[2][TBM][TLD];
-  __shared__ __attribute__((aligned(16))) bf16 Ws[2][TBN][TLD];
+                                                         int ldw, CT* __restrict__ c, int ldc, int M, int N, int K) {
+  constexpr int BM = 64 * WM, BN = 64 * WN;
+  constexpr int CA = BM * TCPR / 256, CW = BN * TCPR / 256;  // chunks a thread moves per k-step
+  __shared__ __attribute__((aligned(16))) bf16 As[2][BM][TLD];
+  __shared__ __attribute__((aligned(16))) bf16 Ws[2][BN][TLD];
   const int tid = threadIdx.x, lane = tid % 64, wave = tid / 64;
-  const int wm = wave / 2, wn = wave % 2;  // 2 x 2 waves, 64 x 64 each
-  const int m0 = blockIdx.y * TBM, n0 = blockIdx.x * TBN;
+  const int wm = wave / 2, wn = wave % 2;
+  const int m0 = blockIdx.y * BM;
+  const int half = N / 2;  // EPI_SILU_MUL: number of gate rows
+  // row of W behind row r of the workgroup's W tile (r = wn*32*WN + j*32 + column)
+  auto w_row = [&](int r) -> int {
+    if (EPI == EPI_SILU_MUL) {
+      const int wv = r / 64, j = (r % 64) / 32, col = r % 32;
+      const int n = blockIdx.x * 64 + wv * 32 + col;
+      return n < half ? (j ? half + n : n) : -1;
+    }
+    const int n = blockIdx.x * BN + r;
+    return n < N ? n : -1;
+  };
 
-  f32x16 acc[2][2];
+  f32x16 acc[WM][WN];
 #pragma unroll
-  for (int i = 0; i < 2; ++i)
+  for (int i = 0; i < WM; ++i)
 #pragma unroll
-    for (int j = 0; j < 2; ++j)
+    for (int j = 0; j < WN; ++j)
 #pragma unroll
       for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
 
-  // each thread moves two 16-byte chunks of A and two of W per k-step
-  bf16x8 ga[2], gw[2];
+  bf16x8 ga[CA], gw[CW];
+  const bf16* asrc[CA];
+  const bf16* wsrc[CW];
+#pragma unroll
+  for (int j = 0; j < CA; ++j) {
+    const int row = m0 + (tid + 256 * j) / TCPR;
+    asrc[j] = row < M ? a + (size_t)row * lda : nullptr;
+  }
+#pragma unroll
+  for (int j = 0; j < CW; ++j) {
+    const int row = w_row((tid + 256 * j) / TCPR);
+    wsrc[j] = row >= 0 ? w + (size_t)row * ldw : nullptr;
+  }
   auto fetch = [&](int k0) {
 #pragma unroll
-    for (int j = 0; j < 2; ++j) {
-      const int ch = tid + 256 * j, row = ch / 4, kc = (ch % 4) * 8;
-      const int gk = k0 + kc;
-      ga[j] = (m0 + row < M && gk < K) ? load8(a + (size_t)(m0 + row) * lda + gk) : zero8();
-      gw[j] = (n0 + row < N && gk < K) ? load8(w + (size_t)(n0 + row) * ldw + gk) : zero8();
+    for (int j = 0; j < CA; ++j) {
+      const int gk = k0 + ((tid + 256 * j) % TCPR) * 8;
+      ga[j] = (asrc[j] && gk < K) ? load8(asrc[j] + gk) : zero8();
+    }
+#pragma unroll
+    for (int j = 0; j < CW; ++j) {
+      const int gk = k0 + ((tid + 256 * j) % TCPR) * 8;
+      gw[j] = (wsrc[j] && gk < K) ? load8(wsrc[j] + gk) : zero8();
     }
   };
   auto stash = [&](int buf) {
 #pragma unroll
-    for (int j = 0; j < 2; ++j) {
-      const int ch = tid + 256 * j, row = ch / 4, kc = (ch % 4) * 8;
-      *reinterpret_cast<bf16x8*>(&As[buf][row][kc]) = ga[j];
-      *reinterpret_cast<bf16x8*>(&Ws[buf][row][kc]) = gw[j];
+    for (int j = 0; j < CA; ++j) {
+      const int ch = tid + 256 * j;
+      *reinterpret_cast<bf16x8*>(&As[buf][ch / TCPR][(ch % TCPR) * 8]) = ga[j];
+    }
+#pragma unroll
+    for (int j = 0; j < CW; ++j) {
+      const int ch = tid + 256 * j;
+      *reinterpret_cast<bf16x8*>(&Ws[buf][ch / TCPR][(ch % TCPR) * 8]) = gw[j];
     }
   };
 
@@ -78,39 +119,92 @@ __global__ __launch_bounds__(256) void gemm_tiled_kernel(const bf16* __restrict_
   stash(0);
   __syncthreads();
   const int steps = (K + TBK - 1) / TBK;
+  const int arow = wm * 32 * WM + lane % 32, wrow = wn * 32 * WN + lane % 32, koff = 8 * (lane / 32);
   for (int s = 0; s < steps; ++s) {
     const int buf = s & 1;
     if (s + 1 < steps) fetch((s + 1) * TBK);
+    // operands of MFMA step ks+1 are read from LDS while the MFMAs of step ks run
+    bf16x8 fa[2][WM], fw[2][WN];
 #pragma unroll
-    for (int ks = 0; ks < TBK / 16; ++ks) {
-      bf16x8 fa[2], fw[2];
-      const int kk = ks * 16 + 8 * (lane / 32);
+    for (int i = 0; i < WM; ++i) fa[0][i] = *reinterpret_cast<const bf16x8*>(&As[buf][arow + i * 32][koff]);
 #pragma unroll
-      for (int i = 0; i < 2; ++i) fa[i] = *reinterpret_cast<const bf16x8*>(&As[buf][wm * 64 + i * 32 + lane % 32][kk]);
+    for (int j = 0; j < WN; ++j) fw[0][j] = *reinterpret_cast<const bf16x8*>(&Ws[buf][wrow + j * 32][koff]);
 #pragma unroll
-      for (int j = 0; j < 2; ++j) fw[j] = *reinterpret_cast<const bf16x8*>(&Ws[buf][wn * 64 + j * 32 + lane % 32][kk]);
+    for (int ks = 0; ks < TKS; ++ks) {
+      const int cur = ks & 1, nxt = cur ^ 1;
+      if (ks + 1 < TKS) {
 #pragma unroll
-      for (int i = 0; i < 2; ++i)
+        for (int i = 0; i < WM; ++i) fa[nxt][i] = *reinterpret_cast<const bf16x8*>(&As[buf][arow + i * 32][(ks + 1) * 16 + koff]);
 #pragma unroll
-        for (int j = 0; j < 2; ++j) acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa[i], fw[j], acc[i][j], 0, 0, 0);
+        for (int j = 0; j < WN; ++j) fw[nxt][j] = *reinterpret_cast<const bf16x8*>(&Ws[buf][wrow + j * 32][(ks + 1) * 16 + koff]);
+      }
+#pragma unroll
+      for (int i = 0; i < WM; ++i)
+#pragma unroll
+        for (int j = 0; j < WN; ++j)
+          acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa[cur][i], fw[cur][j], acc[i][j], 0, 0, 0);
     }
     if (s + 1 < steps) stash(buf ^ 1);
     __syncthreads();
   }
 
   // accumulator layout of a 32x32 tile: lane holds column lane%32, rows 8*(r/4) + 4*(lane/32) + r%4
+  if (EPI == EPI_SILU_MUL) {
+    const int gn = blockIdx.x * 64 + wn * 32 + lane % 32;
+    if (gn >= half) return;
 #pragma unroll
-  for (int i = 0; i < 2; ++i)
+    for (int i = 0; i < WM; ++i)
 #pragma unroll
-    for (int j = 0; j < 2; ++j) {
-      const int gn = n0 + wn * 64 + j * 32 + lane % 32;
+      for (int r = 0; r < 16; ++r) {
+        const int gm = m0 + wm * 32 * WM + i * 32 + 8 * (r / 4) + 4 * (lane / 32) + r % 4;
+        const float g = acc[i][0][r], u = acc[i][WN - 1][r];
+        if (gm < M) c[(size_t)gm * ldc + gn] = (CT)(g / (1.0f + __expf(-g)) * u);
+      }
+    return;
+  }
+#pragma unroll
+  for (int i = 0; i < WM; ++i)
+#pragma unroll
+    for (int j = 0; j < WN; ++j) {
+      const int gn = blockIdx.x * BN + wn * 32 * WN + j * 32 + lane % 32;
       if (gn >= N) continue;
 #pragma unroll
       for (int r = 0; r < 16; ++r) {
-        const int gm = m0 + wm * 64 + i * 32 + 8 * (r / 4) + 4 * (lane / 32) + r % 4;
-        if (gm < M) store_c<CT>(c + (size_t)gm * ldc + gn, acc[i][j][r], accumulate);
+        const int gm = m0 + wm * 32 * WM + i * 32 + 8 * (r / 4) + 4 * (lane / 32) + r % 4;
+        if (gm < M) store_c<CT>(c + (size_t)gm * ldc + gn, acc[i][j][r], EPI == EPI_ACCUMULATE);
       }
     }
+}
+
+// Tile of the workgroup, (64 WM) x (64 WN): large tiles re-read the operands least; smaller ones
+// when the large ones would leave compute units idle.  GB_TILED="wm,wn" overrides (for measurements).
+inline void tiled_plan(int M, int N, int* wm, int* wn) {
+  auto blocks = [&](int a, int b) { return ((M + 64 * a - 1) / (64 * a)) * ((N + 64 * b - 1) / (64 * b)); };
+  // measured at 512..8192 rows on SmolLM2-1.7B shapes: 128 x 128 beats 256 x 128 everywhere (the
+  // larger tile's registers leave one workgroup a compute unit); 128 x 64 when tiles are few
+  *wm = 2, *wn = 2;
+  if (blocks(2, 2) < 384) *wn = 1;
+  if (const char* env = getenv("GB_TILED")) {
+    int a = 0, b = 0;
+    if (sscanf(env, "%d,%d", &a, &b) == 2 && (a == 2 || a == 4) && (b == 1 || b == 2)) *wm = a, *wn = b;
+  }
+}
+
+template <int EPI, typename CT>
+int launch_tiled(const bf16* a, int lda, const bf16* w, int ldw, CT* c, int ldc, int M, int N, int K, hipStream_t stream) {
+  int wm, wn;
+  tiled_plan(M, EPI == EPI_SILU_MUL ? N / 2 * 2 : N, &wm, &wn);
+  if (EPI == EPI_SILU_MUL) wn = 2;
+  const int cols = EPI == EPI_SILU_MUL ? N / 2 : N, bn = EPI == EPI_SILU_MUL ? 64 : 64 * wn;
+  const dim3 grid((cols + bn - 1) / bn, (M + 64 * wm - 1) / (64 * wm)), block(256);
+  GB_REQUIRE(grid.y <= 65535, "gemm_bf16: M=%d needs more than 65535 row tiles", M);
+#define GB_T(A, B)            \
+  if (wm == (A) && wn == (B)) \
+    hipLaunchKernelGGL((gemm_tiled_kernel<(A), (B), EPI, CT>), grid, block, 0, stream, a, lda, w, ldw, c, ldc, M, N, K);
+  GB_T(4, 2) GB_T(2, 2)
+  if (EPI != EPI_SILU_MUL) { GB_T(4, EPI == EPI_SILU_MUL ? 2 : 1) GB_T(2, EPI == EPI_SILU_MUL ? 2 : 1) }
+#undef GB_T
+  return launched("gemm_bf16 (tiled)");
 }
 
 // ------------------------------------------------------------------------ skinny
@@ -126,13 +220,49 @@ __global__ __launch_bounds__(256) void gemm_tiled_kernel(const bf16* __restrict_
 // [0, N/2) and up rows [N/2, N); a tile takes 8 gate rows and the 8 up rows that belong to them
 // and writes act[m, j] = gate / (1 + exp(-gate)) * up (crates/glassbox-core/src/model.rs:336-340)
 // to C[M, N/2].
-enum : int { EPI_STORE = 0, EPI_ACCUMULATE = 1, EPI_SILU_MUL = 2 };
 
-template <int MT, int WAVES, int ITERS, int RT, int EPI, typename CT>
-__global__ __launch_bounds__(WAVES * 64) void gemm_skinny_kernel(const bf16* __restrict__ a, int lda,
+// The A operand of one lane: 8 consecutive k of row m.  Plain: bfloat16 rows as they are.  RMS: the
+// rows are the float32 residual; the operand is bf16(gamma[k] * x[k]) and sum(x^2) is gathered on
+// the way, so that the caller can scale the finished product by 1/sqrt(mean(x^2) + eps): the RMS
+// norm (crates/glassbox-core/src/model.rs:94-100) without a pass of its own.
+template <bool RMS>
+__device__ __forceinline__ bf16x8 load_a(const void* a, int lda, int m, int k, bool ok, const void* gamma, int gamma_f32,
+                                         float& ss) {
+  if (!ok) return zero8();
+  if (!RMS) return load8((const bf16*)a + (size_t)m * lda + k);
+  const float* x = (const float*)a + (size_t)m * lda + k;
+  const f32x4 x0 = *reinterpret_cast<const f32x4*>(x), x1 = *reinterpret_cast<const f32x4*>(x + 4);
+  float g[8];
+  if (gamma_f32) {
+    const f32x4 g0 = *reinterpret_cast<const f32x4*>((const float*)gamma + k);
+    const f32x4 g1 = *reinterpret_cast<const f32x4*>((const float*)gamma + k + 4);
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+      g[e] = g0[e];
+      g[4 + e] = g1[e];
+    }
+  } else {
+    const bf16x8 gb = load8((const bf16*)gamma + k);
+#pragma unroll
+    for (int e = 0; e < 8; ++e) g[e] = (float)gb[e];
+  }
+  bf16x8 out;
+#pragma unroll
+  for (int e = 0; e < 8; ++e) {
+    const float xe = e < 4 ? x0[e] : x1[e - 4];
+    ss += xe * xe;
+    out[e] = (bf16)(g[e] * xe);
+  }
+  return out;
+}
+
+template <int MT, int WAVES, int ITERS, int RT, int EPI, bool RMS, typename CT>
+__global__ __launch_bounds__(WAVES * 64) void gemm_skinny_kernel(const void* __restrict__ a, int lda,
                                                                  const bf16* __restrict__ w, int ldw, CT* __restrict__ c,
-                                                                 int ldc, int M, int N, int K) {
+                                                                 int ldc, int M, int N, int K, const void* __restrict__ gamma,
+                                                                 int gamma_f32, float eps) {
   __shared__ float part[WAVES][RT][MT][64][4];
+  __shared__ float sspart[RMS ? WAVES : 1][MT][64];
   const int tid = threadIdx.x, lane = tid % 64, wave = tid / 64;
   const int r = lane % 16, q = lane / 16;
   const bf16* wrow[RT];
@@ -148,12 +278,15 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_skinny_kernel(const bf16* __r
   }
 
   f32x4 acc[RT][MT];
+  float ss[MT];
 #pragma unroll
-  for (int rt = 0; rt < RT; ++rt)
+  for (int t = 0; t < MT; ++t) {
+    ss[t] = 0.f;
 #pragma unroll
-    for (int t = 0; t < MT; ++t)
+    for (int rt = 0; rt < RT; ++rt)
 #pragma unroll
       for (int e = 0; e < 4; ++e) acc[rt][t][e] = 0.f;
+  }
 
   // a 64-wide k block is two MFMA steps of 32: lane group q holds k = 8q..8q+7 of each
   for (int kbeg = 0; kbeg < K; kbeg += ITERS * WAVES * 64) {
@@ -167,13 +300,12 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_skinny_kernel(const bf16* __r
         wf[rt][it][1] = (row_ok[rt] && k + 32 < K) ? load8(wrow[rt] + k + 32) : zero8();
       }
     if (MT == 1) {
-      const bf16* arow = a + (size_t)(r < M ? r : 0) * lda;
       bf16x8 xf[ITERS][2];
 #pragma unroll
       for (int it = 0; it < ITERS; ++it) {
         const int k = kbeg + (wave + WAVES * it) * 64 + q * 8;
-        xf[it][0] = (r < M && k < K) ? load8(arow + k) : zero8();
-        xf[it][1] = (r < M && k + 32 < K) ? load8(arow + k + 32) : zero8();
+        xf[it][0] = load_a<RMS>(a, lda, r, k, r < M && k < K, gamma, gamma_f32, ss[0]);
+        xf[it][1] = load_a<RMS>(a, lda, r, k + 32, r < M && k + 32 < K, gamma, gamma_f32, ss[0]);
       }
 #pragma unroll
       for (int it = 0; it < ITERS; ++it)
@@ -189,9 +321,8 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_skinny_kernel(const bf16* __r
 #pragma unroll
         for (int t = 0; t < MT; ++t) {
           const int m = t * 16 + r;
-          const bf16* arow = a + (size_t)(m < M ? m : 0) * lda;
-          const bf16x8 x0 = (m < M && k < K) ? load8(arow + k) : zero8();
-          const bf16x8 x1 = (m < M && k + 32 < K) ? load8(arow + k + 32) : zero8();
+          const bf16x8 x0 = load_a<RMS>(a, lda, m, k, m < M && k < K, gamma, gamma_f32, ss[t]);
+          const bf16x8 x1 = load_a<RMS>(a, lda, m, k + 32, m < M && k + 32 < K, gamma, gamma_f32, ss[t]);
 #pragma unroll
           for (int rt = 0; rt < RT; ++rt) {
             acc[rt][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wf[rt][it][0], x0, acc[rt][t], 0, 0, 0);
@@ -207,6 +338,10 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_skinny_kernel(const bf16* __r
     for (int t = 0; t < MT; ++t)
 #pragma unroll
       for (int e = 0; e < 4; ++e) part[wave][rt][t][lane][e] = acc[rt][t][e];
+  if (RMS) {
+#pragma unroll
+    for (int t = 0; t < MT; ++t) sspart[wave][t][lane] = ss[t];
+  }
   __syncthreads();
   if (tid >= 256) return;
 
@@ -215,14 +350,25 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_skinny_kernel(const bf16* __r
   const int l = tid / 4, e = tid % 4;
   float v[RT][MT];
 #pragma unroll
-  for (int rt = 0; rt < RT; ++rt)
+  for (int t = 0; t < MT; ++t) {
+    float scale = 1.f;
+    if (RMS) {
+      // sum(x^2) of row m = t*16 + l%16: its k were spread over the waves and over the four lane groups
+      float tot = 0.f;
 #pragma unroll
-    for (int t = 0; t < MT; ++t) {
+      for (int wv = 0; wv < WAVES; ++wv)
+#pragma unroll
+        for (int qq = 0; qq < 4; ++qq) tot += sspart[wv][t][l % 16 + 16 * qq];
+      scale = 1.0f / sqrtf(tot / (float)K + eps);
+    }
+#pragma unroll
+    for (int rt = 0; rt < RT; ++rt) {
       float s = part[0][rt][t][l][e];
 #pragma unroll
       for (int wv = 1; wv < WAVES; ++wv) s += part[wv][rt][t][l][e];
-      v[rt][t] = s;
+      v[rt][t] = s * scale;
     }
+  }
   const int nrow = 4 * (l / 16) + e;  // row of the tile, 0..15
   if (EPI == EPI_SILU_MUL) {
     // rows 0..7 are gate, 8..15 the matching up rows: the up values travel through LDS.  Only the
@@ -280,15 +426,15 @@ inline void skinny_plan(int tiles, int K, int mt, int* waves, int* iters, int* r
   }
 }
 
-template <int MT, int EPI, typename CT>
-int launch_skinny_mt(int tiles, const bf16* a, int lda, const bf16* w, int ldw, CT* c, int ldc, int M, int N, int K,
-                     hipStream_t stream) {
+template <int MT, int EPI, bool RMS, typename CT>
+int launch_skinny_mt(int tiles, const void* a, int lda, const bf16* w, int ldw, CT* c, int ldc, int M, int N, int K,
+                     const void* gamma, int gamma_f32, float eps, hipStream_t stream) {
   int waves, iters, rt;
   skinny_plan(tiles, K, MT, &waves, &iters, &rt);
-#define GB_CFG(WV, IT, RT)                                                                                                \
-  if (waves == WV && iters == (IT) && rt == RT)                                                                           \
-    hipLaunchKernelGGL((gemm_skinny_kernel<MT, WV, (IT), RT, EPI, CT>), dim3((tiles + RT - 1) / RT), dim3(WV * 64), 0, stream, \
-                       a, lda, w, ldw, c, ldc, M, N, K);
+#define GB_CFG(WV, IT, RT)                                                                                                 \
+  if (waves == WV && iters == (IT) && rt == RT)                                                                            \
+    hipLaunchKernelGGL((gemm_skinny_kernel<MT, WV, (IT), RT, EPI, RMS, CT>), dim3((tiles + RT - 1) / RT), dim3(WV * 64), 0,  \
+                       stream, a, lda, w, ldw, c, ldc, M, N, K, gamma, gamma_f32, eps);
   // the configurations skinny_plan can ask for: two loads in flight only with one column block
   GB_CFG(4, 1, 1) GB_CFG(4, 1, 2) GB_CFG(16, 1, 1) GB_CFG(16, 1, 2)
   if (MT == 1) {
@@ -298,37 +444,48 @@ int launch_skinny_mt(int tiles, const bf16* a, int lda, const bf16* w, int ldw, 
   return launched("gemm_bf16 (skinny)");
 }
 
-template <int EPI, typename CT>
-int launch_skinny(const bf16* a, int lda, const bf16* w, int ldw, CT* c, int ldc, int M, int N, int K, hipStream_t stream) {
+template <int EPI, bool RMS, typename CT>
+int launch_skinny(const void* a, int lda, const bf16* w, int ldw, CT* c, int ldc, int M, int N, int K, const void* gamma,
+                  int gamma_f32, float eps, hipStream_t stream) {
   const int tiles = EPI == EPI_SILU_MUL ? (N / 2 + 7) / 8 : (N + 15) / 16;
   const int mt = (M + 15) / 16;
-  if (mt == 1) return launch_skinny_mt<1, EPI, CT>(tiles, a, lda, w, ldw, c, ldc, M, N, K, stream);
-  if (mt == 2) return launch_skinny_mt<2, EPI, CT>(tiles, a, lda, w, ldw, c, ldc, M, N, K, stream);
-  if (mt == 3) return launch_skinny_mt<3, EPI, CT>(tiles, a, lda, w, ldw, c, ldc, M, N, K, stream);
-  return launch_skinny_mt<4, EPI, CT>(tiles, a, lda, w, ldw, c, ldc, M, N, K, stream);
+#define GB_MT(T) \
+  if (mt == T) return launch_skinny_mt<T, EPI, RMS, CT>(tiles, a, lda, w, ldw, c, ldc, M, N, K, gamma, gamma_f32, eps, stream);
+  GB_MT(1) GB_MT(2) GB_MT(3)
+#undef GB_MT
+  return launch_skinny_mt<4, EPI, RMS, CT>(tiles, a, lda, w, ldw, c, ldc, M, N, K, gamma, gamma_f32, eps, stream);
 }
 
 }  // namespace
 
 // epilogue: 0 store, 1 accumulate (float32 C), 2 SiLU-multiply of stacked gate/up rows (C is [M, N/2]).
+// gamma != nullptr (at most 64 rows, bfloat16 C, epilogue 0 or 2): a is the float32 residual and the
+// product is that of its RMS-normed rows: bf16(gamma * x) as the operand, 1/sqrt(mean(x^2) + eps) on
+// the result.
 extern "C" int gb_gemm_bf16(const void* a, int lda, const void* w, int ldw, void* c, int ldc, int c_dtype, int M, int N,
-                            int K, int epilogue, hipStream_t stream) {
+                            int K, int epilogue, const void* gamma, int gamma_dtype, float eps, hipStream_t stream) {
   GB_REQUIRE(M >= 0 && N > 0 && K > 0, "gemm_bf16: bad sizes M=%d N=%d K=%d", M, N, K);
   GB_REQUIRE(K % 8 == 0, "gemm_bf16: the inner size K=%d must be a multiple of 8 (16-byte operand loads)", K);
-  GB_REQUIRE(lda % 8 == 0 && ldw % 8 == 0, "gemm_bf16: row strides (%d, %d) must be multiples of 8 elements", lda, ldw);
+  GB_REQUIRE(ldw % 8 == 0 && lda % (gamma ? 4 : 8) == 0, "gemm_bf16: row strides (%d, %d) must keep rows 16-byte aligned", lda, ldw);
   GB_REQUIRE(epilogue >= 0 && epilogue <= 2, "gemm_bf16: unknown epilogue %d", epilogue);
   const int ncols = epilogue == EPI_SILU_MUL ? N / 2 : N;
   GB_REQUIRE(epilogue != EPI_SILU_MUL || N % 2 == 0, "gemm_bf16: stacked gate/up rows need an even N, got %d", N);
   GB_REQUIRE(lda >= K && ldw >= K && ldc >= ncols, "gemm_bf16: a leading dimension is shorter than its row");
   GB_REQUIRE(((uintptr_t)a % 16 == 0) && ((uintptr_t)w % 16 == 0), "gemm_bf16: operands must be 16-byte aligned");
   GB_REQUIRE(epilogue != EPI_ACCUMULATE || c_dtype == kF32, "gemm_bf16: accumulation is into a float32 result");
-  GB_REQUIRE(epilogue != EPI_SILU_MUL || M <= 64, "gemm_bf16: the fused SiLU-multiply serves up to 64 rows, got %d", M);
   GB_REQUIRE(c_dtype == kF32 || c_dtype == kBF16, "gemm_bf16: unknown result dtype %d", c_dtype);
+  GB_REQUIRE(!gamma || (M <= 64 && c_dtype == kBF16 && epilogue != EPI_ACCUMULATE && ((uintptr_t)gamma % 16 == 0) &&
+                        (gamma_dtype == kF32 || gamma_dtype == kBF16)),
+             "gemm_bf16: the fused RMS norm serves up to 64 rows with a bfloat16 result");
   if (M == 0) return 0;
-  const bf16* A = (const bf16*)a;
   const bf16* W = (const bf16*)w;
   if (M <= 64) {
-#define GB_SK(EPI, CT) return launch_skinny<EPI, CT>(A, lda, W, ldw, (CT*)c, ldc, M, N, K, stream)
+    const int gf = gamma_dtype == kF32;
+    if (gamma) {
+      if (epilogue == EPI_STORE) return launch_skinny<EPI_STORE, true, bf16>(a, lda, W, ldw, (bf16*)c, ldc, M, N, K, gamma, gf, eps, stream);
+      return launch_skinny<EPI_SILU_MUL, true, bf16>(a, lda, W, ldw, (bf16*)c, ldc, M, N, K, gamma, gf, eps, stream);
+    }
+#define GB_SK(EPI, CT) return launch_skinny<EPI, false, CT>(a, lda, W, ldw, (CT*)c, ldc, M, N, K, nullptr, 0, 0.f, stream)
     if (epilogue == EPI_STORE && c_dtype == kF32) GB_SK(EPI_STORE, float);
     if (epilogue == EPI_STORE && c_dtype == kBF16) GB_SK(EPI_STORE, bf16);
     if (epilogue == EPI_ACCUMULATE) GB_SK(EPI_ACCUMULATE, float);
@@ -336,12 +493,12 @@ extern "C" int gb_gemm_bf16(const void* a, int lda, const void* w, int ldw, void
     GB_SK(EPI_SILU_MUL, bf16);
 #undef GB_SK
   }
-  const dim3 grid((N + TBN - 1) / TBN, (M + TBM - 1) / TBM), block(256);
-  GB_REQUIRE(grid.y <= 65535, "gemm_bf16: M=%d needs more than 65535 row tiles", M);
-  if (c_dtype == kF32)
-    hipLaunchKernelGGL(gemm_tiled_kernel<float>, grid, block, 0, stream, A, lda, W, ldw, (float*)c, ldc, M, N, K,
-                       epilogue == EPI_ACCUMULATE);
-  else
-    hipLaunchKernelGGL(gemm_tiled_kernel<bf16>, grid, block, 0, stream, A, lda, W, ldw, (bf16*)c, ldc, M, N, K, 0);
-  return launched("gemm_bf16 (tiled)");
+  const bf16* A = (const bf16*)a;
+#define GB_TL(EPI, CT) return launch_tiled<EPI, CT>(A, lda, W, ldw, (CT*)c, ldc, M, N, K, stream)
+  if (epilogue == EPI_ACCUMULATE) GB_TL(EPI_ACCUMULATE, float);
+  if (epilogue == EPI_SILU_MUL && c_dtype == kBF16) GB_TL(EPI_SILU_MUL, bf16);
+  if (epilogue == EPI_SILU_MUL) GB_TL(EPI_SILU_MUL, float);
+  if (c_dtype == kF32) GB_TL(EPI_STORE, float);
+  GB_TL(EPI_STORE, bf16);
+#undef GB_TL
 }

@@ -54,6 +54,9 @@ class StepContext:
         #: the same metadata as Python lists, for kernel selection and for parts written in Python
         self.host = host
         self.attention_impl = attention_impl
+        #: whether norms may be computed inside the next matrix product (steps of few rows); "plain" turns
+        #: every fusion off, so that tests can compare the fused kernels with their separate twins
+        self.fuse_norms = attention_impl != "plain"
         self.memo: dict = {}
 
     def buffer(self, name: str, shape, dtype) -> torch.Tensor:

@@ -49,8 +49,8 @@ _SIGS = {
         "gb_gemm_f32": [_vp, _i, _vp, _i, _vp, _i, _i, _i, _i, _i, _vp],
     },
     "gemm_bf16": {
-        # a, lda, w, ldw, c, ldc, c_dtype, M, N, K, epilogue, stream
-        "gb_gemm_bf16": [_vp, _i, _vp, _i, _vp, _i, _i, _i, _i, _i, _i, _vp],
+        # a, lda, w, ldw, c, ldc, c_dtype, M, N, K, epilogue, gamma, gamma_dtype, eps, stream
+        "gb_gemm_bf16": [_vp, _i, _vp, _i, _vp, _i, _i, _i, _i, _i, _i, _vp, _i, _f, _vp],
     },
     "attention_plain": {
         "gb_attention_plain": [_vp, _i, _vp, _i, _i, _vp, _vp, _vp, _i, _vp, _vp, _i, _i, _i, _i, _i, _f, _i, _vp],
@@ -232,22 +232,36 @@ def copy_rows(base: torch.Tensor, src: torch.Tensor, dst: torch.Tensor) -> None:
 SILU_MUL_MAX_ROWS = 64
 
 
-def gemm(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor, accumulate: bool = False, silu_mul: bool = False) -> None:
+FUSED_NORM_MAX_ROWS = 16   # measured: beyond one 16-row block the re-reading of float32 rows costs more than a norm pass
+
+
+def gemm(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor, accumulate: bool = False, silu_mul: bool = False,
+         rms: Optional[tuple] = None) -> None:
     """out (+)= a . w^T with w in the [out features, in features] layout.
     float32 operands take the true 32-bit kernel; bfloat16 operands the matrix-core kernels,
     with out in bfloat16 or float32 (float32 when accumulating into the residual).
     ``silu_mul`` (bfloat16, at most 64 rows): w stacks gate rows over up rows and out[m, j] =
-    silu(a . gate_j) * (a . up_j), of half as many columns."""
+    silu(a . gate_j) * (a . up_j), of half as many columns.
+    ``rms=(gamma, eps)`` (bfloat16 w and out, at most 64 rows): a is the float32 residual and the
+    product is that of its RMS-normed rows, the norm computed inside the product's kernel."""
     _dev(a, w, out)
     M, K = a.shape
     N = w.shape[0]
     if w.shape[1] != K or out.shape != (M, N // 2 if silu_mul else N):
         raise KernelError(f"gemm: shapes do not match: a {tuple(a.shape)}, w {tuple(w.shape)}, out {tuple(out.shape)}")
-    if silu_mul and (a.dtype != torch.bfloat16 or M > SILU_MUL_MAX_ROWS or accumulate or N % 16):
-        raise KernelError("gemm: the fused SiLU-multiply takes bfloat16 operands, at most 64 rows and gate/up "
-                          "stacks of a multiple of 8 rows each")
+    if silu_mul and (w.dtype != torch.bfloat16 or accumulate or N % 16):
+        raise KernelError("gemm: the fused SiLU-multiply takes bfloat16 operands and gate/up stacks of a "
+                          "multiple of 8 rows each")
     lda, ldw, ldc = _rows(a, "a"), _rows(w, "w"), _rows(out, "out")
-    if a.dtype == torch.float32 and w.dtype == torch.float32:
+    if rms is not None:
+        gamma, eps = rms
+        if (a.dtype != torch.float32 or w.dtype != torch.bfloat16 or out.dtype != torch.bfloat16 or accumulate
+                or M > 64 or gamma.numel() != K or not gamma.is_contiguous()):
+            raise KernelError("gemm: the fused RMS norm takes float32 rows (at most 64), bfloat16 weights and result")
+        lib = _lib("gemm_bf16")
+        _check(lib, lib.gb_gemm_bf16(_p(a), lda, _p(w), ldw, _p(out), ldc, BF16, M, N, K, 2 if silu_mul else 0,
+                                     _p(gamma), dtype_code(gamma), float(eps), _stream()))
+    elif a.dtype == torch.float32 and w.dtype == torch.float32:
         if out.dtype != torch.float32:
             raise KernelError("gemm: 32-bit operands need a 32-bit result")
         lib = _lib("gemm_f32")
@@ -257,7 +271,7 @@ def gemm(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor, accumulate: bool =
             raise KernelError("gemm: accumulation is into a 32-bit result")
         lib = _lib("gemm_bf16")
         _check(lib, lib.gb_gemm_bf16(_p(a), lda, _p(w), ldw, _p(out), ldc, dtype_code(out), M, N, K,
-                                     2 if silu_mul else (1 if accumulate else 0), _stream()))
+                                     2 if silu_mul else (1 if accumulate else 0), None, 0, 0.0, _stream()))
     else:
         raise KernelError(f"gemm: operand types {a.dtype} and {w.dtype} do not match a kernel")
 

@@ -54,13 +54,16 @@ class PagedAttention(Mixer):
             self.wqkv = torch.cat([tensors["q_proj.weight"], tensors["k_proj.weight"], tensors["v_proj.weight"]], 0)
         self.wo = tensors["o_proj.weight"].contiguous()
 
-    def forward(self, ctx, h, residual, cache: Optional[LayerCache]):
+    accepts_fused_norm = True
+
+    def forward(self, ctx, h, residual, cache: Optional[LayerCache], norm=None):
+        """``norm=(gamma, eps)``: h is the un-normed float32 residual and the first product norms it."""
         if cache is None or cache.k_pages is None:
             raise ValueError("PagedAttention needs a layer cache with pages")
         n = h.shape[0]
         rows = self.q_dim + (0 if self.shares_kv else 2 * self.kv_dim)
         qkv = ctx.buffer("qkv", (n, rows), ctx.dtype)
-        ops.gemm(h, self.wqkv, qkv)
+        ops.gemm(h, self.wqkv, qkv, rms=norm)
         write = cache.writable and not self.shares_kv
         self.position.apply_and_store(
             ctx, qkv, self.n_heads, 0 if self.shares_kv else self.n_kv_heads, self.head_dim,

@@ -97,6 +97,11 @@ class Norm(Part):
     def forward(self, ctx, x: torch.Tensor, rows: Optional[torch.Tensor] = None, out_name: str = "h") -> torch.Tensor:
         raise NotImplementedError
 
+    def fuse_spec(self, ctx, n: int):
+        """What a following part needs to compute this norm inside its first matrix product, or None
+        (the default) if the norm wants a pass of its own."""
+        return None
+
 
 class PositionEncoding(Part):
     def apply_and_store(self, ctx, qkv, n_heads, n_kv_heads, head_dim, slots, k_pages, v_pages) -> None:

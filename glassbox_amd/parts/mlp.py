@@ -25,13 +25,20 @@ class SwiGLU(FeedForward):
         self.w_gate_up = torch.cat([tensors["gate_proj.weight"], tensors["up_proj.weight"]], 0)
         self.w_down = tensors["down_proj.weight"].contiguous()
 
-    def forward(self, ctx, h, residual):
+    accepts_fused_norm = True
+
+    def forward(self, ctx, h, residual, norm=None):
+        """``norm=(gamma, eps)``: h is the un-normed float32 residual and the first product norms it."""
         n = h.shape[0]
         act = ctx.buffer("act", (n, self.intermediate), ctx.dtype)
-        if h.dtype == torch.bfloat16 and n <= ops.SILU_MUL_MAX_ROWS and self.intermediate % 8 == 0:
-            # few rows (decoding): the activation is applied where the product's tile is finished
-            ops.gemm(h, self.w_gate_up, act, silu_mul=True)
+        if ctx.dtype == torch.bfloat16 and self.intermediate % 8 == 0:
+            # the activation is applied where the product's tile is finished: gate_up never reaches memory
+            ops.gemm(h, self.w_gate_up, act, silu_mul=True, rms=norm)
         else:
+            if norm is not None:   # nothing to fuse it into here: the norm gets its own pass after all
+                normed = ctx.buffer("h", (n, self.width), ctx.dtype)
+                ops.rmsnorm(h, norm[0], norm[1], normed)
+                h = normed
             gate_up = ctx.buffer("gate_up", (n, 2 * self.intermediate), ctx.dtype)
             ops.gemm(h, self.w_gate_up, gate_up)
             ops.silu_mul(gate_up, act)

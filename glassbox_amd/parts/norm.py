@@ -2,7 +2,7 @@
 (crates/glassbox-core/src/model.rs:94-100)."""
 from __future__ import annotations
 
-from typing import Dict, Optional
+from typing import Dict, Optional, Tuple
 
 import torch
 
@@ -27,3 +27,10 @@ class RMSNorm(Norm):
         out = ctx.buffer(out_name, (m, self.width), ctx.dtype)
         ops.rmsnorm(x, self.weight, self.eps, out, rows)
         return out
+
+    def fuse_spec(self, ctx, n: int) -> Optional[Tuple[torch.Tensor, float]]:
+        """(gamma, eps) if the next matrix product may compute this norm itself: bfloat16 steps of
+        few rows, where a pass of its own costs more than the norm's arithmetic."""
+        if ctx.dtype == torch.bfloat16 and n <= ops.FUSED_NORM_MAX_ROWS and ctx.fuse_norms:
+            return (self.weight, self.eps)
+        return None

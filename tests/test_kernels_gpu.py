@@ -57,7 +57,9 @@ def test_gemm_bf16(N, K, M, out):
     assert (got - want).abs().max().item() <= tol
 
 
-@pytest.mark.parametrize("I,K,M", [(8, 32, 1), (176, 64, 5), (144, 80, 16), (200, 2048, 17), (8192, 2048, 8), (88, 4104, 64)])
+@pytest.mark.parametrize("I,K,M", [(8, 32, 1), (176, 64, 5), (144, 80, 16), (200, 2048, 17), (8192, 2048, 8), (88, 4104, 64),
+                                   # more than 64 rows: the tiled kernel's epilogue
+                                   (176, 64, 130), (72, 264, 65), (1024, 520, 300)])
 def test_gemm_bf16_fused_silu_mul(I, K, M):
     """Stacked gate/up rows with the activation applied in the product's epilogue
     (crates/glassbox-core/src/model.rs:335-340), against the formula in float64."""
@@ -75,6 +77,38 @@ def test_gemm_bf16_fused_silu_mul(I, K, M):
     out2 = torch.empty(M, I, device=DEV, dtype=torch.float32)
     ops.gemm(to_dev(a), to_dev(w), out2, silu_mul=True)
     assert torch.equal(out2, out)
+
+
+@pytest.mark.parametrize("N,K,M,silu", [(96, 64, 1, False), (6144, 2048, 8, False), (352, 176, 5, True),
+                                        (16384, 2048, 8, True), (480, 80, 33, False), (512, 4104, 64, True)])
+@pytest.mark.parametrize("gamma_dtype", [torch.float32, torch.bfloat16])
+def test_gemm_bf16_fused_rms_norm(N, K, M, silu, gamma_dtype):
+    """The product that norms its float32 rows on the way, against norm-then-product in float64
+    (crates/glassbox-core/src/model.rs:94-100 and 260 / 335)."""
+    from glassbox_amd import ops
+    x = rnd(M, K, seed=1, scale=3.0).float()
+    x[0] *= 1e-3                                              # a row where eps matters
+    g = (rnd(K, seed=2) * 0.3 + 1.0).to(gamma_dtype)
+    w = (rnd(N, K, seed=3) / math.sqrt(K)).bfloat16()
+    eps = 1e-5
+    h = g.double() * (x.double() * torch.rsqrt(x.double().pow(2).mean(-1, keepdim=True) + eps))
+    prod = h @ w.double().T
+    if silu:
+        gate, up = prod[:, :N // 2], prod[:, N // 2:]
+        want = gate / (1 + torch.exp(-gate)) * up
+    else:
+        want = prod
+    out = torch.full(want.shape, 9.0, device=DEV, dtype=torch.bfloat16)
+    ops.gemm(to_dev(x), to_dev(w), out, silu_mul=silu, rms=(to_dev(g), eps))
+    # bf16(g * x) as the operand: one rounding per element, 2^-9 relative, averaged over k
+    tol = (2 ** -7) * want.abs().max().item() + 1e-3
+    assert (out.cpu().double() - want).abs().max().item() <= tol
+    # the unfused pair of kernels rounds elsewhere (bf16(g * x * s) as the operand) and is as close
+    hn = torch.empty(M, K, device=DEV, dtype=torch.bfloat16)
+    ops.rmsnorm(to_dev(x), to_dev(g), eps, hn)
+    two = torch.empty_like(out)
+    ops.gemm(hn, to_dev(w), two, silu_mul=silu)
+    assert (two.cpu().double() - want).abs().max().item() <= tol
 
 
 def test_gemm_bf16_split_k_is_the_same_on_every_run():
