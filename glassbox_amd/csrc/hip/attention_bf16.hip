@@ -1,10 +1,9 @@
 // Paged attention in bfloat16 on the matrix cores, for decoding and for prompt portions.
 //
-// Per request and kv head the work is out[col] = softmax(q[col] . K^T * scale) . V for up to 16
-// "columns" that share the keys: when decoding, the columns are the query heads of one token that
-// map to the kv head (grouped-query attention reads each key once for the whole group); for a
-// prompt portion they are 16 consecutive tokens of one query head.  Both use the same inner step
-// over 64 keys:
+// Per request and kv head the work is out[col] = softmax(q[col] . K^T * scale) . V for "columns"
+// that share the keys.  When decoding, the columns are the up to 16 query heads of one token that
+// map to the kv head (grouped-query attention reads each key once for the whole group), and the
+// inner step over 64 keys is:
 //   S^T[key, col] = K[key, :] . Q[col, :]     v_mfma_f32_16x16x32_bf16, A = 16 keys x 32 dims straight
 //                                             from the key page (16 bytes a lane), B = the query columns
 //   running max / sum per column in 32-bit, keys outside [lo, hi] of the column masked to -inf
@@ -14,6 +13,8 @@
 //                                             are (the k order of both operands is permuted alike)
 // so neither scores nor probabilities pass through LDS, and keys and values go from memory into
 // MFMA operands directly.  Pages: keys [page][kv head][slot][hd], values [page][kv head][hd][slot].
+// A prompt portion's columns are 32 or 64 consecutive tokens of one query head, with the same
+// scheme on the 32x32x16 instruction (described at its kernel).
 //
 // Decoding splits a request's context into chunks of a multiple of 256 keys, one workgroup per
 // (chunk, kv head, request), four waves taking 64 keys each in turn; partial results are merged
@@ -232,53 +233,316 @@ __global__ void decode_reduce_kernel(const float* __restrict__ ws_acc, const flo
 }
 
 // ---------------------------------------------------------------------------- prefill
-// grid (tiles of 64 tokens, query heads, requests from seq_base on); a wave takes 16 tokens.
+// A wave takes blocks of 32 consecutive tokens of one query head; v_mfma_f32_32x32x16_bf16 throughout.
+// Per 64 keys:
+//   S^T[key, tok]   A = 32 keys x 16 dims (lane: key lane%32, dims 8*(lane/32)..+7 of the k-step),
+//                   B = the query tokens alike; the result lane holds token lane%32 and keys
+//                   8*(r/4) + 4*(lane/32) + r%4 of the 32-key tile
+//   O^T[dim, tok]   A = 32 dims x 16 keys from the transposed value page, B = probabilities: registers
+//                   8h..8h+7 of a score tile are, as they stand, the B operand of the k-step over keys
+//                   16h..16h+15 if slot e of lane group g means key 4g+e (e<4) or 8+4g+(e-4); the value
+//                   operand is loaded in that same order (two 8-byte loads a lane)
+// Scores stay raw in the registers; softmax works on exp2(raw*c - max*c) with c = scale*log2(e).
+// Causal work grows with the position, so a wave takes block i and block n-1-i of its request's
+// portion: every wave then has the same number of (token, key) pairs.  With QB == 2 both blocks are
+// live at once and share the key and value fragments where their key ranges overlap (ACT says
+// which are live in a step); with QB == 1 (head sizes whose accumulators leave no room) one after
+// the other.
+// Where a wave's key and value fragments come from.  Everything here is the same for all lanes of a
+// wave, so page lookups and page addresses are scalar work.
+struct PageSource {
+  const bf16* __restrict__ kp;
+  const bf16* __restrict__ vp;
+  const int32_t* __restrict__ table;
+  int nkv, kvh, shift;  // pages of 1 << shift keys
+  int tlo, thi;         // groups of 16 keys outside [tlo, thi] are redirected into it (their keys are masked anyway)
+  // offset, in elements of a page array of one kv head, of the page and slot that hold key k
+  __device__ __forceinline__ size_t page_of(int k, int* slot) const {
+    const int kc = min(max(k, tlo), thi);
+    *slot = kc & ((1 << shift) - 1);
+    return ((size_t)table[kc >> shift] * nkv + kvh);
+  }
+};
+
 template <int HD>
-__global__ __launch_bounds__(256) void prefill_kernel(const bf16* __restrict__ q, int q_stride, bf16* __restrict__ out,
+__device__ __forceinline__ void load_keys(bf16x8 (&kf)[2][HD / 16], const PageSource& src, int kbase, int lane) {
+  const int col = lane & 31, g = lane >> 5;
+  const int mine = (col & 15) * HD + 8 * g;
+#pragma unroll
+  for (int t = 0; t < 2; ++t) {
+    int s0, s1;  // a tile of 32 keys is two groups of 16, each within one page
+    const size_t p0 = src.page_of(kbase + 32 * t, &s0), p1 = src.page_of(kbase + 32 * t + 16, &s1);
+    const bf16* b0 = src.kp + ((p0 << src.shift) + s0) * HD;
+    const bf16* b1 = src.kp + ((p1 << src.shift) + s1) * HD;
+    const bf16* kb = ((col & 16) ? b1 : b0) + mine;
+#pragma unroll
+    for (int ks = 0; ks < HD / 16; ++ks) kf[t][ks] = load8(kb + 16 * ks);
+  }
+}
+
+template <int HD>
+__device__ __forceinline__ void load_values(bf16x8 (&vf)[(HD + 31) / 32][4], const PageSource& src, int kbase, int lane) {
+  const int col = lane & 31, g = lane >> 5;
+  const int mine = (col << src.shift) + 4 * g;
+#pragma unroll
+  for (int u = 0; u < 4; ++u) {
+    int slot;
+    const size_t pg = src.page_of(kbase + 16 * u, &slot);
+    const bf16* vb = src.vp + ((pg * HD) << src.shift) + slot + mine;
+#pragma unroll
+    for (int b = 0; b < (HD + 31) / 32; ++b) {
+      if (32 * b + 32 <= HD || 32 * b + col < HD) {
+        const bf16x4 a = load4(vb + ((size_t)(32 * b) << src.shift)), bb = load4(vb + ((size_t)(32 * b) << src.shift) + 8);
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          vf[b][u][e] = a[e];
+          vf[b][u][4 + e] = bb[e];
+        }
+      } else {
+        vf[b][u] = zero8();
+      }
+    }
+  }
+}
+
+// One step over the 64 keys from kbase, whose fragments kf and vf hold.  The live blocks take their
+// turn one after the other (scores, softmax, values), so that only one block's scores are in
+// registers at a time; as soon as the last block's score products have read kf it is loaded again
+// for the keys from `next`, and vf likewise after the last value products, so that those loads are
+// in flight during the arithmetic in between.
+template <int HD, int QB, int ACT>
+__device__ __forceinline__ void attend64_q32(float (&m)[QB], float (&l)[QB], f32x16 (&acc)[QB][(HD + 31) / 32],
+                                             const bf16x8* __restrict__ q_lds, int q_at, bf16x8 (&kf)[2][HD / 16],
+                                             bf16x8 (&vf)[(HD + 31) / 32][4], const PageSource& src, int kbase, int next,
+                                             const int (&lo)[QB], const int (&hi)[QB], bool mask, float c, int lane) {
+  constexpr int KS = HD / 16, DB = (HD + 31) / 32;
+  constexpr int LAST = (ACT & 2) ? 1 : 0;
+  const int g = lane >> 5;
+  // the compiler must not know that the query fragments are the same in every step, or it reads them
+  // once before the loop and has no registers to keep them in
+  asm volatile("" : "+v"(q_at));
+  const bf16x8* qf = q_lds + q_at;
+#pragma unroll
+  for (int qb = 0; qb < QB; ++qb) {
+    if (!((ACT >> qb) & 1)) continue;
+    f32x16 s[2];
+#pragma unroll
+    for (int t = 0; t < 2; ++t) {
+#pragma unroll
+      for (int r = 0; r < 16; ++r) s[t][r] = 0.f;
+#pragma unroll
+      for (int ks = 0; ks < KS; ++ks)
+        s[t] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf[t][ks], qf[(qb * KS + ks) * 64], s[t], 0, 0, 0);
+    }
+    if (qb == LAST) {
+      // not earlier: above the score products the old and the new fragments would both need registers
+      __builtin_amdgcn_sched_barrier(0);
+      load_keys<HD>(kf, src, next, lane);
+    }
+    if (mask) {  // the same for the whole wave
+#pragma unroll
+      for (int t = 0; t < 2; ++t)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+          const int key = kbase + 32 * t + 8 * (r >> 2) + 4 * g + (r & 3);
+          if (key < lo[qb] || key > hi[qb]) s[t][r] = -INFINITY;
+        }
+    }
+    float mx = -INFINITY;
+#pragma unroll
+    for (int t = 0; t < 2; ++t)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) mx = fmaxf(mx, s[t][r]);
+    mx = fmaxf(mx, __shfl_xor(mx, 32, kWave));
+    const float m_new = fmaxf(m[qb], mx);
+    const float m_ref = m_new == -INFINITY ? 0.f : m_new;  // a column with no key yet
+    const float alpha = m[qb] == -INFINITY ? 0.f : __builtin_amdgcn_exp2f((m[qb] - m_ref) * c);
+    const float mc = m_ref * c;
+    float sum = 0.f;
+#pragma unroll
+    for (int t = 0; t < 2; ++t)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) {
+        s[t][r] = __builtin_amdgcn_exp2f(fmaf(s[t][r], c, -mc));
+        sum += s[t][r];
+      }
+    l[qb] = l[qb] * alpha + sum;
+    m[qb] = m_new;
+    if (__any(alpha != 1.f)) {
+#pragma unroll
+      for (int b = 0; b < DB; ++b)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) acc[qb][b][r] *= alpha;
+    }
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+      bf16x8 pf;
+#pragma unroll
+      for (int e = 0; e < 8; ++e) pf[e] = (bf16)s[u >> 1][8 * (u & 1) + e];
+#pragma unroll
+      for (int b = 0; b < DB; ++b) acc[qb][b] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vf[b][u], pf, acc[qb][b], 0, 0, 0);
+    }
+  }
+  __builtin_amdgcn_sched_barrier(0);
+  load_values<HD>(vf, src, next, lane);
+}
+
+// What a wave knows of one block of 32 tokens: the keys [first, last] that any of its tokens sees, and
+// the keys [free_lo, free_hi] that all of them see (no mask needed there, if the block is whole).
+struct BlockRange {
+  int first, last, free_lo, free_hi;
+  bool whole;
+  __device__ bool live(int kb) const { return kb <= last && kb + 63 >= first; }
+  __device__ bool unmasked(int kb) const { return whole && kb >= free_lo && kb + 63 <= free_hi; }
+};
+
+__device__ __forceinline__ BlockRange block_range(int t0, int qlen, int p0, int window) {
+  BlockRange r;
+  const int t1 = min(t0 + 32, qlen) - 1;
+  r.whole = t0 + 32 <= qlen;
+  r.last = p0 + t1;
+  r.first = window > 0 ? max(0, p0 + t0 - window + 1) : 0;
+  r.free_hi = p0 + t0;
+  r.free_lo = window > 0 ? max(0, p0 + t1 - window + 1) : 0;
+  return r;
+}
+
+template <int HD>
+__device__ __forceinline__ void store_block(const f32x16 (&acc)[(HD + 31) / 32], float l, bf16* __restrict__ orow, int g) {
+  const float inv = 1.0f / l;
+#pragma unroll
+  for (int b = 0; b < (HD + 31) / 32; ++b)
+#pragma unroll
+    for (int jj = 0; jj < 4; ++jj) {
+      const int d0 = 32 * b + 8 * jj + 4 * g;
+      if (32 * b + 32 <= HD || d0 < HD) {
+        bf16x4 o;
+#pragma unroll
+        for (int r = 0; r < 4; ++r) o[r] = (bf16)(acc[b][4 * jj + r] * inv);
+        *reinterpret_cast<bf16x4*>(orow + d0) = o;
+      }
+    }
+}
+
+// grid (groups of four waves, query heads, requests from seq_base on); wave w of a request takes its
+// blocks w and n-1-w of 32 tokens.
+template <int HD, int QB>
+__global__ __launch_bounds__(256, 2) void prefill_kernel(const bf16* __restrict__ q, int q_stride, bf16* __restrict__ out,
                                                       int out_stride, const int32_t* __restrict__ q_start,
                                                       const int32_t* __restrict__ q_len, const int32_t* __restrict__ pos0,
                                                       int seq_base, const int32_t* __restrict__ tables, int table_stride,
                                                       const bf16* __restrict__ kp, const bf16* __restrict__ vp, int nh, int nkv,
-                                                      int P, float scale, int window) {
-  constexpr int KS = (HD + 31) / 32, DB = HD / 16;
-  const int seq = seq_base + blockIdx.z, head = blockIdx.y;
-  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+                                                      int page_shift, float scale, int window) {
+  constexpr int KS = HD / 16, DB = (HD + 31) / 32;
+  // Workgroups go to the chip's eight dies in turn, each die with an L2 of its own.  The ones that
+  // land on one die are given consecutive units of work, so that a head's keys and values, which all
+  // of its token groups read, are fetched into one L2 rather than eight.
+  constexpr int kDies = 8;
+  const int gx = gridDim.x, gy = gridDim.y, total = gx * gy * gridDim.z;
+  const int linear = blockIdx.x + gx * (blockIdx.y + gy * blockIdx.z);
+  const int die = linear % kDies;
+  const int unit = die * (total / kDies) + min(die, total % kDies) + linear / kDies;
+  const int seq = seq_base + unit / (gx * gy), head = unit / gx % gy, group = unit % gx;
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);  // the same in all lanes: what follows from it is scalar
   const int qlen = q_len[seq];
-  const int t0 = blockIdx.x * 64 + wave * 16;
-  if (t0 >= qlen) return;
-  const int col = lane & 15, c = lane >> 4;
-  const int tok = t0 + col;
-  const bool valid = tok < qlen;
+  const int blocks = (qlen + 31) / 32;
+  const int w = group * 4 + wave;
+  if (2 * w >= blocks) return;
+  const int col = lane & 31, g = lane >> 5;
   const int p0 = pos0[seq];
-  const int p = p0 + tok;
-  const size_t row = (size_t)q_start[seq] + tok;
   const int kvh = head / (nh / nkv);
-  const int32_t* table = tables + (size_t)seq * table_stride;
+  PageSource src{kp, vp, tables + (size_t)seq * table_stride, nkv, kvh, page_shift, 0, 0};
+  const size_t row0 = (size_t)q_start[seq];
+  const float c = scale * 1.4426950408889634f;
+  bf16x8 kf[2][KS];
+  bf16x8 vf[DB][4];
+  // The query fragments wait in LDS, each lane's own in a place of its own (no lane reads another's):
+  // they are needed once per step over 64 keys, and the registers are better spent on the accumulators.
+  __shared__ bf16x8 q_lds[4 * QB * KS * 64];
+  const int q_at = wave * (QB * KS * 64) + lane;
+  bf16x8* qf = q_lds + q_at;
+  // the wave's two blocks start at these tokens; the later one is absent when it is the earlier one itself
+  const int start[2] = {32 * w, 32 * (blocks - 1 - w)};
+  const bool has_second = blocks - 1 - w > w;
 
-  bf16x8 qf[KS];
+  if constexpr (QB == 2) {
+    int lo[2], hi[2];
+    float m[2], l[2];
+    f32x16 acc[2][DB];
+    BlockRange range[2];
 #pragma unroll
-  for (int ks = 0; ks < KS; ++ks) {
-    const int d0 = ks * 32 + c * 8;
-    qf[ks] = (valid && d0 < HD) ? load8(q + row * q_stride + (size_t)head * HD + d0) : zero8();
-  }
-  Running<HD> st;
-  reset(st);
-  const int col_lo = valid ? (window > 0 ? max(0, p - window + 1) : 0) : 1, col_hi = valid ? p : 0;
-  const int wave_hi = p0 + min(t0 + 15, qlen - 1);
-  const int wave_lo = window > 0 ? max(0, p0 + t0 - window + 1) : 0;
-  for (int kb = wave_lo & ~63; kb <= wave_hi; kb += 64)
-    attend64<HD>(st, qf, kp, vp, table, nkv, kvh, P, kb, col_lo, col_hi, wave_lo, wave_hi, scale, lane);
-  st.l += __shfl_xor(st.l, 16, kWave);
-  st.l += __shfl_xor(st.l, 32, kWave);
-  if (!valid) return;
-  const float inv = 1.0f / st.l;
-  bf16* orow = out + row * out_stride + (size_t)head * HD;
+    for (int qb = 0; qb < 2; ++qb) {
+      const int tok = start[qb] + col;
+      const bool valid = tok < qlen && (qb == 0 || has_second);
+      const int p = p0 + tok;
+      lo[qb] = valid ? (window > 0 ? max(0, p - window + 1) : 0) : 1;
+      hi[qb] = valid ? p : 0;
 #pragma unroll
-  for (int b = 0; b < DB; ++b) {
-    bf16x4 o;
+      for (int ks = 0; ks < KS; ++ks)
+        qf[(qb * KS + ks) * 64] = valid ? load8(q + (row0 + tok) * q_stride + (size_t)head * HD + 16 * ks + 8 * g) : zero8();
+      m[qb] = -INFINITY;
+      l[qb] = 0.f;
 #pragma unroll
-    for (int r = 0; r < 4; ++r) o[r] = (bf16)(st.acc[b][r] * inv);
-    *reinterpret_cast<bf16x4*>(orow + 16 * b + 4 * c) = o;
+      for (int b = 0; b < DB; ++b)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) acc[qb][b][r] = 0.f;
+      range[qb] = block_range(start[qb], qlen, p0, window);
+    }
+    const int end = has_second ? range[1].last : range[0].last;
+    src.tlo = range[0].first & ~15;
+    src.thi = end & ~15;
+    int kb = range[0].first & ~63;
+    load_keys<HD>(kf, src, kb, lane);
+    load_values<HD>(vf, src, kb, lane);
+    if (has_second) {
+      // both blocks as far as the earlier one's keys reach (with a window the later one may see none of
+      // them yet: they are masked), then the later block alone
+      while (kb <= range[0].last) {
+        int next = kb + 64;
+        if (next > range[0].last && next + 63 < range[1].first) next = range[1].first & ~63;
+        const bool mask = !(range[0].unmasked(kb) && range[1].unmasked(kb));
+        attend64_q32<HD, 2, 3>(m, l, acc, q_lds, q_at, kf, vf, src, kb, next, lo, hi, mask, c, lane);
+        kb = next;
+      }
+      for (; kb <= range[1].last; kb += 64)
+        attend64_q32<HD, 2, 2>(m, l, acc, q_lds, q_at, kf, vf, src, kb, kb + 64, lo, hi, !range[1].unmasked(kb), c, lane);
+    } else {
+      for (; kb <= range[0].last; kb += 64)
+        attend64_q32<HD, 2, 1>(m, l, acc, q_lds, q_at, kf, vf, src, kb, kb + 64, lo, hi, !range[0].unmasked(kb), c, lane);
+    }
+#pragma unroll
+    for (int qb = 0; qb < 2; ++qb) {
+      const float total = l[qb] + __shfl_xor(l[qb], 32, kWave);
+      const int tok = start[qb] + col;
+      if (tok >= qlen || (qb == 1 && !has_second)) continue;
+      store_block<HD>(acc[qb], total, out + (row0 + tok) * out_stride + (size_t)head * HD, g);
+    }
+  } else {
+    for (int which = 0; which < (has_second ? 2 : 1); ++which) {
+      const int tok = start[which] + col;
+      const bool valid = tok < qlen;
+      const int p = p0 + tok;
+      int lo[1] = {valid ? (window > 0 ? max(0, p - window + 1) : 0) : 1}, hi[1] = {valid ? p : 0};
+      float m[1] = {-INFINITY}, l[1] = {0.f};
+      f32x16 acc[1][DB];
+#pragma unroll
+      for (int ks = 0; ks < KS; ++ks)
+        qf[ks * 64] = valid ? load8(q + (row0 + tok) * q_stride + (size_t)head * HD + 16 * ks + 8 * g) : zero8();
+#pragma unroll
+      for (int b = 0; b < DB; ++b)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) acc[0][b][r] = 0.f;
+      const BlockRange range = block_range(start[which], qlen, p0, window);
+      src.tlo = range.first & ~15;
+      src.thi = range.last & ~15;
+      load_keys<HD>(kf, src, range.first & ~63, lane);
+      load_values<HD>(vf, src, range.first & ~63, lane);
+      for (int kb = range.first & ~63; kb <= range.last; kb += 64)
+        attend64_q32<HD, 1, 1>(m, l, acc, q_lds, q_at, kf, vf, src, kb, kb + 64, lo, hi, !range.unmasked(kb), c, lane);
+      const float total = l[0] + __shfl_xor(l[0], 32, kWave);
+      if (valid) store_block<HD>(acc[0], total, out + (row0 + tok) * out_stride + (size_t)head * HD, g);
+    }
   }
 }
 
@@ -328,17 +592,20 @@ extern "C" int gb_attention_prefill_bf16(const void* q, int q_stride, void* out,
                                          int nh, int nkv, int hd, int page_size, float scale, int window, hipStream_t stream) {
   GB_REQUIRE(n_seqs >= 0 && nh > 0 && nkv > 0 && nh % nkv == 0, "attention_prefill: bad head counts nh=%d nkv=%d", nh, nkv);
   GB_REQUIRE(gb_attention_supported_head_size(hd), "attention_prefill: head size %d is not a multiple of 16 up to 128", hd);
-  GB_REQUIRE(page_size >= 16 && page_size % 16 == 0, "attention_prefill: page size %d is not a multiple of 16", page_size);
+  GB_REQUIRE(page_size >= 16 && (page_size & (page_size - 1)) == 0, "attention_prefill: page size %d is not a power of two from 16 up", page_size);
+  int page_shift = 4;
+  while ((1 << page_shift) < page_size) ++page_shift;
   GB_REQUIRE(q_stride % 8 == 0 && ((uintptr_t)q % 16 == 0) && out_stride % 4 == 0 && ((uintptr_t)out % 8 == 0),
              "attention_prefill: q rows must be 16-byte aligned and out rows 8-byte aligned");
   GB_REQUIRE(n_seqs <= 65535 && nh <= 65535, "attention_prefill: too many requests or heads for one launch");
   if (n_seqs == 0 || max_q_len <= 0) return 0;
-  const dim3 grid((max_q_len + 63) / 64, nh, n_seqs), block(256);
+  // a wave takes two blocks of 32 tokens, a workgroup four waves
+  const dim3 grid((max_q_len + 255) / 256, nh, n_seqs), block(256);
 #define GB_CASE(HD)                                                                                                        \
   if (hd == HD)                                                                                                            \
-    hipLaunchKernelGGL(prefill_kernel<HD>, grid, block, 0, stream, (const bf16*)q, q_stride, (bf16*)out, out_stride,        \
-                       q_start, q_len, pos0, seq_base, tables, table_stride, (const bf16*)k_pages, (const bf16*)v_pages, nh, \
-                       nkv, page_size, scale, window);
+    hipLaunchKernelGGL((prefill_kernel<HD, (HD <= 64 ? 2 : 1)>), grid, block, 0, stream, (const bf16*)q, q_stride,          \
+                       (bf16*)out, out_stride, q_start, q_len, pos0, seq_base, tables, table_stride, (const bf16*)k_pages, \
+                       (const bf16*)v_pages, nh, nkv, page_shift, scale, window);
   GB_FOR_HEAD_SIZES(GB_CASE)
 #undef GB_CASE
   return launched("attention_prefill");

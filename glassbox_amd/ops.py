@@ -301,10 +301,10 @@ def attention_plain(q: torch.Tensor, out: torch.Tensor, positions: torch.Tensor,
 
 def tuned_attention_supports(k_pages: torch.Tensor, n_heads: int, window: int) -> bool:
     """Whether the matrix-core attention kernels take this layer: bfloat16 pages, a head size that is
-    a multiple of 16 up to 128, at most 16 query heads per kv head, pages of a multiple of 16."""
+    a multiple of 16 up to 128, at most 16 query heads per kv head, pages of 16, 32, 64 ... keys."""
     _, nkv, page, hd = k_pages.shape
     return (k_pages.dtype == torch.bfloat16 and hd % 16 == 0 and 16 <= hd <= 128 and n_heads % nkv == 0
-            and n_heads // nkv <= 16 and page % 16 == 0)
+            and n_heads // nkv <= 16 and page >= 16 and page & (page - 1) == 0)
 
 
 def decode_chunk(n_decode: int, n_kv_heads: int, max_context: int) -> int:

@@ -363,6 +363,37 @@ def test_tuned_attention_against_the_plain_kernel(nh, nkv, hd, window, page):
     assert ((out.float() - twin.float()).abs() <= 2 ** -7 * (1 + twin.float().abs())).all()
 
 
+@pytest.mark.parametrize("nh,nkv,hd,window", [(32, 32, 64, 0), (32, 8, 48, 0), (32, 4, 16, 100), (32, 32, 64, 200),
+                                              (32, 16, 32, 0)])
+def test_tuned_prefill_long_portions(nh, nkv, hd, window):
+    """Portions long enough, and heads enough, that a wave takes 64 tokens: one portion starts in the
+    middle of its request and ends off every tile edge, the other is a whole short prompt."""
+    from types import SimpleNamespace
+    from glassbox_amd import ops
+    q_lens, ctx_lens = [1101, 300], [1303, 300]
+    k_pages, v_pages, tables, ks, vs = paged_setup(ctx_lens, nkv, hd, 16, seed=hd + nh, dtype=torch.bfloat16)
+    ctx = BareContext(q_lens, ctx_lens, tables)
+    n = sum(q_lens)
+    q = (rnd(n, nh * hd, seed=12) * 0.7).bfloat16()
+    scale = 1 / math.sqrt(hd)
+    cache = SimpleNamespace(k_pages=to_dev(k_pages), v_pages=to_dev(v_pages), group=0)
+    out = torch.zeros(n, nh * hd, device=DEV, dtype=torch.bfloat16)
+    qd = to_dev(q)
+    ops.attention_prefill(qd, out, ctx, cache, nh, scale, window)
+    twin = torch.zeros_like(out)
+    ops.attention_plain(qd, twin, ctx.positions, torch.tensor(ctx.tok_seq, dtype=torch.int32, device=DEV), ctx.tables[0],
+                        cache.k_pages, cache.v_pages, nh, scale, window)
+    close = (out.float() - twin.float()).abs() <= 2 ** -7 * (1 + twin.float().abs())
+    bad = torch.nonzero(~close.all(dim=1)).flatten().tolist()
+    assert not bad, f"rows {bad[:8]} (request, position) {[(ctx.tok_seq[i], ctx.pos_list[i]) for i in bad[:8]]}"
+    # a sample of rows against the formula in float64: tile edges, the portion's ends, the second request
+    rows = [0, 1, 31, 32, 63, 64, 127, 128, 255, 256, 257, 700, 1023, 1024, 1099, 1100, 1101, 1102, 1400]
+    want = plain_attention_rows(q[rows], ks, vs, [ctx.tok_seq[i] for i in rows], [ctx.pos_list[i] for i in rows], nh,
+                                scale, window)
+    err = (out[rows].cpu().double() - want).abs().max().item()
+    assert err < 2 ** -6, err
+
+
 def test_tuned_decode_finds_one_far_key_in_every_chunk_position():
     """One key is made to stand out: first and last slot of a page, chunk edges, the last position."""
     from types import SimpleNamespace
@@ -385,29 +416,31 @@ def test_tuned_decode_finds_one_far_key_in_every_chunk_position():
             assert (out.cpu().float()[0] - want).abs().max().item() < 2e-2, f"key at {target} was not found"
 
 
-def test_tuned_prefill_sees_exactly_the_causal_keys():
-    """A portion in the middle of a request: token t must find a marked key at its own position and
-    must not see the one after it."""
+@pytest.mark.parametrize("nh,ctxlen,qlen", [(2, 200, 90), (64, 1200, 1090)])   # 32 and 64 tokens a wave
+def test_tuned_prefill_sees_exactly_the_causal_keys(nh, ctxlen, qlen):
+    """A portion in the middle of a request (it starts at position 110): token t must find a marked
+    key at its own position and must not see the one after it."""
     from types import SimpleNamespace
     from glassbox_amd import ops
-    nh, nkv, hd, page = 2, 2, 64, 16
-    ctxlen, qlen = 200, 90                                     # the portion covers positions 110..199
+    nkv, hd, page = 2, 64, 16
     k_pages, v_pages, tables, ks, vs = paged_setup([ctxlen], nkv, hd, page, seed=3, dtype=torch.bfloat16)
     ctx = BareContext([qlen], [ctxlen], tables)
-    g = torch.Generator().manual_seed(5)
-    direction = torch.randn(hd, generator=g)
-    direction /= direction.norm()
-    # every key points along `direction` with a length that grows with its position: the newest visible key wins
+    # every key lies along one axis with a length that grows with its position, through consecutive
+    # bfloat16 numbers from 16.0 on (so that rounding cannot reorder them): the newest visible key wins
+    lengths = (torch.arange(ctxlen, dtype=torch.int32) + 0x4180).to(torch.int16).view(torch.bfloat16)
+    axis = torch.zeros(hd)
+    axis[5] = 1.0
     kp = k_pages.clone()
     for p in range(ctxlen):
-        kp[tables[0, p // page], :, p % page, :] = (direction * (1 + p)).bfloat16()
-    q = (direction * 120).repeat(qlen, nh).bfloat16()
+        kp[tables[0, p // page], :, p % page, :] = (axis * lengths[p].float()).bfloat16()
+    q = (axis * 768).repeat(qlen, nh).bfloat16()             # neighbours differ by 12 and more in score
     out = torch.zeros(qlen, nh * hd, device=DEV, dtype=torch.bfloat16)
     cache = SimpleNamespace(k_pages=to_dev(kp), v_pages=to_dev(v_pages), group=0)
     ops.attention_prefill(to_dev(q), out, ctx, cache, nh, 1 / math.sqrt(hd), 0)
-    for t in range(qlen):
-        want = vs[0][110 + t].float().reshape(-1)             # not the value of position 111 + t
-        assert (out.cpu().float()[t] - want).abs().max().item() < 3e-2, f"token {t} of the portion"
+    got = out.cpu().float().reshape(qlen, nkv, nh // nkv, hd)
+    want = vs[0][110:110 + qlen].float()[:, :, None, :]      # not the value of the position after it
+    worst = (got - want).abs().amax(dim=(1, 2, 3))
+    assert worst.max().item() < 3e-2, f"token {int(worst.argmax())} of the portion"
 
 
 def test_copy_rows():
