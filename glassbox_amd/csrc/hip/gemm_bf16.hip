@@ -13,6 +13,8 @@
 //    through LDS in a fixed order; it can norm float32 rows on the way and apply the SiLU-multiply.
 // In both, every output cell is summed in an order fixed by (K, kernel) alone, not by M or by
 // the cell's neighbours.  C is bfloat16 or float32; accumulation (+=) is into float32.
+#include <type_traits>
+
 #include "common.h"
 
 using namespace gb;
@@ -47,8 +49,8 @@ constexpr int TBK = 64, TLD = TBK + 8;  // k-step; LDS row stride in elements (1
 constexpr int TCPR = TBK / 8;           // 16-byte chunks per row of a k-step
 constexpr int TKS = TBK / 16;           // MFMA k-steps per LDS k-step
 
-template <int WM, int WN, int EPI, typename CT>
-__global__ __launch_bounds__(256) void gemm_tiled_kernel(const bf16* __restrict__ a, int lda, const bf16* __restrict__ w,
+template <int WM, int WN, int DEPTH, int EPI, bool KFULL, typename CT>
+__global__ __launch_bounds__(256, WN == 2 ? 2 : 1) void gemm_tiled_kernel(const bf16* __restrict__ a, int lda, const bf16* __restrict__ w,
                                                          int ldw, CT* __restrict__ c, int ldc, int M, int N, int K) {
   constexpr int BM = 64 * WM, BN = 64 * WN;
   constexpr int CA = BM * TCPR / 256, CW = BN * TCPR / 256;  // chunks a thread moves per k-step
@@ -77,75 +79,118 @@ __global__ __launch_bounds__(256) void gemm_tiled_kernel(const bf16* __restrict_
 #pragma unroll
       for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
 
-  bf16x8 ga[CA], gw[CW];
-  const bf16* asrc[CA];
-  const bf16* wsrc[CW];
+  // Chunks on their way from memory to LDS wait in registers, DEPTH k-steps' worth: a load has DEPTH
+  // k-steps of arithmetic to arrive in before its registers are written to LDS.  Within a k-step the
+  // LDS writes and the loads that refill their registers are spread over the first three of the four
+  // MFMA steps, so that memory requests and arithmetic are issued side by side, not in bursts.
+  // Rows beyond M or N are read from a row that exists (their results are never stored), so that the
+  // loop has no branch around a load.
+  constexpr int CT_ = CA + CW;
+  bf16x8 held[DEPTH][CT_];
+  const bf16* src[CT_];
 #pragma unroll
-  for (int j = 0; j < CA; ++j) {
-    const int row = m0 + (tid + 256 * j) / TCPR;
-    asrc[j] = row < M ? a + (size_t)row * lda : nullptr;
-  }
-#pragma unroll
-  for (int j = 0; j < CW; ++j) {
-    const int row = w_row((tid + 256 * j) / TCPR);
-    wsrc[j] = row >= 0 ? w + (size_t)row * ldw : nullptr;
-  }
-  auto fetch = [&](int k0) {
-#pragma unroll
-    for (int j = 0; j < CA; ++j) {
-      const int gk = k0 + ((tid + 256 * j) % TCPR) * 8;
-      ga[j] = (asrc[j] && gk < K) ? load8(asrc[j] + gk) : zero8();
+  for (int ci = 0; ci < CT_; ++ci) {
+    const int ch = tid + 256 * (ci < CA ? ci : ci - CA);
+    if (ci < CA) {
+      src[ci] = a + (size_t)min(m0 + ch / TCPR, M - 1) * lda + (ch % TCPR) * 8;
+    } else {
+      src[ci] = w + (size_t)max(w_row(ch / TCPR), 0) * ldw + (ch % TCPR) * 8;
     }
-#pragma unroll
-    for (int j = 0; j < CW; ++j) {
-      const int gk = k0 + ((tid + 256 * j) % TCPR) * 8;
-      gw[j] = (wsrc[j] && gk < K) ? load8(wsrc[j] + gk) : zero8();
+  }
+  auto fetch = [&](int ci, int k0, auto set) {
+    if constexpr (KFULL) {
+      held[decltype(set)::value][ci] = load8(src[ci] + k0);
+    } else {
+      const int ch = tid + 256 * (ci < CA ? ci : ci - CA);
+      held[decltype(set)::value][ci] = k0 + (ch % TCPR) * 8 < K ? load8(src[ci] + k0) : zero8();
     }
   };
-  auto stash = [&](int buf) {
-#pragma unroll
-    for (int j = 0; j < CA; ++j) {
-      const int ch = tid + 256 * j;
-      *reinterpret_cast<bf16x8*>(&As[buf][ch / TCPR][(ch % TCPR) * 8]) = ga[j];
-    }
-#pragma unroll
-    for (int j = 0; j < CW; ++j) {
-      const int ch = tid + 256 * j;
-      *reinterpret_cast<bf16x8*>(&Ws[buf][ch / TCPR][(ch % TCPR) * 8]) = gw[j];
-    }
+  auto stash = [&](int ci, int buf, auto set) {
+    const int ch = tid + 256 * (ci < CA ? ci : ci - CA);
+    bf16* dst = ci < CA ? &As[buf][ch / TCPR][(ch % TCPR) * 8] : &Ws[buf][ch / TCPR][(ch % TCPR) * 8];
+    *reinterpret_cast<bf16x8*>(dst) = held[decltype(set)::value][ci];
   };
+  using Set0 = std::integral_constant<int, 0>;
+  using Set1 = std::integral_constant<int, 1>;
+  using Yes = std::true_type;
+  using No = std::false_type;
 
-  fetch(0);
-  stash(0);
-  __syncthreads();
   const int steps = (K + TBK - 1) / TBK;
   const int arow = wm * 32 * WM + lane % 32, wrow = wn * 32 * WN + lane % 32, koff = 8 * (lane / 32);
-  for (int s = 0; s < steps; ++s) {
+  bf16x8 fa[2][WM], fw[2][WN];  // operands of MFMA step ks+1 are read from LDS while the MFMAs of step ks run
+  auto read_operands = [&](int buf, int kk, int into) {
+#pragma unroll
+    for (int i = 0; i < WM; ++i) fa[into][i] = *reinterpret_cast<const bf16x8*>(&As[buf][arow + i * 32][kk * 16 + koff]);
+#pragma unroll
+    for (int j = 0; j < WN; ++j) fw[into][j] = *reinterpret_cast<const bf16x8*>(&Ws[buf][wrow + j * 32][kk * 16 + koff]);
+  };
+  // k-step s is computed from LDS buffer s % 2.  Register set `other` holds k-step s + 1: it is written
+  // to the other buffer (if there is a k-step s + 1: more), and loaded again with k-step s + 1 + DEPTH
+  // (if there is one: refill).  The barrier stands before the last MFMA step: by then every wave has
+  // written its part of k-step s + 1 and has read the last operands of k-step s, so the last MFMA
+  // step can already read the first operands of k-step s + 1.
+  static_assert(TKS == 4, "the schedule below is written for four MFMA steps per k-step");
+  auto step = [&](int s, auto other, auto more, auto refill) {
     const int buf = s & 1;
-    if (s + 1 < steps) fetch((s + 1) * TBK);
-    // operands of MFMA step ks+1 are read from LDS while the MFMAs of step ks run
-    bf16x8 fa[2][WM], fw[2][WN];
-#pragma unroll
-    for (int i = 0; i < WM; ++i) fa[0][i] = *reinterpret_cast<const bf16x8*>(&As[buf][arow + i * 32][koff]);
-#pragma unroll
-    for (int j = 0; j < WN; ++j) fw[0][j] = *reinterpret_cast<const bf16x8*>(&Ws[buf][wrow + j * 32][koff]);
 #pragma unroll
     for (int ks = 0; ks < TKS; ++ks) {
       const int cur = ks & 1, nxt = cur ^ 1;
-      if (ks + 1 < TKS) {
+      if (ks + 1 < TKS)
+        read_operands(buf, ks + 1, nxt);
+      else if (decltype(more)::value)
+        read_operands(buf ^ 1, 0, nxt);
+      if (ks < 3) {
 #pragma unroll
-        for (int i = 0; i < WM; ++i) fa[nxt][i] = *reinterpret_cast<const bf16x8*>(&As[buf][arow + i * 32][(ks + 1) * 16 + koff]);
-#pragma unroll
-        for (int j = 0; j < WN; ++j) fw[nxt][j] = *reinterpret_cast<const bf16x8*>(&Ws[buf][wrow + j * 32][(ks + 1) * 16 + koff]);
+        for (int ci = ks; ci < CT_; ci += 3) {
+          if (decltype(more)::value) stash(ci, buf ^ 1, other);
+          if (decltype(refill)::value) fetch(ci, (s + 1 + DEPTH) * TBK, other);
+        }
       }
 #pragma unroll
       for (int i = 0; i < WM; ++i)
 #pragma unroll
         for (int j = 0; j < WN; ++j)
           acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa[cur][i], fw[cur][j], acc[i][j], 0, 0, 0);
+      if (ks == 2) __syncthreads();
+      __builtin_amdgcn_sched_barrier(0);  // each MFMA step keeps its share of the memory traffic
     }
-    if (s + 1 < steps) stash(buf ^ 1);
-    __syncthreads();
+  };
+
+  auto any_step = [&](int s, auto other) {  // near the end fewer and fewer k-steps have something ahead of them
+    if (s + 1 + DEPTH < steps)
+      step(s, other, Yes{}, Yes{});
+    else if (s + 1 < steps)
+      step(s, other, Yes{}, No{});
+    else
+      step(s, other, No{}, No{});
+  };
+#pragma unroll
+  for (int ci = 0; ci < CT_; ++ci) fetch(ci, 0, Set0{});
+  if (DEPTH == 2 && steps > 1) {
+#pragma unroll
+    for (int ci = 0; ci < CT_; ++ci) fetch(ci, TBK, std::integral_constant<int, DEPTH - 1>{});
+  }
+#pragma unroll
+  for (int ci = 0; ci < CT_; ++ci) stash(ci, 0, Set0{});
+  if (steps > DEPTH) {
+#pragma unroll
+    for (int ci = 0; ci < CT_; ++ci) fetch(ci, DEPTH * TBK, Set0{});
+  }
+  __syncthreads();
+  read_operands(0, 0, 0);
+  int s = 0;
+  if constexpr (DEPTH == 2) {
+    for (; s + 4 < steps; s += 2) {  // both k-steps of a round have a k-step three ahead
+      step(s, Set1{}, Yes{}, Yes{});
+      step(s + 1, Set0{}, Yes{}, Yes{});
+    }
+    for (; s < steps; s += 2) {
+      any_step(s, Set1{});
+      if (s + 1 < steps) any_step(s + 1, Set0{});
+    }
+  } else {
+    for (; s + 2 < steps; ++s) step(s, Set0{}, Yes{}, Yes{});
+    for (; s < steps; ++s) any_step(s, Set0{});
   }
 
   // accumulator layout of a 32x32 tile: lane holds column lane%32, rows 8*(r/4) + 4*(lane/32) + r%4
@@ -176,33 +221,40 @@ __global__ __launch_bounds__(256) void gemm_tiled_kernel(const bf16* __restrict_
     }
 }
 
-// Tile of the workgroup, (64 WM) x (64 WN): large tiles re-read the operands least; smaller ones
-// when the large ones would leave compute units idle.  GB_TILED="wm,wn" overrides (for measurements).
-inline void tiled_plan(int M, int N, int* wm, int* wn) {
-  auto blocks = [&](int a, int b) { return ((M + 64 * a - 1) / (64 * a)) * ((N + 64 * b - 1) / (64 * b)); };
-  // measured at 512..8192 rows on SmolLM2-1.7B shapes: 128 x 128 beats 256 x 128 everywhere (the
-  // larger tile's registers leave one workgroup a compute unit); 128 x 64 when tiles are few
-  *wm = 2, *wn = 2;
-  if (blocks(2, 2) < 384) *wn = 1;
+// Tile of the workgroup, 128 x (64 WN), and the depth of the register prefetch.  128 x 128 re-reads
+// the operands least; 128 x 64 when that would leave compute units idle.  The wide tile's registers
+// allow two workgroups a compute unit only with one k-step of prefetch, the narrow tile's with two.
+// GB_TILED="wn,depth" overrides (for measurements).
+inline void tiled_plan(int M, int N, int* wn, int* depth) {
+  const int blocks = ((M + 127) / 128) * ((N + 127) / 128);
+  *wn = blocks < 384 ? 1 : 2;
+  *depth = *wn == 1 ? 2 : 1;
   if (const char* env = getenv("GB_TILED")) {
-    int a = 0, b = 0;
-    if (sscanf(env, "%d,%d", &a, &b) == 2 && (a == 2 || a == 4) && (b == 1 || b == 2)) *wm = a, *wn = b;
+    int b = 0, d = 0;
+    if (sscanf(env, "%d,%d", &b, &d) == 2 && (b == 1 || b == 2) && (d == 1 || d == 2)) *wn = b, *depth = d;
   }
 }
 
 template <int EPI, typename CT>
 int launch_tiled(const bf16* a, int lda, const bf16* w, int ldw, CT* c, int ldc, int M, int N, int K, hipStream_t stream) {
-  int wm, wn;
-  tiled_plan(M, EPI == EPI_SILU_MUL ? N / 2 * 2 : N, &wm, &wn);
-  if (EPI == EPI_SILU_MUL) wn = 2;
+  int wn, depth;
+  tiled_plan(M, N, &wn, &depth);
+  if (EPI == EPI_SILU_MUL) wn = 2;  // a wave's two column tiles are gate and up
   const int cols = EPI == EPI_SILU_MUL ? N / 2 : N, bn = EPI == EPI_SILU_MUL ? 64 : 64 * wn;
-  const dim3 grid((cols + bn - 1) / bn, (M + 64 * wm - 1) / (64 * wm)), block(256);
+  const dim3 grid((cols + bn - 1) / bn, (M + 127) / 128), block(256);
   GB_REQUIRE(grid.y <= 65535, "gemm_bf16: M=%d needs more than 65535 row tiles", M);
-#define GB_T(A, B)            \
-  if (wm == (A) && wn == (B)) \
-    hipLaunchKernelGGL((gemm_tiled_kernel<(A), (B), EPI, CT>), grid, block, 0, stream, a, lda, w, ldw, c, ldc, M, N, K);
-  GB_T(4, 2) GB_T(2, 2)
-  if (EPI != EPI_SILU_MUL) { GB_T(4, EPI == EPI_SILU_MUL ? 2 : 1) GB_T(2, EPI == EPI_SILU_MUL ? 2 : 1) }
+  const bool kfull = K % TBK == 0;  // then no load needs a check against K
+#define GB_T(B, D)                                                                                                          \
+  if (wn == (B) && depth == (D)) {                                                                                          \
+    if (kfull)                                                                                                              \
+      hipLaunchKernelGGL((gemm_tiled_kernel<2, (B), (D), EPI, true, CT>), grid, block, 0, stream, a, lda, w, ldw, c, ldc, M, \
+                         N, K);                                                                                             \
+    else                                                                                                                    \
+      hipLaunchKernelGGL((gemm_tiled_kernel<2, (B), (D), EPI, false, CT>), grid, block, 0, stream, a, lda, w, ldw, c, ldc,   \
+                         M, N, K);                                                                                          \
+  }
+  GB_T(2, 1) GB_T(2, 2)
+  if (EPI != EPI_SILU_MUL) { GB_T((EPI == EPI_SILU_MUL ? 2 : 1), 1) GB_T((EPI == EPI_SILU_MUL ? 2 : 1), 2) }
 #undef GB_T
   return launched("gemm_bf16 (tiled)");
 }
