@@ -138,17 +138,22 @@ __device__ __forceinline__ void attend64(Running<HD>& st, const bf16x8* qf, cons
 
 // ----------------------------------------------------------------------------- decode
 // grid (chunks, kv heads, requests); request s is row s of q and out, at position positions[s].
-template <int HD>
-__global__ __launch_bounds__(256) void decode_kernel(const bf16* __restrict__ q, int q_stride, bf16* __restrict__ out,
-                                                     int out_stride, float* __restrict__ ws_acc, float* __restrict__ ws_ml,
-                                                     const int32_t* __restrict__ positions, const int32_t* __restrict__ tables,
-                                                     int table_stride, const bf16* __restrict__ kp, const bf16* __restrict__ vp,
-                                                     int nh, int nkv, int P, float scale, int window, int chunk, int splits) {
+// WAVES waves take 64 keys each in turn; dynamic LDS holds their partial results for the merge:
+// WAVES * (32 + HD * G) floats, G the query heads per kv head.
+template <int HD, int WAVES>
+__global__ __launch_bounds__(WAVES * 64) void decode_kernel(const bf16* __restrict__ q, int q_stride, bf16* __restrict__ out,
+                                                            int out_stride, float* __restrict__ ws_acc,
+                                                            float* __restrict__ ws_ml, const int32_t* __restrict__ positions,
+                                                            const int32_t* __restrict__ tables, int table_stride,
+                                                            const bf16* __restrict__ kp, const bf16* __restrict__ vp, int nh,
+                                                            int nkv, int P, float scale, int window, int chunk, int splits) {
   constexpr int KS = (HD + 31) / 32, DB = HD / 16;
-  __shared__ float sm_m[4][16], sm_l[4][16];
-  __shared__ float sm_acc[4][HD][16];
+  extern __shared__ float decode_lds[];
   const int s = blockIdx.z, kvh = blockIdx.y, split = blockIdx.x;
   const int G = nh / nkv;
+  float* sm_m = decode_lds;               // [WAVES][16]
+  float* sm_l = sm_m + WAVES * 16;        // [WAVES][16]
+  float* sm_acc = sm_l + WAVES * 16;      // [WAVES][HD][G]
   const int pos = positions[s];
   const int lo = window > 0 ? max(0, pos - window + 1) : 0;
   const int c0 = split * chunk;
@@ -167,34 +172,36 @@ __global__ __launch_bounds__(256) void decode_kernel(const bf16* __restrict__ q,
   reset(st);
   const int col_lo = col < G ? lo : 1, col_hi = col < G ? pos : 0;
   const int end = min(c0 + chunk, pos + 1);
-  for (int kb = c0 + wave * 64; kb < end; kb += 256) {
+  for (int kb = c0 + wave * 64; kb < end; kb += 64 * WAVES) {
     if (kb + 64 <= lo) continue;
     attend64<HD>(st, qf, kp, vp, table, nkv, kvh, P, kb, col_lo, col_hi, lo, pos, scale, lane);
   }
   st.l += __shfl_xor(st.l, 16, kWave);
   st.l += __shfl_xor(st.l, 32, kWave);
   if (lane < 16) {
-    sm_m[wave][col] = st.m;
-    sm_l[wave][col] = st.l;
+    sm_m[wave * 16 + col] = st.m;
+    sm_l[wave * 16 + col] = st.l;
   }
+  if (col < G) {
 #pragma unroll
-  for (int b = 0; b < DB; ++b)
+    for (int b = 0; b < DB; ++b)
 #pragma unroll
-    for (int r = 0; r < 4; ++r) sm_acc[wave][16 * b + 4 * (lane >> 4) + r][col] = st.acc[b][r];
+      for (int r = 0; r < 4; ++r) sm_acc[((size_t)wave * HD + 16 * b + 4 * (lane >> 4) + r) * G + col] = st.acc[b][r];
+  }
   __syncthreads();
-  // the four waves' partial results, combined in wave order
-  for (int cell = tid; cell < HD * 16; cell += 256) {
-    const int d = cell >> 4, cc = cell & 15;
-    if (cc >= G) continue;
-    float M = sm_m[0][cc];
+  // the waves' partial results, combined in wave order
+  for (int cell = tid; cell < HD * G; cell += WAVES * 64) {
+    const int d = cell / G, cc = cell % G;
+    float M = sm_m[cc];
 #pragma unroll
-    for (int w = 1; w < 4; ++w) M = fmaxf(M, sm_m[w][cc]);
+    for (int w = 1; w < WAVES; ++w) M = fmaxf(M, sm_m[w * 16 + cc]);
     float val = 0.f, L = 0.f;
 #pragma unroll
-    for (int w = 0; w < 4; ++w) {
-      const float f = sm_m[w][cc] == -INFINITY ? 0.f : __expf(sm_m[w][cc] - M);
-      val += sm_acc[w][d][cc] * f;
-      L += sm_l[w][cc] * f;
+    for (int w = 0; w < WAVES; ++w) {
+      const float mw = sm_m[w * 16 + cc];
+      const float f = mw == -INFINITY ? 0.f : __expf(mw - M);
+      val += sm_acc[((size_t)w * HD + d) * G + cc] * f;
+      L += sm_l[w * 16 + cc] * f;
     }
     const int head = kvh * G + cc;
     if (splits == 1) {
@@ -568,12 +575,23 @@ extern "C" int gb_attention_decode_bf16(const void* q, int q_stride, void* out, 
   GB_REQUIRE(n_decode <= 65535 && nkv <= 65535, "attention_decode: too many requests or kv heads for one launch");
   if (n_decode == 0) return 0;
   const int splits = (max_context + chunk - 1) / chunk;
-  const dim3 grid(splits, nkv, n_decode), block(256);
-#define GB_CASE(HD)                                                                                                        \
-  if (hd == HD)                                                                                                            \
-    hipLaunchKernelGGL(decode_kernel<HD>, grid, block, 0, stream, (const bf16*)q, q_stride, (bf16*)out, out_stride,         \
-                       (float*)ws_acc, (float*)ws_ml, positions, tables, table_stride, (const bf16*)k_pages,               \
-                       (const bf16*)v_pages, nh, nkv, page_size, scale, window, chunk, splits);
+  // one workgroup per request and kv head (no chunks to combine afterwards) gets 16 waves, so that as
+  // many loads are in flight as with four workgroups of four
+  const int G = nh / nkv;
+  const int waves = (splits == 1 && 16 * (32 + (size_t)hd * G) * sizeof(float) <= 65536) ? 16 : 4;
+  const size_t lds = (size_t)waves * (32 + (size_t)hd * G) * sizeof(float);
+  const dim3 grid(splits, nkv, n_decode), block(waves * 64);
+#define GB_CASE(HD)                                                                                                         \
+  if (hd == HD) {                                                                                                           \
+    if (waves == 16)                                                                                                        \
+      hipLaunchKernelGGL((decode_kernel<HD, 16>), grid, block, lds, stream, (const bf16*)q, q_stride, (bf16*)out, out_stride, \
+                         (float*)ws_acc, (float*)ws_ml, positions, tables, table_stride, (const bf16*)k_pages,              \
+                         (const bf16*)v_pages, nh, nkv, page_size, scale, window, chunk, splits);                           \
+    else                                                                                                                    \
+      hipLaunchKernelGGL((decode_kernel<HD, 4>), grid, block, lds, stream, (const bf16*)q, q_stride, (bf16*)out, out_stride,  \
+                         (float*)ws_acc, (float*)ws_ml, positions, tables, table_stride, (const bf16*)k_pages,              \
+                         (const bf16*)v_pages, nh, nkv, page_size, scale, window, chunk, splits);                           \
+  }
   GB_FOR_HEAD_SIZES(GB_CASE)
 #undef GB_CASE
   if (int rc = launched("attention_decode")) return rc;

@@ -129,7 +129,7 @@ extern "C" int gb_rope_table(const int32_t* pos, const float* inv, float* cosv, 
 // With slots == nullptr nothing is stored (a layer that reads another layer's cache).
 // With nkv == 0 the row holds queries only.
 template <typename T>
-__global__ void rope_store_kernel(T* __restrict__ qkv, int row_stride, const float* __restrict__ cosv,
+__global__ void rope_store_scalar_kernel(T* __restrict__ qkv, int row_stride, const float* __restrict__ cosv,
                                   const float* __restrict__ sinv, const int32_t* __restrict__ slots,
                                   T* __restrict__ k_pages, T* __restrict__ v_pages, int nh, int nkv, int hd,
                                   int page_size, int rotate) {
@@ -186,6 +186,60 @@ __global__ void rope_store_kernel(T* __restrict__ qkv, int row_stride, const flo
   }
 }
 
+// The same for head sizes that are a multiple of 4 and rows aligned to two elements: grid (tokens,
+// groups of heads), 16 lanes a head, a lane takes two neighbouring pairs as two-element words.  Every
+// lane's loads are independent of every store, so one round trip to memory covers a token, and few
+// tokens (decoding) still spread over many waves.  A "unit" is a query head, a key head or a value head
+// in the order of the row.
+template <typename T>
+struct Pair {
+  T a, b;
+};
+
+template <typename T>
+__global__ void rope_store_kernel(T* __restrict__ qkv, int row_stride, const float* __restrict__ cosv,
+                                  const float* __restrict__ sinv, const int32_t* __restrict__ slots,
+                                  T* __restrict__ k_pages, T* __restrict__ v_pages, int nh, int nkv, int hd,
+                                  int page_size, int rotate) {
+  using P = Pair<T>;
+  const int t = blockIdx.x;
+  const int half = hd / 2;
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int unit = (blockIdx.y * (blockDim.x >> 6) + wave) * 4 + (lane >> 4);
+  const int units = nh + nkv + (slots ? nkv : 0);
+  if (unit >= units) return;
+  T* head = qkv + (size_t)t * row_stride + (size_t)unit * hd;
+  const bool is_v = unit >= nh + nkv, is_k = unit >= nh && !is_v;
+  const int slot = (slots && unit >= nh) ? slots[t] : -1;
+  const int page = slot >= 0 ? slot / page_size : 0, off = slot >= 0 ? slot % page_size : 0;
+  for (int j = (lane & 15) * 2; j < half; j += 32) {
+    const P x0 = *reinterpret_cast<const P*>(head + j), x1 = *reinterpret_cast<const P*>(head + half + j);
+    P y0 = x0, y1 = x1;
+    if (!is_v && rotate) {
+      const float2 c = *reinterpret_cast<const float2*>(cosv + (size_t)t * half + j);
+      const float2 sn = *reinterpret_cast<const float2*>(sinv + (size_t)t * half + j);
+      y0.a = from_f<T>(to_f(x0.a) * c.x - to_f(x1.a) * sn.x);
+      y0.b = from_f<T>(to_f(x0.b) * c.y - to_f(x1.b) * sn.y);
+      y1.a = from_f<T>(to_f(x1.a) * c.x + to_f(x0.a) * sn.x);
+      y1.b = from_f<T>(to_f(x1.b) * c.y + to_f(x0.b) * sn.y);
+      *reinterpret_cast<P*>(head + j) = y0;  // rotated keys stay in the row too: parts may read them back
+      *reinterpret_cast<P*>(head + half + j) = y1;
+    }
+    if (slot < 0) continue;
+    if (is_k) {
+      T* dst = k_pages + (((size_t)page * nkv + (unit - nh)) * page_size + off) * hd;
+      *reinterpret_cast<P*>(dst + j) = y0;
+      *reinterpret_cast<P*>(dst + half + j) = y1;
+    } else if (is_v) {
+      T* dst = v_pages + ((size_t)page * nkv + (unit - nh - nkv)) * hd * page_size + off;
+      dst[(size_t)j * page_size] = x0.a;
+      dst[(size_t)(j + 1) * page_size] = x0.b;
+      dst[(size_t)(half + j) * page_size] = x1.a;
+      dst[(size_t)(half + j + 1) * page_size] = x1.b;
+    }
+  }
+}
+
 extern "C" int gb_rope_store(void* qkv, int dtype, int row_stride, const float* cosv, const float* sinv,
                              const int32_t* slots, void* k_pages, void* v_pages, int n, int nh, int nkv, int hd,
                              int page_size, int rotate, hipStream_t stream) {
@@ -195,12 +249,29 @@ extern "C" int gb_rope_store(void* qkv, int dtype, int row_stride, const float* 
   GB_REQUIRE(slots == nullptr || (k_pages && v_pages && page_size > 0), "rope_store: slots given without pages");
   GB_REQUIRE(!rotate || (cosv && sinv), "rope_store: rotation asked without a table");
   if (n == 0) return 0;
+  const bool pairs_of_two = hd % 4 == 0 && row_stride % 2 == 0 && (uintptr_t)qkv % 8 == 0 && (uintptr_t)k_pages % 8 == 0 &&
+                            (!rotate || ((uintptr_t)cosv % 8 == 0 && (uintptr_t)sinv % 8 == 0));
+  if (pairs_of_two) {
+    const int units = nh + nkv + (slots ? nkv : 0);
+    const int threads = n <= 64 ? 64 : 256;  // few tokens: more, smaller workgroups
+    const dim3 grid(n, (units + threads / 16 - 1) / (threads / 16));
+    GB_REQUIRE(grid.y <= 65535, "rope_store: %d heads are too many for one launch", units);
+    if (dtype == kF32)
+      hipLaunchKernelGGL(rope_store_kernel<float>, grid, dim3(threads), 0, stream, (float*)qkv, row_stride, cosv, sinv, slots,
+                         (float*)k_pages, (float*)v_pages, nh, nkv, hd, page_size, rotate);
+    else if (dtype == kBF16)
+      hipLaunchKernelGGL(rope_store_kernel<bf16>, grid, dim3(threads), 0, stream, (bf16*)qkv, row_stride, cosv, sinv, slots,
+                         (bf16*)k_pages, (bf16*)v_pages, nh, nkv, hd, page_size, rotate);
+    else
+      return fail("rope_store: unknown dtype %d", dtype);
+    return launched("rope_store");
+  }
   const int threads = (nh + nkv) * hd / 2 >= 256 ? 256 : 64;
   if (dtype == kF32)
-    hipLaunchKernelGGL(rope_store_kernel<float>, dim3(n), dim3(threads), 0, stream, (float*)qkv, row_stride, cosv, sinv,
+    hipLaunchKernelGGL(rope_store_scalar_kernel<float>, dim3(n), dim3(threads), 0, stream, (float*)qkv, row_stride, cosv, sinv,
                        slots, (float*)k_pages, (float*)v_pages, nh, nkv, hd, page_size, rotate);
   else if (dtype == kBF16)
-    hipLaunchKernelGGL(rope_store_kernel<bf16>, dim3(n), dim3(threads), 0, stream, (bf16*)qkv, row_stride, cosv, sinv,
+    hipLaunchKernelGGL(rope_store_scalar_kernel<bf16>, dim3(n), dim3(threads), 0, stream, (bf16*)qkv, row_stride, cosv, sinv,
                        slots, (bf16*)k_pages, (bf16*)v_pages, nh, nkv, hd, page_size, rotate);
   else
     return fail("rope_store: unknown dtype %d", dtype);

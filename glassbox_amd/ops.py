@@ -308,9 +308,11 @@ def tuned_attention_supports(k_pages: torch.Tensor, n_heads: int, window: int) -
 
 
 def decode_chunk(n_decode: int, n_kv_heads: int, max_context: int) -> int:
-    """Keys per workgroup of the decode kernel: a multiple of 256, small enough that the launch has
-    about a thousand workgroups, large enough that a workgroup's fixed costs are spread."""
-    want_splits = max(1, 1024 // max(1, n_decode * n_kv_heads))
+    """Keys per workgroup of the decode kernel: a multiple of 256.  With a workgroup for every compute
+    unit from requests and kv heads alone, each takes a whole context (and sixteen waves: nothing is
+    left to combine afterwards); otherwise small enough that the launch has about a thousand workgroups."""
+    groups = max(1, n_decode * n_kv_heads)
+    want_splits = 1 if groups >= 256 else max(1, 1024 // groups)
     chunk = -(-max_context // want_splits)
     return max(256, -(-chunk // 256) * 256)
 

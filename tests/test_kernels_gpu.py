@@ -184,7 +184,8 @@ def test_silu_mul():
     assert (out.cpu().double() - want).abs().max().item() < 1e-5
 
 
-@pytest.mark.parametrize("hd,theta", [(16, 10000.0), (48, 500000.0), (128, 130000.0)])
+@pytest.mark.parametrize("hd,theta", [(16, 10000.0), (48, 500000.0), (128, 130000.0), (80, 10000.0),
+                                      (10, 10000.0)])   # 10: no multiple of 4, the kernel that goes pair by pair
 def test_rope_table_and_rotation(hd, theta):
     """Against the plain implementation: pairing (i, i + hd/2), sign, 32-bit angle at long positions."""
     from glassbox_amd import ops
@@ -392,6 +393,29 @@ def test_tuned_prefill_long_portions(nh, nkv, hd, window):
                                 scale, window)
     err = (out[rows].cpu().double() - want).abs().max().item()
     assert err < 2 ** -6, err
+
+
+@pytest.mark.parametrize("nh,nkv,hd,window", [(8, 8, 64, 0), (16, 8, 32, 0), (8, 8, 128, 0), (24, 8, 48, 200)])
+def test_tuned_decode_with_a_workgroup_per_request_and_kv_head(nh, nkv, hd, window):
+    """Requests and kv heads enough that no context is split over workgroups: sixteen waves share one,
+    and their results are combined within the workgroup."""
+    from types import SimpleNamespace
+    from glassbox_amd import ops
+    g = torch.Generator().manual_seed(nh + hd)
+    ctx_lens = [1, 2, 63, 64, 65, 255, 256, 257, 1023, 1024, 1025, 1500] + torch.randint(1, 1400, (24,), generator=g).tolist()
+    assert ops.decode_chunk(len(ctx_lens), nkv, 1536) >= 1536          # one chunk takes it all
+    k_pages, v_pages, tables, ks, vs = paged_setup(ctx_lens, nkv, hd, 16, seed=hd, dtype=torch.bfloat16)
+    ctx = BareContext([1] * len(ctx_lens), ctx_lens, tables, max_context=1536)
+    n = len(ctx_lens)
+    q = (rnd(n, nh * hd, seed=13) * 0.7).bfloat16()
+    scale = 1 / math.sqrt(hd)
+    cache = SimpleNamespace(k_pages=to_dev(k_pages), v_pages=to_dev(v_pages), group=0)
+    out = torch.zeros(n, nh * hd, device=DEV, dtype=torch.bfloat16)
+    ops.attention_decode(to_dev(q), out, ctx, cache, nh, scale, window)
+    want = plain_attention_rows(q, ks, vs, ctx.tok_seq, ctx.pos_list, nh, scale, window)
+    err = (out.cpu().double() - want).abs().max(dim=1).values
+    bad = torch.nonzero(err > 2 ** -6).flatten().tolist()
+    assert not bad, f"requests {bad[:8]} with contexts {[ctx_lens[i] for i in bad[:8]]}: {err[bad[:8]]}"
 
 
 def test_tuned_decode_finds_one_far_key_in_every_chunk_position():
