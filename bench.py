@@ -81,8 +81,11 @@ def main() -> int:
     T = PREFILL_TOKENS
     pf_flops = 2 * T * layer_params * L + L * 4 * qd * (T * (T + 1) // 2) + 2 * d * vocab
     peak = PEAK["bf16_tflops"] if a.dtype == "bfloat16" else PEAK["fp32_tflops"]
-    prefill = {"value": round(T / pf, 1), "tokens": T, "ms": round(pf * 1e3, 3),
-               "frac": round(pf_flops / pf / (peak * 1e12), 4)}
+    if a.only == "decode":   # not measured in this run: null, which JSON has and NaN is not
+        prefill = {"value": None, "tokens": T, "ms": None, "frac": None}
+    else:
+        prefill = {"value": round(T / pf, 1), "tokens": T, "ms": round(pf * 1e3, 3),
+                   "frac": round(pf_flops / pf / (peak * 1e12), 4)}
 
     # ---- decode
     def decode_run(batch, steps, warmup):
