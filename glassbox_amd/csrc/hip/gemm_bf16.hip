@@ -3,7 +3,7 @@
 // (crates/glassbox-core/src/kernels.rs:381,586).  Both operands are contiguous along k, which
 // is the layout MFMA operands want: every lane loads 8 consecutive k as one 16-byte word.
 //
-// Two kernels:
+// Three kernels:
 //  * tiled  (M > 64, prompt portions): a workgroup of 2x2 waves, each wave a block of up to 4x2
 //    v_mfma_f32_32x32x16_bf16 tiles (workgroup tile up to 256x128), operands staged through LDS in
 //    k-steps of 32 with two buffers; the SiLU-multiply of stacked gate/up rows can be its epilogue.
@@ -11,7 +11,9 @@
 //    waves take interleaved 64-wide k blocks, stream W straight from memory into MFMA operands
 //    (v_mfma_f32_16x16x32_bf16, W as the A operand so that the 16 rows fill the tile) and combine
 //    through LDS in a fixed order; it can norm float32 rows on the way and apply the SiLU-multiply.
-// In both, every output cell is summed in an order fixed by (K, kernel) alone, not by M or by
+//  * folded (M <= 8 and few rows of W): the skinny kernel with two k ranges side by side in a tile,
+//    so that a workgroup owns 8 rows of W and there are twice as many workgroups.
+// In all, every output cell is summed in an order fixed by (K, kernel) alone, not by M or by
 // the cell's neighbours.  C is bfloat16 or float32; accumulation (+=) is into float32.
 #include <type_traits>
 
@@ -262,7 +264,7 @@ int launch_tiled(const bf16* a, int lda, const bf16* w, int ldw, CT* c, int ldc,
 // ------------------------------------------------------------------------ skinny
 // grid (row tiles of W).  A workgroup of WAVES waves owns 16 rows of W and walks all of k in slices
 // of ITERS*WAVES*64: wave w takes the 64-wide k blocks w, w+WAVES, ... of a slice; inside a block
-// lane group q holds k = 16q..16q+15 as two operands of 8 (the same split for W and for A, so the
+// lane group q holds k = 8q..8q+7 of each half of 32 (the same split for W and for A, so the
 // products pair up).  All loads of a slice are issued before its first MFMA.  The waves combine
 // through LDS in wave order.  Few rows of W (a small N) are given many waves each, so that the
 // launch still keeps enough loads in flight to use the memory system; no partial result ever
@@ -457,6 +459,116 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_skinny_kernel(const void* __r
   }
 }
 
+// ------------------------------------------------------------------------ folded (M <= 8)
+// With at most 8 rows of A, a 16 x 16 tile has room for two k ranges side by side.  Rows 0..7 of the
+// tile are 8 rows of W over the first half of a 128-wide k block and rows 8..15 the same 8 rows of W
+// over its second half; columns 0..7 are the rows of A over the first half, columns 8..15 over the
+// second.  Cells (n, m) and (n + 8, m + 8) then hold the two halves of one sum; the other two
+// quarters of the tile pair the wrong halves and are dropped.  A workgroup so owns 8 rows of W, not
+// 16, and a product with few rows of W (decoding: the O and down projections) has a workgroup for
+// every compute unit: one compute unit draws only a fraction of the memory bandwidth.
+template <int WAVES, int ITERS, int RT, int EPI, bool RMS, typename CT>
+__global__ __launch_bounds__(WAVES * 64) void gemm_fold_kernel(const void* __restrict__ a, int lda,
+                                                               const bf16* __restrict__ w, int ldw, CT* __restrict__ c,
+                                                               int ldc, int M, int N, int K, const void* __restrict__ gamma,
+                                                               int gamma_f32, float eps) {
+  static_assert(EPI != EPI_SILU_MUL && WAVES >= 4, "folded tiles store or accumulate; the first four waves finish");
+  __shared__ float part[WAVES][RT][64][4];
+  __shared__ float sspart[RMS ? WAVES : 1][64];
+  const int tid = threadIdx.x, lane = tid % 64, wave = tid / 64;
+  const int r = lane % 16, q = lane / 16;
+  const int r8 = r & 7, khalf = (r >> 3) * 64;  // row of W and of A; which half of a k block
+  const bf16* wrow[RT];
+  bool row_ok[RT];
+#pragma unroll
+  for (int rt = 0; rt < RT; ++rt) {
+    const int row = (blockIdx.x * RT + rt) * 8 + r8;
+    row_ok[rt] = row < N;
+    wrow[rt] = w + (size_t)(row_ok[rt] ? row : 0) * ldw;
+  }
+  f32x4 acc[RT];
+  float ss = 0.f;
+#pragma unroll
+  for (int rt = 0; rt < RT; ++rt)
+#pragma unroll
+    for (int e = 0; e < 4; ++e) acc[rt][e] = 0.f;
+
+  for (int kbeg = 0; kbeg < K; kbeg += ITERS * WAVES * 128) {
+    bf16x8 wf[RT][ITERS][2], xf[ITERS][2];
+#pragma unroll
+    for (int rt = 0; rt < RT; ++rt)
+#pragma unroll
+      for (int it = 0; it < ITERS; ++it) {
+        const int k = kbeg + (wave + WAVES * it) * 128 + khalf + q * 8;
+        wf[rt][it][0] = (row_ok[rt] && k < K) ? load8(wrow[rt] + k) : zero8();
+        wf[rt][it][1] = (row_ok[rt] && k + 32 < K) ? load8(wrow[rt] + k + 32) : zero8();
+      }
+#pragma unroll
+    for (int it = 0; it < ITERS; ++it) {
+      const int k = kbeg + (wave + WAVES * it) * 128 + khalf + q * 8;
+      xf[it][0] = load_a<RMS>(a, lda, r8, k, r8 < M && k < K, gamma, gamma_f32, ss);
+      xf[it][1] = load_a<RMS>(a, lda, r8, k + 32, r8 < M && k + 32 < K, gamma, gamma_f32, ss);
+    }
+#pragma unroll
+    for (int it = 0; it < ITERS; ++it)
+#pragma unroll
+      for (int rt = 0; rt < RT; ++rt) {
+        acc[rt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wf[rt][it][0], xf[it][0], acc[rt], 0, 0, 0);
+        acc[rt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wf[rt][it][1], xf[it][1], acc[rt], 0, 0, 0);
+      }
+  }
+#pragma unroll
+  for (int rt = 0; rt < RT; ++rt)
+#pragma unroll
+    for (int e = 0; e < 4; ++e) part[wave][rt][lane][e] = acc[rt][e];
+  if (RMS) sspart[wave][lane] = ss;
+  __syncthreads();
+  if (tid >= 256) return;
+  // D[n, m]: lane l holds column m = l%16 and rows n = 4*(l/16) + e; thread tid owns cell (l = tid/4, e = tid%4)
+  const int l = tid / 4, e = tid % 4;
+  const int nrow = 4 * (l / 16) + e, m = l % 16;
+  if (nrow >= 8 || m >= 8) return;
+  float scale = 1.f;
+  if (RMS) {
+    // sum(x^2) of row m: its k were spread over the waves, the four lane groups and the two halves
+    float tot = 0.f;
+#pragma unroll
+    for (int wv = 0; wv < WAVES; ++wv)
+#pragma unroll
+      for (int qq = 0; qq < 4; ++qq) tot += sspart[wv][m + 16 * qq] + sspart[wv][m + 8 + 16 * qq];
+    scale = 1.0f / sqrtf(tot / (float)K + eps);
+  }
+#pragma unroll
+  for (int rt = 0; rt < RT; ++rt) {
+    float sum = 0.f;
+#pragma unroll
+    for (int wv = 0; wv < WAVES; ++wv) sum += part[wv][rt][l][e] + part[wv][rt][l + 40][e];  // cell (n + 8, m + 8)
+    const int n = (blockIdx.x * RT + rt) * 8 + nrow;
+    if (m < M && n < N) store_c<CT>(c + (size_t)m * ldc + n, sum * scale, EPI == EPI_ACCUMULATE);
+  }
+}
+
+// Folded tiles pay when the product has at most 8 rows and whole tiles of 16 rows of W would leave
+// compute units without a workgroup (measured: with 384 such tiles they no longer do).
+inline bool fold_pays(int M, int N) { return M <= 8 && (N + 15) / 16 < 256; }
+
+template <int EPI, bool RMS, typename CT>
+int launch_fold(const void* a, int lda, const bf16* w, int ldw, CT* c, int ldc, int M, int N, int K, const void* gamma,
+                int gamma_f32, float eps, hipStream_t stream) {
+  const int tiles = (N + 7) / 8, blocks = (K + 127) / 128;  // 128-wide k blocks
+  const int waves = blocks >= 16 ? 16 : 4;
+  const int rt = tiles >= 512 ? 2 : 1;
+  const int iters = (blocks + waves - 1) / waves >= 2 ? 2 : 1;  // four loads in flight a wave were measured no faster
+#define GB_CFG(WV, IT, RT)                                                                                                \
+  if (waves == WV && iters == IT && rt == RT)                                                                             \
+    hipLaunchKernelGGL((gemm_fold_kernel<WV, IT, RT, EPI, RMS, CT>), dim3((tiles + RT - 1) / RT), dim3(WV * 64), 0, stream, \
+                       a, lda, w, ldw, c, ldc, M, N, K, gamma, gamma_f32, eps);
+  GB_CFG(4, 1, 1) GB_CFG(4, 1, 2) GB_CFG(4, 2, 1) GB_CFG(4, 2, 2)
+  GB_CFG(16, 1, 1) GB_CFG(16, 1, 2) GB_CFG(16, 2, 1) GB_CFG(16, 2, 2)
+#undef GB_CFG
+  return launched("gemm_bf16 (folded)");
+}
+
 // Waves per workgroup, loads in flight per wave and row tiles per workgroup.
 // GB_SKINNY="waves,iters,rowtiles" overrides (for measurements).
 inline void skinny_plan(int tiles, int K, int mt, int* waves, int* iters, int* rt) {
@@ -533,6 +645,12 @@ extern "C" int gb_gemm_bf16(const void* a, int lda, const void* w, int ldw, void
   const bf16* W = (const bf16*)w;
   if (M <= 64) {
     const int gf = gamma_dtype == kF32;
+    if (fold_pays(M, N) && epilogue != EPI_SILU_MUL) {
+      if (gamma) return launch_fold<EPI_STORE, true, bf16>(a, lda, W, ldw, (bf16*)c, ldc, M, N, K, gamma, gf, eps, stream);
+      if (epilogue == EPI_ACCUMULATE) return launch_fold<EPI_ACCUMULATE, false, float>(a, lda, W, ldw, (float*)c, ldc, M, N, K, nullptr, 0, 0.f, stream);
+      if (c_dtype == kF32) return launch_fold<EPI_STORE, false, float>(a, lda, W, ldw, (float*)c, ldc, M, N, K, nullptr, 0, 0.f, stream);
+      return launch_fold<EPI_STORE, false, bf16>(a, lda, W, ldw, (bf16*)c, ldc, M, N, K, nullptr, 0, 0.f, stream);
+    }
     if (gamma) {
       if (epilogue == EPI_STORE) return launch_skinny<EPI_STORE, true, bf16>(a, lda, W, ldw, (bf16*)c, ldc, M, N, K, gamma, gf, eps, stream);
       return launch_skinny<EPI_SILU_MUL, true, bf16>(a, lda, W, ldw, (bf16*)c, ldc, M, N, K, gamma, gf, eps, stream);
