@@ -242,13 +242,17 @@ __global__ void decode_reduce_kernel(const float* __restrict__ ws_acc, const flo
 // ---------------------------------------------------------------------------- prefill
 // A wave takes blocks of 32 consecutive tokens of one query head; v_mfma_f32_32x32x16_bf16 throughout.
 // Per 64 keys:
-//   S^T[key, tok]   A = 32 keys x 16 dims (lane: key lane%32, dims 8*(lane/32)..+7 of the k-step),
-//                   B = the query tokens alike; the result lane holds token lane%32 and keys
-//                   8*(r/4) + 4*(lane/32) + r%4 of the 32-key tile
+//   S^T[key, tok]   A = 32 keys x 16 dims (lane: row lane%32, dims 8*(lane/32)..+7 of the k-step),
+//                   B = the query tokens alike; the result lane holds token lane%32 and rows
+//                   8*(r/4) + 4*(lane/32) + r%4 of the 32-row tile
 //   O^T[dim, tok]   A = 32 dims x 16 keys from the transposed value page, B = probabilities: registers
-//                   8h..8h+7 of a score tile are, as they stand, the B operand of the k-step over keys
-//                   16h..16h+15 if slot e of lane group g means key 4g+e (e<4) or 8+4g+(e-4); the value
-//                   operand is loaded in that same order (two 8-byte loads a lane)
+//                   8h..8h+7 of a score tile are, as they stand, the B operand of the k-step over rows
+//                   16h..16h+15, lane group g holding rows 4g..4g+3 and 8+4g..8+4g+3 of them
+// Which key a row of the score tile stands for is free: within each group of 16 rows the keys are
+// dealt so that those eight rows of a lane group are the neighbouring keys 8g..8g+7.  The value
+// operand of a lane is then one 16-byte word of its dimension's row in the page, and a load
+// instruction of the wave reads whole 32-byte rows (the cache serves 64 bytes at a time; half-used
+// pieces were what bounded this kernel).
 // Scores stay raw in the registers; softmax works on exp2(raw*c - max*c) with c = scale*log2(e).
 // Causal work grows with the position, so a wave takes block i and block n-1-i of its request's
 // portion: every wave then has the same number of (token, key) pairs.  With QB == 2 both blocks are
@@ -274,7 +278,10 @@ struct PageSource {
 template <int HD>
 __device__ __forceinline__ void load_keys(bf16x8 (&kf)[2][HD / 16], const PageSource& src, int kbase, int lane) {
   const int col = lane & 31, g = lane >> 5;
-  const int mine = (col & 15) * HD + 8 * g;
+  // row r of a group of 16 rows of the score tile takes key 8*((r>>2)&1) + 4*(r>>3) + (r&3) of the group:
+  // the probabilities a lane then holds for a value product are those of 8 neighbouring keys
+  const int r16 = col & 15, key16 = ((r16 >> 2) & 1) * 8 + (r16 >> 3) * 4 + (r16 & 3);
+  const int mine = key16 * HD + 8 * g;
 #pragma unroll
   for (int t = 0; t < 2; ++t) {
     int s0, s1;  // a tile of 32 keys is two groups of 16, each within one page
@@ -290,25 +297,15 @@ __device__ __forceinline__ void load_keys(bf16x8 (&kf)[2][HD / 16], const PageSo
 template <int HD>
 __device__ __forceinline__ void load_values(bf16x8 (&vf)[(HD + 31) / 32][4], const PageSource& src, int kbase, int lane) {
   const int col = lane & 31, g = lane >> 5;
-  const int mine = (col << src.shift) + 4 * g;
+  const int mine = (col << src.shift) + 8 * g;
 #pragma unroll
   for (int u = 0; u < 4; ++u) {
     int slot;
     const size_t pg = src.page_of(kbase + 16 * u, &slot);
     const bf16* vb = src.vp + ((pg * HD) << src.shift) + slot + mine;
 #pragma unroll
-    for (int b = 0; b < (HD + 31) / 32; ++b) {
-      if (32 * b + 32 <= HD || 32 * b + col < HD) {
-        const bf16x4 a = load4(vb + ((size_t)(32 * b) << src.shift)), bb = load4(vb + ((size_t)(32 * b) << src.shift) + 8);
-#pragma unroll
-        for (int e = 0; e < 4; ++e) {
-          vf[b][u][e] = a[e];
-          vf[b][u][4 + e] = bb[e];
-        }
-      } else {
-        vf[b][u] = zero8();
-      }
-    }
+    for (int b = 0; b < (HD + 31) / 32; ++b)
+      vf[b][u] = (32 * b + 32 <= HD || 32 * b + col < HD) ? load8(vb + ((size_t)(32 * b) << src.shift)) : zero8();
   }
 }
 
@@ -351,7 +348,7 @@ __device__ __forceinline__ void attend64_q32(float (&m)[QB], float (&l)[QB], f32
       for (int t = 0; t < 2; ++t)
 #pragma unroll
         for (int r = 0; r < 16; ++r) {
-          const int key = kbase + 32 * t + 8 * (r >> 2) + 4 * g + (r & 3);
+          const int key = kbase + 32 * t + 16 * (r >> 3) + 8 * g + 4 * ((r >> 2) & 1) + (r & 3);
           if (key < lo[qb] || key > hi[qb]) s[t][r] = -INFINITY;
         }
     }
