@@ -200,13 +200,13 @@ template <typename T>
 __global__ void rope_store_kernel(T* __restrict__ qkv, int row_stride, const float* __restrict__ cosv,
                                   const float* __restrict__ sinv, const int32_t* __restrict__ slots,
                                   T* __restrict__ k_pages, T* __restrict__ v_pages, int nh, int nkv, int hd,
-                                  int page_size, int rotate) {
+                                  int page_size, int rotate, int v_rows) {
   using P = Pair<T>;
   const int t = blockIdx.x;
   const int half = hd / 2;
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int unit = (blockIdx.y * (blockDim.x >> 6) + wave) * 4 + (lane >> 4);
-  const int units = nh + nkv + (slots ? nkv : 0);
+  const int units = nh + nkv + ((slots && t < v_rows) ? nkv : 0);  // rows from v_rows on: values are stored by tiles
   if (unit >= units) return;
   T* head = qkv + (size_t)t * row_stride + (size_t)unit * hd;
   const bool is_v = unit >= nh + nkv, is_k = unit >= nh && !is_v;
@@ -240,15 +240,98 @@ __global__ void rope_store_kernel(T* __restrict__ qkv, int row_stride, const flo
   }
 }
 
+// Values of prompt portions, sixteen positions at a time: the transposed page holds the sixteen slots
+// of one dimension side by side, so a tile of 16 tokens x hd is turned in LDS and written as whole
+// 16-byte words instead of two bytes at a time.  grid (groups of 16 positions, kv heads, requests
+// from seq_base on); request s has q_len[s] rows from row q_start[s] on, the first at position pos0[s].
+template <typename T>
+__global__ void store_values_kernel(const T* __restrict__ qkv, int row_stride, const int32_t* __restrict__ slots,
+                                    T* __restrict__ v_pages, const int32_t* __restrict__ q_start,
+                                    const int32_t* __restrict__ q_len, const int32_t* __restrict__ pos0, int seq_base,
+                                    int nh, int nkv, int hd, int page_size) {
+  extern __shared__ unsigned char tile_bytes[];
+  T* tile = reinterpret_cast<T*>(tile_bytes);  // [16][hd + 2]
+  const int ld = hd + 2;
+  const int seq = seq_base + blockIdx.z, kvh = blockIdx.y;
+  const int first = pos0[seq], n = q_len[seq];
+  const int p_lo = (first / 16 + blockIdx.x) * 16;  // the group's first position
+  const int j_lo = p_lo - first;                     // its token index in the portion (may be negative)
+  if (j_lo >= n) return;
+  const int row0 = q_start[seq];
+  const int chunks = hd / 8;
+  for (int idx = threadIdx.x; idx < 16 * chunks; idx += blockDim.x) {
+    const int i = idx / chunks, ch = idx % chunks, j = j_lo + i;
+    if (j < 0 || j >= n) continue;
+    const T* src = qkv + (size_t)(row0 + j) * row_stride + (size_t)(nh + nkv + kvh) * hd + ch * 8;
+    alignas(16) T got[8];
+    *reinterpret_cast<uint4*>(got) = *reinterpret_cast<const uint4*>(src);
+    if (sizeof(T) == 4) *reinterpret_cast<uint4*>(got + 4) = *reinterpret_cast<const uint4*>(src + 4);
+#pragma unroll
+    for (int e = 0; e < 8; ++e) tile[i * ld + ch * 8 + e] = got[e];
+  }
+  __syncthreads();
+  // the page and the first slot of the group, from any token of it that exists
+  const int j_any = max(j_lo, 0);
+  const int slot_any = slots[row0 + j_any];
+  const int page = slot_any / page_size, off0 = slot_any % page_size - (j_any - j_lo);
+  T* dst_page = v_pages + ((size_t)page * nkv + kvh) * hd * page_size + off0;
+  for (int idx = threadIdx.x; idx < 2 * hd; idx += blockDim.x) {
+    const int d = idx / 2, h8 = idx % 2;
+    T* dst = dst_page + (size_t)d * page_size + 8 * h8;
+    const int i0 = 8 * h8;
+    if (j_lo + i0 >= 0 && j_lo + i0 + 8 <= n) {
+      alignas(16) T word[8];
+#pragma unroll
+      for (int e = 0; e < 8; ++e) word[e] = tile[(i0 + e) * ld + d];
+      if (sizeof(T) == 2) {
+        *reinterpret_cast<uint4*>(dst) = *reinterpret_cast<const uint4*>(word);
+      } else {
+        *reinterpret_cast<uint4*>(dst) = *reinterpret_cast<const uint4*>(word);
+        *reinterpret_cast<uint4*>(dst + 4) = *reinterpret_cast<const uint4*>(word + 4);
+      }
+    } else {
+#pragma unroll
+      for (int e = 0; e < 8; ++e) {
+        const int j = j_lo + i0 + e;
+        if (j >= 0 && j < n) dst[e] = tile[(i0 + e) * ld + d];
+      }
+    }
+  }
+}
+
+// Rows v_rows .. n-1 are prompt portions described by q_start, q_len and pos0 of requests seq_base ..
+// seq_base + n_seqs - 1 (the longest has max_q_len rows): their values are stored tile by tile.  With
+// v_rows == n there are none.
 extern "C" int gb_rope_store(void* qkv, int dtype, int row_stride, const float* cosv, const float* sinv,
                              const int32_t* slots, void* k_pages, void* v_pages, int n, int nh, int nkv, int hd,
-                             int page_size, int rotate, hipStream_t stream) {
+                             int page_size, int rotate, int v_rows, const int32_t* q_start, const int32_t* q_len,
+                             const int32_t* pos0, int seq_base, int n_seqs, int max_q_len, hipStream_t stream) {
   GB_REQUIRE(n >= 0 && nh >= 0 && nkv >= 0 && hd > 0 && hd % 2 == 0, "rope_store: bad sizes n=%d nh=%d nkv=%d hd=%d", n, nh, nkv, hd);
   GB_REQUIRE(row_stride >= (nh + 2 * nkv) * hd || (slots == nullptr && row_stride >= (nh + nkv) * hd),
              "rope_store: row stride %d is shorter than the stacked heads", row_stride);
   GB_REQUIRE(slots == nullptr || (k_pages && v_pages && page_size > 0), "rope_store: slots given without pages");
   GB_REQUIRE(!rotate || (cosv && sinv), "rope_store: rotation asked without a table");
   if (n == 0) return 0;
+  // the tile kernel takes pages of a multiple of 16 slots, head sizes of a multiple of 8 and aligned rows
+  const bool tiles = slots && v_rows < n && n_seqs > 0 && q_start && q_len && pos0 && page_size % 16 == 0 && hd % 8 == 0 &&
+                     (uintptr_t)v_pages % 16 == 0 && (uintptr_t)qkv % 16 == 0 && row_stride % 8 == 0;
+  if (!tiles) v_rows = n;
+  if (tiles) {
+    const dim3 grid((max_q_len + 15) / 16 + 1, nkv, n_seqs);
+    GB_REQUIRE(nkv <= 65535 && n_seqs <= 65535, "rope_store: too many kv heads or requests for one launch");
+    const int threads = 2 * hd >= 256 ? 256 : 128;
+    if (dtype == kF32)
+      hipLaunchKernelGGL(store_values_kernel<float>, grid, dim3(threads), 16 * (hd + 2) * sizeof(float), stream,
+                         (const float*)qkv, row_stride, slots, (float*)v_pages, q_start, q_len, pos0, seq_base, nh, nkv, hd,
+                         page_size);
+    else if (dtype == kBF16)
+      hipLaunchKernelGGL(store_values_kernel<bf16>, grid, dim3(threads), 16 * (hd + 2) * sizeof(bf16), stream,
+                         (const bf16*)qkv, row_stride, slots, (bf16*)v_pages, q_start, q_len, pos0, seq_base, nh, nkv, hd,
+                         page_size);
+    else
+      return fail("rope_store: unknown dtype %d", dtype);
+    if (int rc = launched("rope_store (values)")) return rc;
+  }
   const bool pairs_of_two = hd % 4 == 0 && row_stride % 2 == 0 && (uintptr_t)qkv % 8 == 0 && (uintptr_t)k_pages % 8 == 0 &&
                             (!rotate || ((uintptr_t)cosv % 8 == 0 && (uintptr_t)sinv % 8 == 0));
   if (pairs_of_two) {
@@ -258,10 +341,10 @@ extern "C" int gb_rope_store(void* qkv, int dtype, int row_stride, const float* 
     GB_REQUIRE(grid.y <= 65535, "rope_store: %d heads are too many for one launch", units);
     if (dtype == kF32)
       hipLaunchKernelGGL(rope_store_kernel<float>, grid, dim3(threads), 0, stream, (float*)qkv, row_stride, cosv, sinv, slots,
-                         (float*)k_pages, (float*)v_pages, nh, nkv, hd, page_size, rotate);
+                         (float*)k_pages, (float*)v_pages, nh, nkv, hd, page_size, rotate, v_rows);
     else if (dtype == kBF16)
       hipLaunchKernelGGL(rope_store_kernel<bf16>, grid, dim3(threads), 0, stream, (bf16*)qkv, row_stride, cosv, sinv, slots,
-                         (bf16*)k_pages, (bf16*)v_pages, nh, nkv, hd, page_size, rotate);
+                         (bf16*)k_pages, (bf16*)v_pages, nh, nkv, hd, page_size, rotate, v_rows);
     else
       return fail("rope_store: unknown dtype %d", dtype);
     return launched("rope_store");

@@ -62,6 +62,15 @@ class StepContext:
     def buffer(self, name: str, shape, dtype) -> torch.Tensor:
         return self.workspace.buffer(name, shape, dtype)
 
+    def portions(self):
+        """The rows that are prompt portions, in the form ``ops.rope_store`` takes: requests with one row
+        come first in a step, one row each, so the portions are the requests and rows after them.
+        None when the step has none."""
+        n_dec = self.host["n_decode"]
+        if n_dec >= self.num_seqs:
+            return None
+        return (n_dec, self.q_start, self.q_len, self.pos0, n_dec, self.num_seqs - n_dec, int(self.host["max_q_len"]))
+
     # -------------------------------------------------------------------------------
     def attention(self, q: torch.Tensor, out: torch.Tensor, cache, n_heads: int, scale: float, window: int) -> None:
         """Paged attention of every row of the step over its request's cache.

@@ -41,7 +41,9 @@ _SIGS = {
         "gb_embed": [_vp, _i, _vp, _vp, _i, _i, _i, _vp],
         "gb_rmsnorm": [_vp, _vp, _i, _vp, _vp, _i, _i, _i, _f, _vp],
         "gb_rope_table": [_vp, _vp, _vp, _vp, _i, _i, _vp],
-        "gb_rope_store": [_vp, _i, _i, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _vp],
+        # qkv, dtype, stride, cos, sin, slots, k, v, n, nh, nkv, hd, page, rotate, v_rows, q_start, q_len, pos0,
+        # seq_base, n_seqs, max_q_len, stream
+        "gb_rope_store": [_vp, _i, _i, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _i, _vp, _vp, _vp, _i, _i, _i, _vp],
         "gb_silu_mul": [_vp, _vp, _i, _i, _i, _vp],
         "gb_copy_rows": [_vp, C.c_longlong, _vp, _vp, _i, _vp],
     },
@@ -180,9 +182,13 @@ def rope_table(positions: torch.Tensor, inv_freq: torch.Tensor, cos: torch.Tenso
 
 def rope_store(qkv: torch.Tensor, cos: Optional[torch.Tensor], sin: Optional[torch.Tensor],
                slots: Optional[torch.Tensor], k_pages: Optional[torch.Tensor], v_pages: Optional[torch.Tensor],
-               n_heads: int, n_kv_heads: int, head_dim: int, rotate: bool = True) -> None:
+               n_heads: int, n_kv_heads: int, head_dim: int, rotate: bool = True, portions=None) -> None:
     """Rotate the query and key heads of each stacked row in place and write keys and values
-    to the pages at ``slots``.  ``slots`` None: nothing is stored."""
+    to the pages at ``slots``.  ``slots`` None: nothing is stored.
+
+    ``portions = (first_row, q_start, q_len, pos0, seq_base, n_seqs, max_q_len)`` says that the rows from
+    first_row on are prompt portions of requests seq_base .. seq_base + n_seqs - 1 (device arrays indexed
+    by request): their values are then written to the transposed pages sixteen positions at a time."""
     _dev(qkv, cos, sin, slots, k_pages, v_pages)
     n = qkv.shape[0]
     stride = _rows(qkv, "qkv")
@@ -199,10 +205,20 @@ def rope_store(qkv: torch.Tensor, cos: Optional[torch.Tensor], sin: Optional[tor
         if cos.shape[1] != head_dim // 2 or cos.dtype != torch.float32 or not cos.is_contiguous() \
                 or not sin.is_contiguous():
             raise KernelError("rope_store: cos/sin must be contiguous float32 [n, head_dim/2]")
+    v_rows, q_start, q_len, pos0, seq_base, n_seqs, max_q_len = n, None, None, None, 0, 0, 0
+    if portions is not None and slots is not None:
+        v_rows, q_start, q_len, pos0, seq_base, n_seqs, max_q_len = portions
+        _dev(q_start, q_len, pos0)
+        for name, t in (("q_start", q_start), ("q_len", q_len), ("pos0", pos0)):
+            if t.dtype != torch.int32 or not t.is_contiguous() or t.numel() < seq_base + n_seqs:
+                raise KernelError(f"rope_store: {name} must be contiguous int32, one entry per request")
+        if not 0 <= v_rows <= n:
+            raise KernelError("rope_store: the first portion row lies outside the batch")
     lib = _lib("elementwise")
     _check(lib, lib.gb_rope_store(_p(qkv), dtype_code(qkv), stride, _p(cos), _p(sin), _p(slots), _p(k_pages),
                                   _p(v_pages), n, n_heads, n_kv_heads, head_dim, page_size, 1 if rotate else 0,
-                                  _stream()))
+                                  int(v_rows), _p(q_start), _p(q_len), _p(pos0), int(seq_base), int(n_seqs),
+                                  int(max_q_len), _stream()))
 
 
 def silu_mul(gate_up: torch.Tensor, out: torch.Tensor) -> None:

@@ -46,7 +46,8 @@ class Rotary(PositionEncoding):
         if head_dim != self.head_dim:
             raise ValueError(f"rotary built for head size {self.head_dim}, used with {head_dim}")
         cos, sin = self.table(ctx)
-        ops.rope_store(qkv, cos, sin, slots, k_pages, v_pages, n_heads, n_kv_heads, head_dim, rotate=True)
+        ops.rope_store(qkv, cos, sin, slots, k_pages, v_pages, n_heads, n_kv_heads, head_dim, rotate=True,
+                       portions=ctx.portions())
 
 
 class NoPosition(PositionEncoding):
@@ -54,4 +55,5 @@ class NoPosition(PositionEncoding):
 
     def apply_and_store(self, ctx, qkv, n_heads, n_kv_heads, head_dim, slots, k_pages, v_pages):
         if slots is not None:
-            ops.rope_store(qkv, None, None, slots, k_pages, v_pages, n_heads, n_kv_heads, head_dim, rotate=False)
+            ops.rope_store(qkv, None, None, slots, k_pages, v_pages, n_heads, n_kv_heads, head_dim, rotate=False,
+                           portions=ctx.portions())

@@ -219,6 +219,39 @@ def test_rope_table_and_rotation(hd, theta):
         assert torch.equal(got_v, qkv[i, (nh + nkv) * hd:].reshape(nkv, hd))
 
 
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("hd,page", [(16, 16), (64, 16), (128, 32), (40, 16)])
+def test_rope_store_writes_values_of_portions_in_tiles(dtype, hd, page):
+    """Values of prompt portions go to the transposed pages sixteen positions at a time: the pages must
+    come out as when every row is written by itself.  Portions that start in the middle of a page, end
+    in the middle of one, are shorter than a page, and single rows before them."""
+    from glassbox_amd import ops
+    nh, nkv = 3, 2
+    q_lens, pos0 = [1, 1, 40, 16, 7, 33], [9, 0, 5, 32, 0, 47]
+    n, n_dec = sum(q_lens), 2
+    q_start = np.concatenate([[0], np.cumsum(q_lens)[:-1]]).tolist()
+    pages_of, slots, next_page = [], [], 0
+    for length, first in zip(q_lens, pos0):                   # every request has pages of its own, in a scrambled order
+        count = -(-(first + length) // page)
+        mine = [next_page + (7 * i) % count for i in range(count)] if count % 7 else list(range(next_page, next_page + count))
+        next_page += count
+        pages_of.append(mine)
+        slots += [mine[p // page] * page + p % page for p in range(first, first + length)]
+    i32 = lambda v: torch.tensor(v, dtype=torch.int32, device=DEV)
+    qkv = rnd(n, (nh + 2 * nkv) * hd, seed=5).to(dtype)
+    cos, sin = torch.rand(n, hd // 2, device=DEV), torch.rand(n, hd // 2, device=DEV)
+    results = []
+    for portions in (None, (n_dec, i32(q_start), i32(q_lens), i32(pos0), n_dec, len(q_lens) - n_dec, max(q_lens))):
+        k_pages = torch.zeros(next_page, nkv, page, hd, device=DEV, dtype=dtype)
+        v_pages = torch.zeros(next_page, nkv, hd, page, device=DEV, dtype=dtype)
+        buf = to_dev(qkv.clone())
+        ops.rope_store(buf, cos, sin, i32(slots), k_pages, v_pages, nh, nkv, hd, portions=portions)
+        results.append((buf.cpu(), k_pages.cpu(), v_pages.cpu()))
+    for a, b in zip(*results):
+        assert torch.equal(a, b)
+    assert results[0][2].abs().sum() > 0
+
+
 # ---------------------------------------------------------------------- attention
 def paged_setup(ctx_lens, nkv, hd, page, seed, dtype, scatter=True):
     """Keys and values of several requests scattered over pages in a shuffled order."""
