@@ -23,7 +23,12 @@ TINY_B = dict(architectures=["LlamaForCausalLM"], hidden_size=96, intermediate_s
 TINY_C = dict(architectures=["LlamaForCausalLM"], hidden_size=80, intermediate_size=144, num_hidden_layers=2,
               num_attention_heads=6, num_key_value_heads=2, head_dim=48, vocab_size=331, rope_theta=130000.0,
               rms_norm_eps=3e-5, tie_word_embeddings=True, max_position_embeddings=512)
-TINY = {"A": TINY_A, "B": TINY_B, "C": TINY_C}
+# two layers of SmolLM2-360M's widths (a width of 960, 15 heads in 5 groups): large enough that the
+# products take their many-step paths and attention crosses many pages, small enough for the plain oracle
+MID_M = dict(architectures=["LlamaForCausalLM"], hidden_size=960, intermediate_size=2560, num_hidden_layers=2,
+             num_attention_heads=15, num_key_value_heads=5, vocab_size=1000, rope_theta=100000.0,
+             rms_norm_eps=1e-5, tie_word_embeddings=True, max_position_embeddings=8192)
+TINY = {"A": TINY_A, "B": TINY_B, "C": TINY_C, "M": MID_M}
 
 
 class ModelDirs:

@@ -25,8 +25,12 @@ def to_dev(t, dtype=None):
 GEMM_SHAPES_F32 = [(1, 32, 1), (8, 64, 2), (17, 64, 3), (33, 96, 9), (50, 160, 17), (331, 100, 70), (130, 257, 129)]
 GEMM_SHAPES_BF16 = [(1, 32, 1), (8, 64, 2), (17, 64, 3), (33, 96, 9), (50, 160, 17), (331, 104, 64), (331, 104, 65),
                     (130, 264, 129), (16, 2048, 8), (272, 72, 300), (49, 520, 33),
-                    # few rows of W and a long k: the skinny kernel splits k over workgroups
-                    (2048, 2048, 8), (2048, 8192, 8), (64, 2056, 1), (100, 4104, 33), (2048, 2048, 64), (48, 8192, 17)]
+                    # few rows of W and a long k: the skinny kernels split k over the waves of a workgroup
+                    (2048, 2048, 8), (2048, 8192, 8), (64, 2056, 1), (100, 4104, 33), (2048, 2048, 64), (48, 8192, 17),
+                    # the tiled kernel over many k-steps, k a multiple of its step and not, one and two
+                    # k-steps of prefetch (few and many tiles), fewer k-steps than the prefetch reaches
+                    (512, 1024, 200), (2048, 2048, 130), (96, 8192, 70), (1536, 1088, 520), (200, 128, 66), (3000, 192, 300),
+                    (640, 1032, 257)]
 
 
 @pytest.mark.parametrize("N,K,M", GEMM_SHAPES_F32)
@@ -59,7 +63,7 @@ def test_gemm_bf16(N, K, M, out):
 
 @pytest.mark.parametrize("I,K,M", [(8, 32, 1), (176, 64, 5), (144, 80, 16), (200, 2048, 17), (8192, 2048, 8), (88, 4104, 64),
                                    # more than 64 rows: the tiled kernel's epilogue
-                                   (176, 64, 130), (72, 264, 65), (1024, 520, 300)])
+                                   (176, 64, 130), (72, 264, 65), (1024, 520, 300), (2560, 960, 200), (1000, 2048, 129)])
 def test_gemm_bf16_fused_silu_mul(I, K, M):
     """Stacked gate/up rows with the activation applied in the product's epilogue
     (crates/glassbox-core/src/model.rs:335-340), against the formula in float64."""
@@ -73,7 +77,7 @@ def test_gemm_bf16_fused_silu_mul(I, K, M):
         ops.gemm(to_dev(a), to_dev(w), out, silu_mul=True)
         tol = 1e-4 + (2 ** -8) * want.abs().max().item() * (dt == torch.bfloat16)
         assert (out.cpu().double() - want).abs().max().item() <= tol
-    # twice in a row: the tile counters were left at zero
+    # twice in a row: the same again
     out2 = torch.empty(M, I, device=DEV, dtype=torch.float32)
     ops.gemm(to_dev(a), to_dev(w), out2, silu_mul=True)
     assert torch.equal(out2, out)

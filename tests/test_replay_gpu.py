@@ -1,6 +1,7 @@
 """The engine against the plain implementation under every way of cutting requests into steps:
 whole, last 32 tokens one by one, portions of changing size, and mixed batches with so few pages
 that they are used again; in 32-bit and in bfloat16."""
+import functools
 import json
 import os
 import subprocess
@@ -38,11 +39,11 @@ def make_requests_det(name, more=False):
             for i, (rid, n) in enumerate(lengths.items())}
 
 
-def check(folder, requests, got, dtype, what):
+def check(folder, requests, got, dtype, what, tol=None):
     for rid, toks in requests.items():
         want = helpers.plain_logits(folder, tuple(toks))
         assert got[rid].shape == want.shape, f"{what} {rid}: shape {got[rid].shape} vs {want.shape}"
-        bad = helpers.first_bad(got[rid], want, TOL[dtype])
+        bad = helpers.first_bad(got[rid], want, tol or TOL[dtype])
         assert bad is None, (f"{what}, request {rid} ({len(toks)} tokens), {dtype}: first wrong position {bad[0]} "
                              f"(page offset {bad[0] % 16}), max abs error {bad[1]:.3e}")
 
@@ -89,6 +90,31 @@ def test_mixed_batches_with_page_reuse(model_dirs, name, dtype):
         eng.cache.check_invariants()
         assert eng.cache.used_pages() == 0
         assert sum(len(t) for t in requests.values()) > peak, "the schedule did not reuse pages"
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_layers_of_real_width(engines, model_dirs, dtype):
+    """Two layers as wide as SmolLM2-360M's: the tiled products run many k-steps, prompt attention pairs
+    blocks of 32 tokens over dozens of pages, and a request of 700 tokens is cut in every way."""
+    folder = model_dirs.get("M")
+    vocab = helpers.TINY["M"]["vocab_size"]
+    requests = {"m0": helpers.random_tokens(vocab, 700, seed=31), "m1": helpers.random_tokens(vocab, 129, seed=32)}
+    eng = engines("M", dtype, max_tokens=2048)
+    # 32-bit: the same 1e-4.  bfloat16: rounding errors grow with the logits, whose root mean square is
+    # 0.63 here against 0.19 to 0.3 in the tiny models (measured: mean error 4.3e-3, largest 3.1e-2, the
+    # same at the first position as at the last and the same with the plain kernels): the tolerance
+    # keeps its ratio to them
+    tol = TOL[dtype] * (0.63 / 0.25 if dtype == "bfloat16" else 1.0)
+    check = functools.partial(globals()["check"], tol=tol)
+    for mode, make in (("whole", helpers.schedule_whole), ("tail32", helpers.schedule_tail),
+                       ("chunks", lambda r: helpers.schedule_chunks(r, sizes=(200, 2, 131, 64, 33, 300)))):
+        got = helpers.replay(eng, make(requests))
+        check(folder, requests, got, dtype, mode)
+    steps, peak = helpers.schedule_mixed(requests, seed=3, live=2)
+    got = helpers.replay(eng, steps)
+    check(folder, requests, got, dtype, "mixed")
+    eng.cache.check_invariants()
+    assert eng.cache.used_pages() == 0
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
