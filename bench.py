@@ -2,6 +2,7 @@
 """Decode and prefill throughput of the engine on SmolLM2-1.7B shapes with random weights.
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--batch 8] [--context 4096] [--layers 24]
+                    [--shapes smollm2-1.7b|smollm2-360m|llama-3-8b]
 
 A step is one decode step of the whole batch through Engine.step and the device sampler, the
 sampled tokens fed back as the next step's input.  The batch is first prefilled (through the same
@@ -13,10 +14,19 @@ import json
 import sys
 import time
 
-# SmolLM2-1.7B shapes: the benchmark configuration
-MODEL = dict(architectures=["LlamaForCausalLM"], hidden_size=2048, intermediate_size=8192, num_hidden_layers=24,
-             num_attention_heads=32, num_key_value_heads=32, vocab_size=49152, rope_theta=130000.0,
-             rms_norm_eps=1e-5, tie_word_embeddings=True, max_position_embeddings=8192)
+# SmolLM2-1.7B shapes: the benchmark configuration (the default); the others for measurements at further sizes
+SHAPES = {
+    "smollm2-1.7b": dict(architectures=["LlamaForCausalLM"], hidden_size=2048, intermediate_size=8192,
+                         num_hidden_layers=24, num_attention_heads=32, num_key_value_heads=32, vocab_size=49152,
+                         rope_theta=130000.0, rms_norm_eps=1e-5, tie_word_embeddings=True, max_position_embeddings=8192),
+    "smollm2-360m": dict(architectures=["LlamaForCausalLM"], hidden_size=960, intermediate_size=2560,
+                         num_hidden_layers=32, num_attention_heads=15, num_key_value_heads=5, vocab_size=49152,
+                         rope_theta=100000.0, rms_norm_eps=1e-5, tie_word_embeddings=True, max_position_embeddings=8192),
+    "llama-3-8b": dict(architectures=["LlamaForCausalLM"], hidden_size=4096, intermediate_size=14336,
+                       num_hidden_layers=32, num_attention_heads=32, num_key_value_heads=8, vocab_size=128256,
+                       rope_theta=500000.0, rms_norm_eps=1e-5, tie_word_embeddings=False, max_position_embeddings=8192),
+}
+NAMES = {"smollm2-1.7b": "SmolLM2-1.7B shapes", "smollm2-360m": "SmolLM2-360M shapes", "llama-3-8b": "Llama-3-8B shapes"}
 PEAK = {"hbm_gbs": 8000.0, "bf16_tflops": 2500.0, "fp32_tflops": 157.3}   # MI355X, dense
 PREFILL_TOKENS = 2048
 
@@ -28,7 +38,8 @@ def main() -> int:
     ap.add_argument("--warmup", type=int, default=8)
     ap.add_argument("--batch", type=int, default=8)
     ap.add_argument("--context", type=int, default=4096)
-    ap.add_argument("--layers", type=int, default=MODEL["num_hidden_layers"])
+    ap.add_argument("--shapes", default="smollm2-1.7b", choices=sorted(SHAPES))
+    ap.add_argument("--layers", type=int, default=None, help="fewer layers than the model has (both numbers are reported)")
     ap.add_argument("--dtype", default="bfloat16", choices=["bfloat16", "float32"])
     ap.add_argument("--no-points", action="store_true", help="skip the batch 1 and 64 points")
     ap.add_argument("--only", choices=["decode", "prefill"], default=None,
@@ -45,7 +56,8 @@ def main() -> int:
     from glassbox_amd.engine.decode_loop import DecodeLoop
     from glassbox_amd.weights import build_model, init_random
 
-    cfg = config_from_dict(dict(MODEL, num_hidden_layers=a.layers))
+    MODEL = SHAPES[a.shapes]
+    cfg = config_from_dict(dict(MODEL, num_hidden_layers=a.layers or MODEL["num_hidden_layers"]))
     model = build_model(cfg)
     init_random(model, seed=0, dtype=a.dtype, device="cuda:0")
     batches = [a.batch] + ([] if a.no_points else [b for b in (1, 64) if b != a.batch])
@@ -127,11 +139,12 @@ def main() -> int:
             points[f"decode_b{b}"] = round(b * k / pdt, 1)
 
     out = {
-        "metric": "decode tok/s at batch 8, SmolLM2-1.7B shapes, context 4096 (prefill tok/s at 2,048 tokens beside it)",
+        "metric": f"decode tok/s at batch {a.batch}, {NAMES[a.shapes]}, context {a.context} "
+                  "(prefill tok/s at 2,048 tokens beside it)",
         "value": round(value, 1), "unit": "tok/s", "n_gpus": 1, "steps": a.steps, "warmup": a.warmup,
         "ms_per_step": round(step_s * 1e3, 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "bf16" if a.dtype == "bfloat16" else "fp32", "data": "synthetic token ids, random N(0, 0.02) weights",
-        "config": {"model": "SmolLM2-1.7B shapes", "layers": cfg.num_hidden_layers, "layers_of_model": MODEL["num_hidden_layers"],
+        "config": {"model": NAMES[a.shapes], "layers": cfg.num_hidden_layers, "layers_of_model": MODEL["num_hidden_layers"],
                    "hidden": d, "heads": cfg.num_attention_heads, "kv_heads": cfg.num_key_value_heads,
                    "head_dim": cfg.head_size, "intermediate": I, "vocab": vocab, "rope_theta": cfg.rope_theta,
                    "rms_norm_eps": cfg.rms_norm_eps, "tied": cfg.tie_word_embeddings, "global_batch": a.batch,
