@@ -33,6 +33,23 @@ __device__ __forceinline__ bf16x8 zero8() {
   return z;
 }
 
+// What a product of at most 8 rows may do for the RMS norm that follows it or precedes it.
+//  * emit (the folded kernel, accumulating into the float32 residual): besides the new residual r it
+//    writes h[m, n] = bf16(gamma[n] * r[m, n]), the operand of the next product, and for every tile of 8
+//    columns the sums over them of r[m, n]^2 to ss[tile * 8 + m]: the next norm's pass over the residual
+//    is done where the residual is made.
+//  * parts (the skinny kernel): the rows of A are such an h; the product is scaled by
+//    1 / sqrt(sum of the n_parts partial sums of row m / K + eps), added up in the order of the tiles.
+struct NormExtras {
+  const void* emit_gamma;
+  int emit_gamma_f32;
+  bf16* emit_h;
+  int emit_ldh;
+  float* emit_ss;
+  const float* parts;
+  int n_parts;
+};
+
 template <typename CT> __device__ __forceinline__ void store_c(CT* c, float v, int accumulate);
 template <> __device__ __forceinline__ void store_c<float>(float* c, float v, int accumulate) { *c = accumulate ? *c + v : v; }
 template <> __device__ __forceinline__ void store_c<bf16>(bf16* c, float v, int) { *c = (bf16)v; }
@@ -314,11 +331,23 @@ template <int MT, int WAVES, int ITERS, int RT, int EPI, bool RMS, typename CT>
 __global__ __launch_bounds__(WAVES * 64) void gemm_skinny_kernel(const void* __restrict__ a, int lda,
                                                                  const bf16* __restrict__ w, int ldw, CT* __restrict__ c,
                                                                  int ldc, int M, int N, int K, const void* __restrict__ gamma,
-                                                                 int gamma_f32, float eps) {
+                                                                 int gamma_f32, float eps, const float* __restrict__ parts,
+                                                                 int n_parts) {
   __shared__ float part[WAVES][RT][MT][64][4];
   __shared__ float sspart[RMS ? WAVES : 1][MT][64];
+  __shared__ float red[64][8];
   const int tid = threadIdx.x, lane = tid % 64, wave = tid / 64;
   const int r = lane % 16, q = lane / 16;
+  if (!RMS && parts != nullptr) {
+    // partial sums of squares of the (at most 8) rows, one per tile of the product that made them:
+    // 64 threads a row add up every 64th, the epilogue adds up those 64, both in a fixed order
+    for (int t = tid; t < 512; t += WAVES * 64) {
+      const int m = t & 7, j = t >> 3;
+      float sum = 0.f;
+      for (int p = j; p < n_parts; p += 64) sum += parts[p * 8 + m];
+      red[j][m] = sum;
+    }
+  }
   const bf16* wrow[RT];
   bool row_ok[RT];
 #pragma unroll
@@ -414,6 +443,11 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_skinny_kernel(const void* __r
 #pragma unroll
         for (int qq = 0; qq < 4; ++qq) tot += sspart[wv][t][l % 16 + 16 * qq];
       scale = 1.0f / sqrtf(tot / (float)K + eps);
+    } else if (parts != nullptr && l % 16 < 8) {
+      float tot = 0.f;
+#pragma unroll 8
+      for (int j = 0; j < 64; ++j) tot += red[j][l % 16];
+      scale = 1.0f / sqrtf(tot / (float)K + eps);
     }
 #pragma unroll
     for (int rt = 0; rt < RT; ++rt) {
@@ -471,10 +505,11 @@ template <int WAVES, int ITERS, int RT, int EPI, bool RMS, typename CT>
 __global__ __launch_bounds__(WAVES * 64) void gemm_fold_kernel(const void* __restrict__ a, int lda,
                                                                const bf16* __restrict__ w, int ldw, CT* __restrict__ c,
                                                                int ldc, int M, int N, int K, const void* __restrict__ gamma,
-                                                               int gamma_f32, float eps) {
+                                                               int gamma_f32, float eps, NormExtras extra) {
   static_assert(EPI != EPI_SILU_MUL && WAVES >= 4, "folded tiles store or accumulate; the first four waves finish");
   __shared__ float part[WAVES][RT][64][4];
   __shared__ float sspart[RMS ? WAVES : 1][64];
+  __shared__ float squares[RT][8][8];
   const int tid = threadIdx.x, lane = tid % 64, wave = tid / 64;
   const int r = lane % 16, q = lane / 16;
   const int r8 = r & 7, khalf = (r >> 3) * 64;  // row of W and of A; which half of a k block
@@ -527,9 +562,11 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_fold_kernel(const void* __res
   // D[n, m]: lane l holds column m = l%16 and rows n = 4*(l/16) + e; thread tid owns cell (l = tid/4, e = tid%4)
   const int l = tid / 4, e = tid % 4;
   const int nrow = 4 * (l / 16) + e, m = l % 16;
-  if (nrow >= 8 || m >= 8) return;
+  const bool emits = EPI == EPI_ACCUMULATE && extra.emit_h != nullptr;
+  const bool mine = nrow < 8 && m < 8;
+  if (!mine && !emits) return;
   float scale = 1.f;
-  if (RMS) {
+  if (RMS && mine) {
     // sum(x^2) of row m: its k were spread over the waves, the four lane groups and the two halves
     float tot = 0.f;
 #pragma unroll
@@ -540,11 +577,32 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_fold_kernel(const void* __res
   }
 #pragma unroll
   for (int rt = 0; rt < RT; ++rt) {
-    float sum = 0.f;
-#pragma unroll
-    for (int wv = 0; wv < WAVES; ++wv) sum += part[wv][rt][l][e] + part[wv][rt][l + 40][e];  // cell (n + 8, m + 8)
     const int n = (blockIdx.x * RT + rt) * 8 + nrow;
-    if (m < M && n < N) store_c<CT>(c + (size_t)m * ldc + n, sum * scale, EPI == EPI_ACCUMULATE);
+    float now = 0.f;  // the cell's new value
+    if (mine && m < M && n < N) {
+      float sum = 0.f;
+#pragma unroll
+      for (int wv = 0; wv < WAVES; ++wv) sum += part[wv][rt][l][e] + part[wv][rt][l + 40][e];  // cell (n + 8, m + 8)
+      CT* cell = c + (size_t)m * ldc + n;
+      now = EPI == EPI_ACCUMULATE ? (float)*cell + sum * scale : sum * scale;
+      *cell = (CT)now;
+      if (emits) {
+        const float g = extra.emit_gamma_f32 ? ((const float*)extra.emit_gamma)[n] : (float)((const bf16*)extra.emit_gamma)[n];
+        extra.emit_h[(size_t)m * extra.emit_ldh + n] = (bf16)(g * now);
+      }
+    }
+    if (emits && mine) squares[rt][m][nrow] = now * now;
+  }
+  if (!emits) return;
+  __syncthreads();  // the waves that are still here
+  if (mine && nrow == 0) {
+#pragma unroll
+    for (int rt = 0; rt < RT; ++rt) {
+      float tot = 0.f;
+#pragma unroll
+      for (int j = 0; j < 8; ++j) tot += squares[rt][m][j];
+      extra.emit_ss[(size_t)(blockIdx.x * RT + rt) * 8 + m] = tot;
+    }
   }
 }
 
@@ -554,7 +612,7 @@ inline bool fold_pays(int M, int N) { return M <= 8 && (N + 15) / 16 < 256; }
 
 template <int EPI, bool RMS, typename CT>
 int launch_fold(const void* a, int lda, const bf16* w, int ldw, CT* c, int ldc, int M, int N, int K, const void* gamma,
-                int gamma_f32, float eps, hipStream_t stream) {
+                int gamma_f32, float eps, const NormExtras& extra, hipStream_t stream) {
   const int tiles = (N + 7) / 8, blocks = (K + 127) / 128;  // 128-wide k blocks
   const int waves = blocks >= 16 ? 16 : 4;
   const int rt = tiles >= 512 ? 2 : 1;
@@ -562,7 +620,7 @@ int launch_fold(const void* a, int lda, const bf16* w, int ldw, CT* c, int ldc, 
 #define GB_CFG(WV, IT, RT)                                                                                                \
   if (waves == WV && iters == IT && rt == RT)                                                                             \
     hipLaunchKernelGGL((gemm_fold_kernel<WV, IT, RT, EPI, RMS, CT>), dim3((tiles + RT - 1) / RT), dim3(WV * 64), 0, stream, \
-                       a, lda, w, ldw, c, ldc, M, N, K, gamma, gamma_f32, eps);
+                       a, lda, w, ldw, c, ldc, M, N, K, gamma, gamma_f32, eps, extra);
   GB_CFG(4, 1, 1) GB_CFG(4, 1, 2) GB_CFG(4, 2, 1) GB_CFG(4, 2, 2)
   GB_CFG(16, 1, 1) GB_CFG(16, 1, 2) GB_CFG(16, 2, 1) GB_CFG(16, 2, 2)
 #undef GB_CFG
@@ -592,13 +650,13 @@ inline void skinny_plan(int tiles, int K, int mt, int* waves, int* iters, int* r
 
 template <int MT, int EPI, bool RMS, typename CT>
 int launch_skinny_mt(int tiles, const void* a, int lda, const bf16* w, int ldw, CT* c, int ldc, int M, int N, int K,
-                     const void* gamma, int gamma_f32, float eps, hipStream_t stream) {
+                     const void* gamma, int gamma_f32, float eps, const NormExtras& extra, hipStream_t stream) {
   int waves, iters, rt;
   skinny_plan(tiles, K, MT, &waves, &iters, &rt);
 #define GB_CFG(WV, IT, RT)                                                                                                 \
   if (waves == WV && iters == (IT) && rt == RT)                                                                            \
     hipLaunchKernelGGL((gemm_skinny_kernel<MT, WV, (IT), RT, EPI, RMS, CT>), dim3((tiles + RT - 1) / RT), dim3(WV * 64), 0,  \
-                       stream, a, lda, w, ldw, c, ldc, M, N, K, gamma, gamma_f32, eps);
+                       stream, a, lda, w, ldw, c, ldc, M, N, K, gamma, gamma_f32, eps, extra.parts, extra.n_parts);
   // the configurations skinny_plan can ask for: two loads in flight only with one column block
   GB_CFG(4, 1, 1) GB_CFG(4, 1, 2) GB_CFG(16, 1, 1) GB_CFG(16, 1, 2)
   if (MT == 1) {
@@ -610,14 +668,14 @@ int launch_skinny_mt(int tiles, const void* a, int lda, const bf16* w, int ldw, 
 
 template <int EPI, bool RMS, typename CT>
 int launch_skinny(const void* a, int lda, const bf16* w, int ldw, CT* c, int ldc, int M, int N, int K, const void* gamma,
-                  int gamma_f32, float eps, hipStream_t stream) {
+                  int gamma_f32, float eps, const NormExtras& extra, hipStream_t stream) {
   const int tiles = EPI == EPI_SILU_MUL ? (N / 2 + 7) / 8 : (N + 15) / 16;
   const int mt = (M + 15) / 16;
 #define GB_MT(T) \
-  if (mt == T) return launch_skinny_mt<T, EPI, RMS, CT>(tiles, a, lda, w, ldw, c, ldc, M, N, K, gamma, gamma_f32, eps, stream);
+  if (mt == T) return launch_skinny_mt<T, EPI, RMS, CT>(tiles, a, lda, w, ldw, c, ldc, M, N, K, gamma, gamma_f32, eps, extra, stream);
   GB_MT(1) GB_MT(2) GB_MT(3)
 #undef GB_MT
-  return launch_skinny_mt<4, EPI, RMS, CT>(tiles, a, lda, w, ldw, c, ldc, M, N, K, gamma, gamma_f32, eps, stream);
+  return launch_skinny_mt<4, EPI, RMS, CT>(tiles, a, lda, w, ldw, c, ldc, M, N, K, gamma, gamma_f32, eps, extra, stream);
 }
 
 }  // namespace
@@ -626,8 +684,16 @@ int launch_skinny(const void* a, int lda, const bf16* w, int ldw, CT* c, int ldc
 // gamma != nullptr (at most 64 rows, bfloat16 C, epilogue 0 or 2): a is the float32 residual and the
 // product is that of its RMS-normed rows: bf16(gamma * x) as the operand, 1/sqrt(mean(x^2) + eps) on
 // the result.
+// emit_h != nullptr (accumulating product that gb_gemm_bf16_emit_parts accepts): the next norm's operand and
+// partial sums are written beside the residual, see NormExtras.  parts != nullptr (at most 8 rows, no
+// gamma): the rows of a are such an operand and the product is scaled by the norm's factor from n_parts
+// partial sums; eps is that norm's.
+extern "C" int gb_gemm_bf16_emit_parts(int M, int N) { return fold_pays(M, N) ? (N + 7) / 8 : 0; }
+
 extern "C" int gb_gemm_bf16(const void* a, int lda, const void* w, int ldw, void* c, int ldc, int c_dtype, int M, int N,
-                            int K, int epilogue, const void* gamma, int gamma_dtype, float eps, hipStream_t stream) {
+                            int K, int epilogue, const void* gamma, int gamma_dtype, float eps, const void* emit_gamma,
+                            int emit_gamma_dtype, void* emit_h, int emit_ldh, float* emit_ss, const float* parts, int n_parts,
+                            hipStream_t stream) {
   GB_REQUIRE(M >= 0 && N > 0 && K > 0, "gemm_bf16: bad sizes M=%d N=%d K=%d", M, N, K);
   GB_REQUIRE(K % 8 == 0, "gemm_bf16: the inner size K=%d must be a multiple of 8 (16-byte operand loads)", K);
   GB_REQUIRE(ldw % 8 == 0 && lda % (gamma ? 4 : 8) == 0, "gemm_bf16: row strides (%d, %d) must keep rows 16-byte aligned", lda, ldw);
@@ -641,21 +707,27 @@ extern "C" int gb_gemm_bf16(const void* a, int lda, const void* w, int ldw, void
   GB_REQUIRE(!gamma || (M <= 64 && c_dtype == kBF16 && epilogue != EPI_ACCUMULATE && ((uintptr_t)gamma % 16 == 0) &&
                         (gamma_dtype == kF32 || gamma_dtype == kBF16)),
              "gemm_bf16: the fused RMS norm serves up to 64 rows with a bfloat16 result");
+  GB_REQUIRE(!emit_h || (epilogue == EPI_ACCUMULATE && fold_pays(M, N) && emit_gamma && emit_ss && emit_ldh >= N &&
+                         (emit_gamma_dtype == kF32 || emit_gamma_dtype == kBF16)),
+             "gemm_bf16: only an accumulating product that gb_gemm_bf16_emit_parts accepts can prepare the next norm");
+  GB_REQUIRE(!parts || (M <= 8 && !gamma && n_parts > 0 && epilogue != EPI_ACCUMULATE),
+             "gemm_bf16: partial sums of a norm go with at most 8 rows, no gamma, and a storing epilogue");
+  const NormExtras extra{emit_gamma, emit_gamma_dtype == kF32, (bf16*)emit_h, emit_ldh, emit_ss, parts, n_parts};
   if (M == 0) return 0;
   const bf16* W = (const bf16*)w;
   if (M <= 64) {
     const int gf = gamma_dtype == kF32;
-    if (fold_pays(M, N) && epilogue != EPI_SILU_MUL) {
-      if (gamma) return launch_fold<EPI_STORE, true, bf16>(a, lda, W, ldw, (bf16*)c, ldc, M, N, K, gamma, gf, eps, stream);
-      if (epilogue == EPI_ACCUMULATE) return launch_fold<EPI_ACCUMULATE, false, float>(a, lda, W, ldw, (float*)c, ldc, M, N, K, nullptr, 0, 0.f, stream);
-      if (c_dtype == kF32) return launch_fold<EPI_STORE, false, float>(a, lda, W, ldw, (float*)c, ldc, M, N, K, nullptr, 0, 0.f, stream);
-      return launch_fold<EPI_STORE, false, bf16>(a, lda, W, ldw, (bf16*)c, ldc, M, N, K, nullptr, 0, 0.f, stream);
+    if (fold_pays(M, N) && epilogue != EPI_SILU_MUL && !parts) {
+      if (gamma) return launch_fold<EPI_STORE, true, bf16>(a, lda, W, ldw, (bf16*)c, ldc, M, N, K, gamma, gf, eps, extra, stream);
+      if (epilogue == EPI_ACCUMULATE) return launch_fold<EPI_ACCUMULATE, false, float>(a, lda, W, ldw, (float*)c, ldc, M, N, K, nullptr, 0, 0.f, extra, stream);
+      if (c_dtype == kF32) return launch_fold<EPI_STORE, false, float>(a, lda, W, ldw, (float*)c, ldc, M, N, K, nullptr, 0, 0.f, extra, stream);
+      return launch_fold<EPI_STORE, false, bf16>(a, lda, W, ldw, (bf16*)c, ldc, M, N, K, nullptr, 0, 0.f, extra, stream);
     }
     if (gamma) {
-      if (epilogue == EPI_STORE) return launch_skinny<EPI_STORE, true, bf16>(a, lda, W, ldw, (bf16*)c, ldc, M, N, K, gamma, gf, eps, stream);
-      return launch_skinny<EPI_SILU_MUL, true, bf16>(a, lda, W, ldw, (bf16*)c, ldc, M, N, K, gamma, gf, eps, stream);
+      if (epilogue == EPI_STORE) return launch_skinny<EPI_STORE, true, bf16>(a, lda, W, ldw, (bf16*)c, ldc, M, N, K, gamma, gf, eps, extra, stream);
+      return launch_skinny<EPI_SILU_MUL, true, bf16>(a, lda, W, ldw, (bf16*)c, ldc, M, N, K, gamma, gf, eps, extra, stream);
     }
-#define GB_SK(EPI, CT) return launch_skinny<EPI, false, CT>(a, lda, W, ldw, (CT*)c, ldc, M, N, K, nullptr, 0, 0.f, stream)
+#define GB_SK(EPI, CT) return launch_skinny<EPI, false, CT>(a, lda, W, ldw, (CT*)c, ldc, M, N, K, nullptr, 0, eps, extra, stream)
     if (epilogue == EPI_STORE && c_dtype == kF32) GB_SK(EPI_STORE, float);
     if (epilogue == EPI_STORE && c_dtype == kBF16) GB_SK(EPI_STORE, bf16);
     if (epilogue == EPI_ACCUMULATE) GB_SK(EPI_ACCUMULATE, float);

@@ -51,8 +51,10 @@ _SIGS = {
         "gb_gemm_f32": [_vp, _i, _vp, _i, _vp, _i, _i, _i, _i, _i, _vp],
     },
     "gemm_bf16": {
-        # a, lda, w, ldw, c, ldc, c_dtype, M, N, K, epilogue, gamma, gamma_dtype, eps, stream
-        "gb_gemm_bf16": [_vp, _i, _vp, _i, _vp, _i, _i, _i, _i, _i, _i, _vp, _i, _f, _vp],
+        # a, lda, w, ldw, c, ldc, c_dtype, M, N, K, epilogue, gamma, gamma_dtype, eps,
+        # emit_gamma, emit_gamma_dtype, emit_h, emit_ldh, emit_ss, parts, n_parts, stream
+        "gb_gemm_bf16": [_vp, _i, _vp, _i, _vp, _i, _i, _i, _i, _i, _i, _vp, _i, _f, _vp, _i, _vp, _i, _vp, _vp, _i, _vp],
+        "gb_gemm_bf16_emit_parts": [_i, _i],
     },
     "attention_plain": {
         "gb_attention_plain": [_vp, _i, _vp, _i, _i, _vp, _vp, _vp, _i, _vp, _vp, _i, _i, _i, _i, _i, _f, _i, _vp],
@@ -251,15 +253,26 @@ SILU_MUL_MAX_ROWS = 64
 FUSED_NORM_MAX_ROWS = 16   # measured: beyond one 16-row block the re-reading of float32 rows costs more than a norm pass
 
 
+def gemm_emit_parts(rows: int, n: int) -> int:
+    """How many partial sums an accumulating bfloat16 product of ``rows`` rows and ``n`` columns writes when
+    asked to prepare the norm that follows (``gemm(..., emit=...)``); 0 if that product cannot."""
+    return int(_lib("gemm_bf16").gb_gemm_bf16_emit_parts(int(rows), int(n)))
+
+
 def gemm(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor, accumulate: bool = False, silu_mul: bool = False,
-         rms: Optional[tuple] = None) -> None:
+         rms: Optional[tuple] = None, emit: Optional[tuple] = None, rms_parts: Optional[tuple] = None) -> None:
     """out (+)= a . w^T with w in the [out features, in features] layout.
     float32 operands take the true 32-bit kernel; bfloat16 operands the matrix-core kernels,
     with out in bfloat16 or float32 (float32 when accumulating into the residual).
     ``silu_mul`` (bfloat16, at most 64 rows): w stacks gate rows over up rows and out[m, j] =
     silu(a . gate_j) * (a . up_j), of half as many columns.
     ``rms=(gamma, eps)`` (bfloat16 w and out, at most 64 rows): a is the float32 residual and the
-    product is that of its RMS-normed rows, the norm computed inside the product's kernel."""
+    product is that of its RMS-normed rows, the norm computed inside the product's kernel.
+    ``emit=(gamma, h, parts)`` (accumulating bfloat16 product with ``gemm_emit_parts(M, N) > 0``): besides
+    the new residual r in out, h[m, n] = bf16(gamma[n] r[m, n]) and float32 parts[tile, m] (8 columns a
+    tile) of sum(r^2) are written: the work of the RMS norm that reads the residual next.
+    ``rms_parts=(parts, n_parts, eps)`` (at most 8 rows): a is such an h, and the product is scaled by
+    1 / sqrt(sum(parts[:, m]) / K + eps) to that of the normed rows."""
     _dev(a, w, out)
     M, K = a.shape
     N = w.shape[0]
@@ -274,9 +287,12 @@ def gemm(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor, accumulate: bool =
         if (a.dtype != torch.float32 or w.dtype != torch.bfloat16 or out.dtype != torch.bfloat16 or accumulate
                 or M > 64 or gamma.numel() != K or not gamma.is_contiguous()):
             raise KernelError("gemm: the fused RMS norm takes float32 rows (at most 64), bfloat16 weights and result")
+        if emit is not None or rms_parts is not None:
+            raise KernelError("gemm: one way of fusing the norm at a time")
         lib = _lib("gemm_bf16")
         _check(lib, lib.gb_gemm_bf16(_p(a), lda, _p(w), ldw, _p(out), ldc, BF16, M, N, K, 2 if silu_mul else 0,
-                                     _p(gamma), dtype_code(gamma), float(eps), _stream()))
+                                     _p(gamma), dtype_code(gamma), float(eps), None, 0, None, 0, None, None, 0,
+                                     _stream()))
     elif a.dtype == torch.float32 and w.dtype == torch.float32:
         if out.dtype != torch.float32:
             raise KernelError("gemm: 32-bit operands need a 32-bit result")
@@ -286,8 +302,29 @@ def gemm(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor, accumulate: bool =
         if accumulate and out.dtype != torch.float32:
             raise KernelError("gemm: accumulation is into a 32-bit result")
         lib = _lib("gemm_bf16")
+        e_gamma = e_h = e_ss = parts = None
+        e_ldh = n_parts = 0
+        eps = 0.0
+        if emit is not None:
+            e_gamma, e_h, e_ss = emit
+            _dev(e_gamma, e_h, e_ss)
+            want = gemm_emit_parts(M, N)
+            if (not accumulate or want == 0 or e_gamma.numel() != N or not e_gamma.is_contiguous()
+                    or e_h.dtype != torch.bfloat16 or e_h.shape != (M, N) or e_ss.dtype != torch.float32
+                    or not e_ss.is_contiguous() or e_ss.numel() < want * 8):
+                raise KernelError("gemm: emit needs an accumulating product that gemm_emit_parts accepts, gamma of N "
+                                  "entries, a bfloat16 [M, N] operand buffer and 8 float32 per part")
+            e_ldh = _rows(e_h, "emit h")
+        if rms_parts is not None:
+            parts, n_parts, eps = rms_parts
+            _dev(parts)
+            if (M > 8 or accumulate or parts.dtype != torch.float32 or not parts.is_contiguous()
+                    or parts.numel() < n_parts * 8 or n_parts <= 0):
+                raise KernelError("gemm: partial sums of a norm go with at most 8 rows and a storing product")
         _check(lib, lib.gb_gemm_bf16(_p(a), lda, _p(w), ldw, _p(out), ldc, dtype_code(out), M, N, K,
-                                     2 if silu_mul else (1 if accumulate else 0), None, 0, 0.0, _stream()))
+                                     2 if silu_mul else (1 if accumulate else 0), None, 0, float(eps),
+                                     _p(e_gamma), dtype_code(e_gamma) if e_gamma is not None else 0, _p(e_h), e_ldh,
+                                     _p(e_ss), _p(parts), int(n_parts), _stream()))
     else:
         raise KernelError(f"gemm: operand types {a.dtype} and {w.dtype} do not match a kernel")
 

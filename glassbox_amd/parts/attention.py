@@ -15,7 +15,7 @@ from typing import Dict, Optional
 import torch
 
 from .. import ops
-from .base import FULL, WINDOW, CacheSpec, LayerCache, Mixer, PositionEncoding, TensorSpec
+from .base import FULL, WINDOW, CacheSpec, LayerCache, Mixer, PositionEncoding, PreNormed, TensorSpec, emit_target
 
 
 class PagedAttention(Mixer):
@@ -55,15 +55,21 @@ class PagedAttention(Mixer):
         self.wo = tensors["o_proj.weight"].contiguous()
 
     accepts_fused_norm = True
+    accepts_emit_norm = True
 
-    def forward(self, ctx, h, residual, cache: Optional[LayerCache], norm=None):
-        """``norm=(gamma, eps)``: h is the un-normed float32 residual and the first product norms it."""
+    def forward(self, ctx, h, residual, cache: Optional[LayerCache], norm=None, emit=None):
+        """``norm=(gamma, eps)``: h is the un-normed float32 residual and the first product norms it;
+        ``norm=PreNormed``: the product before has done most of that.  ``emit=(gamma, eps)``: the output
+        projection may prepare the norm that reads the residual next (returns a PreNormed if it did)."""
         if cache is None or cache.k_pages is None:
             raise ValueError("PagedAttention needs a layer cache with pages")
         n = h.shape[0]
         rows = self.q_dim + (0 if self.shares_kv else 2 * self.kv_dim)
         qkv = ctx.buffer("qkv", (n, rows), ctx.dtype)
-        ops.gemm(h, self.wqkv, qkv, rms=norm)
+        if isinstance(norm, PreNormed):
+            ops.gemm(norm.rows, self.wqkv, qkv, rms_parts=norm.as_gemm_arg())
+        else:
+            ops.gemm(h, self.wqkv, qkv, rms=norm)
         write = cache.writable and not self.shares_kv
         self.position.apply_and_store(
             ctx, qkv, self.n_heads, 0 if self.shares_kv else self.n_kv_heads, self.head_dim,
@@ -71,4 +77,6 @@ class PagedAttention(Mixer):
             cache.v_pages if write else None)
         att = ctx.buffer("att", (n, self.q_dim), ctx.dtype)
         ctx.attention(qkv[:, :self.q_dim], att, cache, self.n_heads, self.scale, self.window)
-        ops.gemm(att, self.wo, residual, accumulate=True)
+        target, handed_on = emit_target(ctx, n, self.width, emit, "mixer")
+        ops.gemm(att, self.wo, residual, accumulate=True, emit=target)
+        return handed_on

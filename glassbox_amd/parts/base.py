@@ -18,11 +18,17 @@ Interfaces (all activations are [tokens, width] tensors on the device;
       .state_spec  -> StateSpec | None              fixed-size per-request state it needs
   FeedForward.forward(ctx, h, residual)             adds its output into ``residual`` (float32)
   Block.forward(ctx, x, cache)                      one layer: arrangement of the four above
+
+Optional, for steps of few rows (each part says by a class attribute whether it takes part):
+  ``accepts_fused_norm``: forward(..., norm=) takes the un-normed residual and either the norm's
+      ``(gamma, eps)`` or a ``PreNormed`` and lets its first product do the norm's work;
+  ``accepts_emit_norm``: forward(..., emit=(gamma, eps)) may let its last product, which adds into the
+      residual, prepare the norm that reads the residual next, and returns a ``PreNormed`` if it did.
 """
 from __future__ import annotations
 
 from dataclasses import dataclass
-from typing import Dict, Iterator, Optional, Tuple
+from typing import Dict, Iterator, NamedTuple, Optional, Tuple
 
 import torch
 
@@ -106,6 +112,35 @@ class Norm(Part):
 class PositionEncoding(Part):
     def apply_and_store(self, ctx, qkv, n_heads, n_kv_heads, head_dim, slots, k_pages, v_pages) -> None:
         raise NotImplementedError
+
+
+class PreNormed(NamedTuple):
+    """The work of an RMS norm done by the product that made the residual: ``rows`` = bf16(gamma * residual)
+    and partial sums of the residual's squares, ``parts[:n_parts]``, 8 floats a part (row m in column m).
+    The product that takes it scales its result by 1 / sqrt(sum of parts / width + eps)."""
+    rows: torch.Tensor
+    parts: torch.Tensor
+    n_parts: int
+    eps: float
+
+    def as_gemm_arg(self):
+        return (self.parts, self.n_parts, self.eps)
+
+
+def emit_target(ctx, n: int, width: int, emit, tag: str):
+    """Buffers for a product of n rows and ``width`` columns that is asked (``emit=(gamma, eps)``) to prepare
+    the next norm: ``(gemm emit argument, PreNormed to hand on)``, or ``(None, None)`` when nothing is asked
+    or this step's product cannot do it (more than 8 rows, a 32-bit step, too wide a residual)."""
+    from .. import ops
+    if emit is None or ctx.dtype != torch.bfloat16 or not ctx.fuse_norms:
+        return None, None
+    n_parts = ops.gemm_emit_parts(n, width)
+    if n_parts == 0:
+        return None, None
+    gamma, eps = emit
+    rows = ctx.buffer(f"prenorm_rows_{tag}", (n, width), torch.bfloat16)
+    parts = ctx.buffer(f"prenorm_parts_{tag}", (n_parts, 8), torch.float32)
+    return (gamma, rows, parts), PreNormed(rows, parts, n_parts, float(eps))
 
 
 class Mixer(Part):

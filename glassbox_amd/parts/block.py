@@ -4,7 +4,10 @@ float32 in both precisions; mixer and feed-forward add into it themselves.
 
 A mixer or feed-forward with ``accepts_fused_norm = True`` may be handed the un-normed residual
 and the norm's constants instead of normed rows (``forward(..., norm=(gamma, eps))``): its first
-matrix product then computes the norm on the way (few rows only; ``Norm.fuse_spec`` decides)."""
+matrix product then computes the norm on the way (few rows only; ``Norm.fuse_spec`` decides).
+With ``accepts_emit_norm = True`` it may also be asked to prepare the norm that reads the residual
+after it (``forward(..., emit=(gamma, eps))``, returning a ``PreNormed``): then the norm's pass over the
+residual happens where the residual is made, inside a block and from one block to the next."""
 from __future__ import annotations
 
 from typing import Dict, Optional
@@ -21,15 +24,27 @@ class PreNormBlock(Part):
     def children(self) -> Dict[str, Part]:
         return dict(zip(self.names, (self.mixer_norm, self.mixer, self.ffn_norm, self.ffn)))
 
-    def forward(self, ctx, x, cache: Optional[LayerCache]):
+    def entry_norm(self, ctx, n: int):
+        """``(gamma, eps)`` of the norm this block begins with, if the product that made the residual before
+        it may prepare that norm (``forward(..., pre=)`` then takes what it prepared); else None."""
+        return self.mixer_norm.fuse_spec(ctx, n) if getattr(self.mixer, "accepts_fused_norm", False) else None
+
+    def forward(self, ctx, x, cache: Optional[LayerCache], pre=None, emit=None):
+        """``pre``: a PreNormed for this block's first norm, from the block before; ``emit``: the ``entry_norm``
+        of the block after.  Returns a PreNormed for that block if the feed-forward prepared one."""
         n = x.shape[0]
-        spec = self.mixer_norm.fuse_spec(ctx, n) if getattr(self.mixer, "accepts_fused_norm", False) else None
+        fused = getattr(self.mixer, "accepts_fused_norm", False)
+        spec = (pre if pre is not None else self.mixer_norm.fuse_spec(ctx, n)) if fused else None
+        ffn_fused = getattr(self.ffn, "accepts_fused_norm", False)
+        more = {}
+        if ffn_fused and getattr(self.mixer, "accepts_emit_norm", False):
+            more["emit"] = self.ffn_norm.fuse_spec(ctx, n)
         if spec is not None:
-            self.mixer.forward(ctx, x, x, cache, norm=spec)
+            mid = self.mixer.forward(ctx, x, x, cache, norm=spec, **more)
         else:
-            self.mixer.forward(ctx, self.mixer_norm.forward(ctx, x), x, cache)
-        spec = self.ffn_norm.fuse_spec(ctx, n) if getattr(self.ffn, "accepts_fused_norm", False) else None
+            mid = self.mixer.forward(ctx, self.mixer_norm.forward(ctx, x), x, cache, **more)
+        spec = (mid if mid is not None else self.ffn_norm.fuse_spec(ctx, n)) if ffn_fused else None
+        more = {"emit": emit} if emit is not None and getattr(self.ffn, "accepts_emit_norm", False) else {}
         if spec is not None:
-            self.ffn.forward(ctx, x, x, norm=spec)
-        else:
-            self.ffn.forward(ctx, self.ffn_norm.forward(ctx, x), x)
+            return self.ffn.forward(ctx, x, x, norm=spec, **more)
+        return self.ffn.forward(ctx, self.ffn_norm.forward(ctx, x), x, **more)

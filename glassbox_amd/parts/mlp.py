@@ -7,7 +7,7 @@ from typing import Dict, Optional
 import torch
 
 from .. import ops
-from .base import FeedForward, TensorSpec
+from .base import FeedForward, PreNormed, TensorSpec, emit_target
 
 
 class SwiGLU(FeedForward):
@@ -26,12 +26,17 @@ class SwiGLU(FeedForward):
         self.w_down = tensors["down_proj.weight"].contiguous()
 
     accepts_fused_norm = True
+    accepts_emit_norm = True
 
-    def forward(self, ctx, h, residual, norm=None):
-        """``norm=(gamma, eps)``: h is the un-normed float32 residual and the first product norms it."""
+    def forward(self, ctx, h, residual, norm=None, emit=None):
+        """``norm=(gamma, eps)``: h is the un-normed float32 residual and the first product norms it;
+        ``norm=PreNormed``: the product before has done most of that.  ``emit=(gamma, eps)``: the down
+        projection may prepare the norm that reads the residual next (returns a PreNormed if it did)."""
         n = h.shape[0]
         act = ctx.buffer("act", (n, self.intermediate), ctx.dtype)
-        if ctx.dtype == torch.bfloat16 and self.intermediate % 8 == 0:
+        if isinstance(norm, PreNormed):
+            ops.gemm(norm.rows, self.w_gate_up, act, silu_mul=True, rms_parts=norm.as_gemm_arg())
+        elif ctx.dtype == torch.bfloat16 and self.intermediate % 8 == 0:
             # the activation is applied where the product's tile is finished: gate_up never reaches memory
             ops.gemm(h, self.w_gate_up, act, silu_mul=True, rms=norm)
         else:
@@ -42,4 +47,6 @@ class SwiGLU(FeedForward):
             gate_up = ctx.buffer("gate_up", (n, 2 * self.intermediate), ctx.dtype)
             ops.gemm(h, self.w_gate_up, gate_up)
             ops.silu_mul(gate_up, act)
-        ops.gemm(act, self.w_down, residual, accumulate=True)
+        target, handed_on = emit_target(ctx, n, self.width, emit, "ffn")
+        ops.gemm(act, self.w_down, residual, accumulate=True, emit=target)
+        return handed_on

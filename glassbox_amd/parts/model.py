@@ -81,7 +81,8 @@ class DecoderModel(Part):
         """Runs the tokens of ``ctx`` through every scheduled layer; logits [wanted, vocab] float32."""
         x = ctx.buffer("x", (ctx.n, self.width), torch.float32)
         self.embedding.forward(ctx, x)
-        for call in self.schedule:
+        pre = None   # what the block before prepared of this block's first norm
+        for i, call in enumerate(self.schedule):
             if call.cache is not None:
                 cache = caches[call.cache]
             elif call.reads is not None:
@@ -89,7 +90,14 @@ class DecoderModel(Part):
                 cache = LayerCache(src.k_pages, src.v_pages, src.group, src.state, writable=False)
             else:
                 cache = None
-            self.blocks[call.block].forward(ctx, x, cache)
+            block = self.blocks[call.block]
+            if hasattr(block, "entry_norm"):
+                after = self.blocks[self.schedule[i + 1].block] if i + 1 < len(self.schedule) else None
+                emit = after.entry_norm(ctx, ctx.n) if hasattr(after, "entry_norm") else None
+                pre = block.forward(ctx, x, cache, pre=pre, emit=emit)
+            else:
+                block.forward(ctx, x, cache)
+                pre = None
         if ctx.want.numel() == 0:
             return ctx.buffer("logits", (0, self.vocab_size), torch.float32)
         rows = self.final_norm.forward(ctx, x, rows=ctx.want, out_name="h_out")

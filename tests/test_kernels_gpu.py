@@ -115,6 +115,45 @@ def test_gemm_bf16_fused_rms_norm(N, K, M, silu, gamma_dtype):
     assert (two.cpu().double() - want).abs().max().item() <= tol
 
 
+@pytest.mark.parametrize("M,N,K,N2,silu", [(1, 64, 176, 96, False), (5, 352, 64, 176, True), (8, 2048, 2048, 6144, False),
+                                           (8, 2048, 8192, 16384, True), (3, 960, 2560, 2880, False)])
+@pytest.mark.parametrize("gamma_dtype", [torch.float32, torch.bfloat16])
+def test_gemm_bf16_prepares_the_next_norm(M, N, K, N2, silu, gamma_dtype):
+    """The product that adds into the residual and, on its way out, writes what the RMS norm that reads
+    the residual next would compute (bf16(gamma * r) and partial sums of r^2), and the product that takes
+    those: against norm-then-product in float64 (crates/glassbox-core/src/model.rs:94-100, 323-335)."""
+    from glassbox_amd import ops
+    parts_n = ops.gemm_emit_parts(M, N)
+    assert parts_n == -(-N // 8)
+    a, w = rnd(M, K, seed=1).bfloat16(), (rnd(N, K, seed=2) / math.sqrt(K)).bfloat16()
+    r0 = rnd(M, N, seed=3, scale=2.0).float()
+    g = (rnd(N, seed=4) * 0.3 + 1.0).to(gamma_dtype)
+    eps = 1e-5
+    plain = to_dev(r0.clone())
+    ops.gemm(to_dev(a), to_dev(w), plain, accumulate=True)
+    res, h = to_dev(r0.clone()), torch.zeros(M, N, device=DEV, dtype=torch.bfloat16)
+    parts = torch.full((parts_n, 8), 7.0, device=DEV)
+    ops.gemm(to_dev(a), to_dev(w), res, accumulate=True, emit=(to_dev(g), h, parts))
+    assert torch.equal(res, plain)                                        # the residual is what it was without
+    assert torch.equal(h, (to_dev(g).float() * res).bfloat16())
+    ss = res.double().pow(2).sum(-1).cpu()
+    assert ((parts[:, :M].double().sum(0).cpu() - ss).abs() <= 1e-5 * ss).all()
+    assert (parts[:, M:] == 0).all()
+    # the product that follows
+    w2 = (rnd(N2, N, seed=5) / math.sqrt(N)).bfloat16()
+    x = res.double().cpu()
+    normed = g.double() * (x * torch.rsqrt(x.pow(2).mean(-1, keepdim=True) + eps))
+    prod = normed @ w2.double().T
+    want = prod if not silu else prod[:, :N2 // 2] / (1 + torch.exp(-prod[:, :N2 // 2])) * prod[:, N2 // 2:]
+    out = torch.full(want.shape, 9.0, device=DEV, dtype=torch.bfloat16)
+    ops.gemm(h, to_dev(w2), out, silu_mul=silu, rms_parts=(parts, parts_n, eps))
+    tol = (2 ** -7) * want.abs().max().item() + 1e-3                      # as for the norm computed on the way in
+    assert (out.cpu().double() - want).abs().max().item() <= tol
+    again = torch.empty_like(out)
+    ops.gemm(res, to_dev(w2), again, silu_mul=silu, rms=(to_dev(g), eps))
+    assert ((out.float() - again.float()).abs() <= 2 ** -6 * (1 + again.float().abs())).all()
+
+
 def test_gemm_bf16_split_k_is_the_same_on_every_run():
     from glassbox_amd import ops
     a, w = to_dev(rnd(8, 8192, seed=1).bfloat16()), to_dev(rnd(2048, 8192, seed=2).bfloat16())
