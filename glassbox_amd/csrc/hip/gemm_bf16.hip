@@ -50,6 +50,21 @@ struct NormExtras {
   int n_parts;
 };
 
+// EPI_ROPE (the skinny kernel; the QKV product of a decode step): W stacks nh query heads, nkv key heads
+// and nkv value heads of hd rows each.  The product rotates query and key heads by the angles of each
+// row's position (pairs (i, i + hd/2), crates/glassbox-core/src/model.rs:102-115) while the sums are
+// still 32-bit, writes the stacked rows to C as usual, and the key and value heads straight into the
+// cache pages at slots[m] (keys [page][kv head][slot][hd], values [page][kv head][hd][slot]) if slots is
+// given: the rotation kernel and its round trip through memory are not needed.
+struct RopeExtras {
+  const float* cosv;   // [M][hd/2], nullptr: no rotation
+  const float* sinv;
+  const int32_t* slots;  // [M], nullptr: nothing is stored
+  bf16* k_pages;
+  bf16* v_pages;
+  int nh, nkv, hd, page_size;
+};
+
 template <typename CT> __device__ __forceinline__ void store_c(CT* c, float v, int accumulate);
 template <> __device__ __forceinline__ void store_c<float>(float* c, float v, int accumulate) { *c = accumulate ? *c + v : v; }
 template <> __device__ __forceinline__ void store_c<bf16>(bf16* c, float v, int) { *c = (bf16)v; }
@@ -63,7 +78,7 @@ template <> __device__ __forceinline__ void store_c<bf16>(bf16* c, float v, int)
 // tiles the first holds 32 gate columns and the second the 32 up columns that belong to them, so
 // act = gate / (1 + exp(-gate)) * up (crates/glassbox-core/src/model.rs:336-340) is formed in
 // registers and C is [M, N/2].
-enum : int { EPI_STORE = 0, EPI_ACCUMULATE = 1, EPI_SILU_MUL = 2 };
+enum : int { EPI_STORE = 0, EPI_ACCUMULATE = 1, EPI_SILU_MUL = 2, EPI_ROPE = 3 };
 constexpr int TBK = 64, TLD = TBK + 8;  // k-step; LDS row stride in elements (144 bytes)
 constexpr int TCPR = TBK / 8;           // 16-byte chunks per row of a k-step
 constexpr int TKS = TBK / 16;           // MFMA k-steps per LDS k-step
@@ -332,7 +347,7 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_skinny_kernel(const void* __r
                                                                  const bf16* __restrict__ w, int ldw, CT* __restrict__ c,
                                                                  int ldc, int M, int N, int K, const void* __restrict__ gamma,
                                                                  int gamma_f32, float eps, const float* __restrict__ parts,
-                                                                 int n_parts) {
+                                                                 int n_parts, RopeExtras rope) {
   __shared__ float part[WAVES][RT][MT][64][4];
   __shared__ float sspart[RMS ? WAVES : 1][MT][64];
   __shared__ float red[64][8];
@@ -354,8 +369,15 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_skinny_kernel(const void* __r
   for (int rt = 0; rt < RT; ++rt) {
     const int tile = blockIdx.x * RT + rt;
     int row;
-    if (EPI == EPI_SILU_MUL) row = r < 8 ? tile * 8 + r : N / 2 + tile * 8 + (r - 8);
-    else row = tile * 16 + r;
+    if (EPI == EPI_SILU_MUL) {
+      row = r < 8 ? tile * 8 + r : N / 2 + tile * 8 + (r - 8);
+    } else if (EPI == EPI_ROPE) {
+      // a tile is 8 pairs of one head: its dims d0..d0+7 and those hd/2 further on
+      const int per_head = rope.hd / 16, head = tile / per_head, d0 = (tile % per_head) * 8;
+      row = head * rope.hd + (r < 8 ? d0 + r : rope.hd / 2 + d0 + (r - 8));
+    } else {
+      row = tile * 16 + r;
+    }
     row_ok[rt] = EPI == EPI_SILU_MUL ? (tile * 8 + (r & 7) < N / 2) : row < N;
     wrow[rt] = w + (size_t)(row_ok[rt] ? row : 0) * ldw;
   }
@@ -477,6 +499,45 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_skinny_kernel(const void* __r
           const int m = t * 16 + l % 16;
           const float g = v[rt][t], u = up[(rt * MT + t) * 256 + tid + 128];
           if (m < M && j < N / 2) c[(size_t)m * ldc + j] = (CT)(g / (1.0f + __expf(-g)) * u);
+        }
+      }
+    }
+  } else if (EPI == EPI_ROPE) {
+    // rows 0..7 and 8..15 of a tile are each other's partners: they meet through LDS as gate and up do
+    float* other = &part[WAVES - 1][0][0][0][0];
+    __syncthreads();
+#pragma unroll
+    for (int rt = 0; rt < RT; ++rt)
+#pragma unroll
+      for (int t = 0; t < MT; ++t) other[(rt * MT + t) * 256 + tid] = v[rt][t];
+    __syncthreads();
+    const int half = rope.hd / 2, per_head = rope.hd / 16;
+    const bool upper = nrow >= 8;
+#pragma unroll
+    for (int rt = 0; rt < RT; ++rt) {
+      const int tile = blockIdx.x * RT + rt;
+      const int head = tile / per_head, pair = (tile % per_head) * 8 + (nrow & 7);
+      const int dim = upper ? half + pair : pair;
+      if (head * rope.hd + dim >= N) continue;
+      const bool is_value = head >= rope.nh + rope.nkv, is_key = head >= rope.nh && !is_value;
+#pragma unroll
+      for (int t = 0; t < MT; ++t) {
+        const int m = t * 16 + l % 16;
+        if (m >= M) continue;
+        float y = v[rt][t];
+        if (!is_value && rope.cosv != nullptr) {
+          const float p = other[(rt * MT + t) * 256 + (tid ^ 128)];
+          const float cs = rope.cosv[(size_t)m * half + pair], sn = rope.sinv[(size_t)m * half + pair];
+          y = upper ? y * cs + p * sn : y * cs - p * sn;
+        }
+        const bf16 yb = (bf16)y;
+        c[(size_t)m * ldc + head * rope.hd + dim] = (CT)yb;
+        if (rope.slots != nullptr && head >= rope.nh) {
+          const int slot = rope.slots[m], page = slot / rope.page_size, off = slot % rope.page_size;
+          if (is_key)
+            rope.k_pages[(((size_t)page * rope.nkv + (head - rope.nh)) * rope.page_size + off) * rope.hd + dim] = yb;
+          else
+            rope.v_pages[(((size_t)page * rope.nkv + (head - rope.nh - rope.nkv)) * rope.hd + dim) * rope.page_size + off] = yb;
         }
       }
     }
@@ -650,13 +711,14 @@ inline void skinny_plan(int tiles, int K, int mt, int* waves, int* iters, int* r
 
 template <int MT, int EPI, bool RMS, typename CT>
 int launch_skinny_mt(int tiles, const void* a, int lda, const bf16* w, int ldw, CT* c, int ldc, int M, int N, int K,
-                     const void* gamma, int gamma_f32, float eps, const NormExtras& extra, hipStream_t stream) {
+                     const void* gamma, int gamma_f32, float eps, const NormExtras& extra, const RopeExtras& rope,
+                     hipStream_t stream) {
   int waves, iters, rt;
   skinny_plan(tiles, K, MT, &waves, &iters, &rt);
 #define GB_CFG(WV, IT, RT)                                                                                                 \
   if (waves == WV && iters == (IT) && rt == RT)                                                                            \
     hipLaunchKernelGGL((gemm_skinny_kernel<MT, WV, (IT), RT, EPI, RMS, CT>), dim3((tiles + RT - 1) / RT), dim3(WV * 64), 0,  \
-                       stream, a, lda, w, ldw, c, ldc, M, N, K, gamma, gamma_f32, eps, extra.parts, extra.n_parts);
+                       stream, a, lda, w, ldw, c, ldc, M, N, K, gamma, gamma_f32, eps, extra.parts, extra.n_parts, rope);
   // the configurations skinny_plan can ask for: two loads in flight only with one column block
   GB_CFG(4, 1, 1) GB_CFG(4, 1, 2) GB_CFG(16, 1, 1) GB_CFG(16, 1, 2)
   if (MT == 1) {
@@ -668,14 +730,14 @@ int launch_skinny_mt(int tiles, const void* a, int lda, const bf16* w, int ldw, 
 
 template <int EPI, bool RMS, typename CT>
 int launch_skinny(const void* a, int lda, const bf16* w, int ldw, CT* c, int ldc, int M, int N, int K, const void* gamma,
-                  int gamma_f32, float eps, const NormExtras& extra, hipStream_t stream) {
-  const int tiles = EPI == EPI_SILU_MUL ? (N / 2 + 7) / 8 : (N + 15) / 16;
+                  int gamma_f32, float eps, const NormExtras& extra, hipStream_t stream, const RopeExtras& rope = RopeExtras{}) {
+  const int tiles = EPI == EPI_SILU_MUL ? (N / 2 + 7) / 8 : (N + 15) / 16;  // EPI_ROPE: N is a multiple of 16
   const int mt = (M + 15) / 16;
 #define GB_MT(T) \
-  if (mt == T) return launch_skinny_mt<T, EPI, RMS, CT>(tiles, a, lda, w, ldw, c, ldc, M, N, K, gamma, gamma_f32, eps, extra, stream);
+  if (mt == T) return launch_skinny_mt<T, EPI, RMS, CT>(tiles, a, lda, w, ldw, c, ldc, M, N, K, gamma, gamma_f32, eps, extra, rope, stream);
   GB_MT(1) GB_MT(2) GB_MT(3)
 #undef GB_MT
-  return launch_skinny_mt<4, EPI, RMS, CT>(tiles, a, lda, w, ldw, c, ldc, M, N, K, gamma, gamma_f32, eps, extra, stream);
+  return launch_skinny_mt<4, EPI, RMS, CT>(tiles, a, lda, w, ldw, c, ldc, M, N, K, gamma, gamma_f32, eps, extra, rope, stream);
 }
 
 }  // namespace
@@ -743,4 +805,31 @@ extern "C" int gb_gemm_bf16(const void* a, int lda, const void* w, int ldw, void
   if (c_dtype == kF32) GB_TL(EPI_STORE, float);
   GB_TL(EPI_STORE, bf16);
 #undef GB_TL
+}
+
+// The QKV product of a step of at most 64 rows with EPI_ROPE (see RopeExtras): c is the stacked rows
+// [M][(nh + 2 nkv) hd] (or [M][nh hd] with nkv == 0: queries only), bfloat16.  gamma / parts as in
+// gb_gemm_bf16 (the norm before the product).
+extern "C" int gb_gemm_bf16_rope(const void* a, int lda, const void* w, int ldw, void* c, int ldc, int M, int N, int K,
+                                 const void* gamma, int gamma_dtype, float eps, const float* parts, int n_parts,
+                                 const float* cosv, const float* sinv, const int32_t* slots, void* k_pages, void* v_pages,
+                                 int nh, int nkv, int hd, int page_size, hipStream_t stream) {
+  GB_REQUIRE(M > 0 && M <= 64 && N > 0 && K > 0 && K % 8 == 0, "gemm_bf16_rope: bad sizes M=%d N=%d K=%d (at most 64 rows)", M, N, K);
+  GB_REQUIRE(hd >= 16 && hd % 16 == 0 && nh > 0 && nkv >= 0 && N == (nh + 2 * nkv) * hd,
+             "gemm_bf16_rope: N=%d is not (nh + 2 nkv) hd with nh=%d nkv=%d hd=%d (a multiple of 16)", N, nh, nkv, hd);
+  GB_REQUIRE(ldw % 8 == 0 && lda % (gamma ? 4 : 8) == 0 && lda >= K && ldw >= K && ldc >= N && ((uintptr_t)a % 16 == 0) &&
+                 ((uintptr_t)w % 16 == 0),
+             "gemm_bf16_rope: operands must be 16-byte aligned rows");
+  GB_REQUIRE((cosv == nullptr) == (sinv == nullptr), "gemm_bf16_rope: cos and sin come together");
+  GB_REQUIRE(!slots || (k_pages && v_pages && page_size > 0 && nkv > 0), "gemm_bf16_rope: slots given without pages");
+  GB_REQUIRE(!gamma || (((uintptr_t)gamma % 16 == 0) && (gamma_dtype == kF32 || gamma_dtype == kBF16) && !parts),
+             "gemm_bf16_rope: gamma must be aligned float32 or bfloat16, and not given together with parts");
+  GB_REQUIRE(!parts || (M <= 8 && n_parts > 0), "gemm_bf16_rope: partial sums of a norm go with at most 8 rows");
+  const NormExtras extra{nullptr, 0, nullptr, 0, nullptr, parts, n_parts};
+  const RopeExtras rope{cosv, sinv, slots, (bf16*)k_pages, (bf16*)v_pages, nh, nkv, hd, page_size};
+  if (gamma)
+    return launch_skinny<EPI_ROPE, true, bf16>(a, lda, (const bf16*)w, ldw, (bf16*)c, ldc, M, N, K, gamma, gamma_dtype == kF32,
+                                               eps, extra, stream, rope);
+  return launch_skinny<EPI_ROPE, false, bf16>(a, lda, (const bf16*)w, ldw, (bf16*)c, ldc, M, N, K, nullptr, 0, eps, extra,
+                                              stream, rope);
 }

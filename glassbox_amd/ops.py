@@ -55,6 +55,10 @@ _SIGS = {
         # emit_gamma, emit_gamma_dtype, emit_h, emit_ldh, emit_ss, parts, n_parts, stream
         "gb_gemm_bf16": [_vp, _i, _vp, _i, _vp, _i, _i, _i, _i, _i, _i, _vp, _i, _f, _vp, _i, _vp, _i, _vp, _vp, _i, _vp],
         "gb_gemm_bf16_emit_parts": [_i, _i],
+        # a, lda, w, ldw, c, ldc, M, N, K, gamma, gamma_dtype, eps, parts, n_parts, cos, sin, slots, k, v,
+        # nh, nkv, hd, page, stream
+        "gb_gemm_bf16_rope": [_vp, _i, _vp, _i, _vp, _i, _i, _i, _i, _vp, _i, _f, _vp, _i, _vp, _vp, _vp, _vp, _vp,
+                              _i, _i, _i, _i, _vp],
     },
     "attention_plain": {
         "gb_attention_plain": [_vp, _i, _vp, _i, _i, _vp, _vp, _vp, _i, _vp, _vp, _i, _i, _i, _i, _i, _f, _i, _vp],
@@ -327,6 +331,53 @@ def gemm(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor, accumulate: bool =
                                      _p(e_ss), _p(parts), int(n_parts), _stream()))
     else:
         raise KernelError(f"gemm: operand types {a.dtype} and {w.dtype} do not match a kernel")
+
+
+ROPE_PRODUCT_MAX_ROWS = 64
+
+
+def gemm_rope(a: torch.Tensor, w: torch.Tensor, qkv: torch.Tensor, n_heads: int, n_kv_heads: int, head_dim: int,
+              cos: Optional[torch.Tensor], sin: Optional[torch.Tensor], slots: Optional[torch.Tensor],
+              k_pages: Optional[torch.Tensor], v_pages: Optional[torch.Tensor], rms: Optional[tuple] = None,
+              rms_parts: Optional[tuple] = None) -> None:
+    """The stacked query/key/value product of a step of at most 64 rows that rotates query and key heads
+    (``cos``/``sin`` float32 ``[M, head_dim/2]``; None: no rotation) and writes key and value heads into
+    the pages at ``slots`` (None: nothing stored) in its epilogue, besides writing ``qkv`` as ``gemm``
+    does.  ``n_kv_heads`` 0: w holds query heads only.  ``rms`` / ``rms_parts`` as in ``gemm``."""
+    _dev(a, w, qkv, cos, sin, slots, k_pages, v_pages)
+    M, K = a.shape
+    N = w.shape[0]
+    if w.shape[1] != K or qkv.shape != (M, N) or N != (n_heads + 2 * n_kv_heads) * head_dim:
+        raise KernelError(f"gemm_rope: shapes do not match: a {tuple(a.shape)}, w {tuple(w.shape)}, qkv {tuple(qkv.shape)}")
+    if w.dtype != torch.bfloat16 or qkv.dtype != torch.bfloat16 or M > ROPE_PRODUCT_MAX_ROWS or head_dim % 16:
+        raise KernelError("gemm_rope: bfloat16 weights and rows, at most 64 rows, head sizes in steps of 16")
+    page_size = 0
+    if slots is not None:
+        _i32(slots, "slots", M)
+        _check_pages(k_pages, v_pages, torch.bfloat16, "gemm_rope")
+        if (k_pages.shape[1], k_pages.shape[3]) != (n_kv_heads, head_dim):
+            raise KernelError("gemm_rope: pages do not have this layer's kv heads and head size")
+        page_size = k_pages.shape[2]
+    if cos is not None:
+        if sin is None or cos.shape[1] != head_dim // 2 or cos.shape[0] < M or cos.dtype != torch.float32 \
+                or not cos.is_contiguous() or not sin.is_contiguous() or sin.shape != cos.shape:
+            raise KernelError("gemm_rope: cos/sin must be contiguous float32 [M, head_dim/2]")
+    gamma, eps, parts, n_parts = None, 0.0, None, 0
+    if rms is not None:
+        gamma, eps = rms
+        if a.dtype != torch.float32 or gamma.numel() != K or not gamma.is_contiguous():
+            raise KernelError("gemm_rope: the fused RMS norm takes float32 rows and a gamma of K entries")
+    elif a.dtype != torch.bfloat16:
+        raise KernelError("gemm_rope: rows must be bfloat16 (float32 only with rms=)")
+    if rms_parts is not None:
+        parts, n_parts, eps = rms_parts
+        if rms is not None or M > 8 or parts.dtype != torch.float32 or not parts.is_contiguous() or parts.numel() < n_parts * 8:
+            raise KernelError("gemm_rope: partial sums of a norm go with at most 8 rows and no gamma")
+    lib = _lib("gemm_bf16")
+    _check(lib, lib.gb_gemm_bf16_rope(_p(a), _rows(a, "a"), _p(w), _rows(w, "w"), _p(qkv), _rows(qkv, "qkv"), M, N, K,
+                                      _p(gamma), dtype_code(gamma) if gamma is not None else 0, float(eps), _p(parts),
+                                      int(n_parts), _p(cos), _p(sin), _p(slots), _p(k_pages), _p(v_pages), n_heads,
+                                      n_kv_heads, head_dim, page_size, _stream()))
 
 
 # ----------------------------------------------------------------------- attention

@@ -66,15 +66,24 @@ class PagedAttention(Mixer):
         n = h.shape[0]
         rows = self.q_dim + (0 if self.shares_kv else 2 * self.kv_dim)
         qkv = ctx.buffer("qkv", (n, rows), ctx.dtype)
-        if isinstance(norm, PreNormed):
-            ops.gemm(norm.rows, self.wqkv, qkv, rms_parts=norm.as_gemm_arg())
-        else:
-            ops.gemm(h, self.wqkv, qkv, rms=norm)
         write = cache.writable and not self.shares_kv
-        self.position.apply_and_store(
-            ctx, qkv, self.n_heads, 0 if self.shares_kv else self.n_kv_heads, self.head_dim,
-            ctx.slots[cache.group] if write else None, cache.k_pages if write else None,
-            cache.v_pages if write else None)
+        store = (ctx.slots[cache.group], cache.k_pages, cache.v_pages) if write else (None, None, None)
+        n_kv = 0 if self.shares_kv else self.n_kv_heads
+        pre = isinstance(norm, PreNormed)
+        # few rows (decoding): the product's epilogue rotates the heads and writes the cache itself
+        tables = None
+        if (ctx.dtype == torch.bfloat16 and ctx.fuse_norms and n <= ops.ROPE_PRODUCT_MAX_ROWS
+                and self.head_dim % 16 == 0):
+            tables = self.position.fuse_spec(ctx, self.head_dim)
+        if tables is not None:
+            ops.gemm_rope(norm.rows if pre else h, self.wqkv, qkv, self.n_heads, n_kv, self.head_dim, tables[0],
+                          tables[1], *store, rms=None if pre else norm, rms_parts=norm.as_gemm_arg() if pre else None)
+        else:
+            if pre:
+                ops.gemm(norm.rows, self.wqkv, qkv, rms_parts=norm.as_gemm_arg())
+            else:
+                ops.gemm(h, self.wqkv, qkv, rms=norm)
+            self.position.apply_and_store(ctx, qkv, self.n_heads, n_kv, self.head_dim, *store)
         att = ctx.buffer("att", (n, self.q_dim), ctx.dtype)
         ctx.attention(qkv[:, :self.q_dim], att, cache, self.n_heads, self.scale, self.window)
         target, handed_on = emit_target(ctx, n, self.width, emit, "mixer")

@@ -113,6 +113,13 @@ class PositionEncoding(Part):
     def apply_and_store(self, ctx, qkv, n_heads, n_kv_heads, head_dim, slots, k_pages, v_pages) -> None:
         raise NotImplementedError
 
+    def fuse_spec(self, ctx, head_dim: int):
+        """``(cos, sin)`` tables of the step's rows (float32 ``[n, head_dim/2]``; ``(None, None)`` for no
+        rotation) if a kernel that has the query and key heads in hand may apply this encoding (the
+        half-split rotation by these angles) and write the cache itself instead of calling
+        ``apply_and_store``; None (the default) if this encoding has to do its own work."""
+        return None
+
 
 class PreNormed(NamedTuple):
     """The work of an RMS norm done by the product that made the residual: ``rows`` = bf16(gamma * residual)

@@ -50,8 +50,15 @@ class Rotary(PositionEncoding):
                        portions=ctx.portions())
 
 
+    def fuse_spec(self, ctx, head_dim: int):
+        return self.table(ctx) if head_dim == self.head_dim else None
+
+
 class NoPosition(PositionEncoding):
     """Keys and queries as they are; only the cache write."""
+
+    def fuse_spec(self, ctx, head_dim: int):
+        return (None, None)
 
     def apply_and_store(self, ctx, qkv, n_heads, n_kv_heads, head_dim, slots, k_pages, v_pages):
         if slots is not None:

@@ -262,6 +262,65 @@ def test_rope_table_and_rotation(hd, theta):
         assert torch.equal(got_v, qkv[i, (nh + nkv) * hd:].reshape(nkv, hd))
 
 
+ROPE_PRODUCTS = [(1, 4, 2, 16, 64), (8, 3, 1, 32, 96), (5, 6, 2, 48, 80), (8, 32, 32, 64, 2048), (33, 8, 2, 128, 264),
+                 (64, 15, 5, 64, 960), (7, 4, 0, 32, 64)]
+
+
+@pytest.mark.parametrize("M,nh,nkv,hd,K,normed", [p + (False,) for p in ROPE_PRODUCTS] +
+                         [p + (True,) for p in ROPE_PRODUCTS if p[0] <= 16])   # the norm on the way in serves 16 rows
+def test_gemm_bf16_rotates_and_writes_the_cache(M, nh, nkv, hd, K, normed):
+    """The stacked q/k/v product whose epilogue rotates query and key heads and writes keys and values into
+    the pages: against the product, the rotation and the cache write in float64
+    (crates/glassbox-core/src/model.rs:260-276), and against the two kernels it replaces."""
+    from glassbox_amd import ops
+    from plain import llama
+    page, N = 16, (nh + 2 * nkv) * hd
+    g = torch.Generator().manual_seed(M + hd)
+    x = rnd(M, K, seed=1, scale=2.0).float()
+    gamma, eps = (rnd(K, seed=2) * 0.3 + 1.0).float(), 1e-5
+    w = (rnd(N, K, seed=3) / math.sqrt(K)).bfloat16()
+    pos = torch.randint(0, 5000, (M,), generator=g).tolist()
+    theta = 130000.0
+    s64, c64 = llama.rope_angles(pos, hd, theta)
+    cos, sin = to_dev(torch.from_numpy(c64).float()), to_dev(torch.from_numpy(s64).float())
+    slots = torch.randperm(4 * page, generator=g)[:M].to(torch.int32)
+    if normed:
+        a_dev = to_dev(x)
+        h64 = gamma.double() * (x.double() * torch.rsqrt(x.double().pow(2).mean(-1, keepdim=True) + eps))
+        rms = (to_dev(gamma), eps)
+    else:
+        a_dev = to_dev(x.bfloat16())
+        h64 = x.bfloat16().double()
+        rms = None
+    prod = h64 @ w.double().T
+    q_want = llama.rope(prod[:, :nh * hd].reshape(M, nh, hd), pos, theta).reshape(M, nh * hd)
+    store = nkv > 0
+    k_pages = torch.zeros(4, max(nkv, 1), page, hd, device=DEV, dtype=torch.bfloat16)
+    v_pages = torch.zeros(4, max(nkv, 1), hd, page, device=DEV, dtype=torch.bfloat16)
+    qkv = torch.full((M, N), 9.0, device=DEV, dtype=torch.bfloat16)
+    ops.gemm_rope(a_dev, to_dev(w), qkv, nh, nkv, hd, cos, sin, to_dev(slots) if store else None,
+                  k_pages if store else None, v_pages if store else None, rms=rms)
+    tol = (2 ** -7) * prod.abs().max().item() + 1e-3
+    assert (qkv[:, :nh * hd].cpu().double() - q_want).abs().max().item() <= tol
+    if store:
+        k_want = llama.rope(prod[:, nh * hd:(nh + nkv) * hd].reshape(M, nkv, hd), pos, theta)
+        v_want = prod[:, (nh + nkv) * hd:].reshape(M, nkv, hd)
+        for i, sl in enumerate(slots.tolist()):
+            assert (k_pages[sl // page, :, sl % page, :].cpu().double() - k_want[i]).abs().max().item() <= tol
+            assert (v_pages[sl // page, :, :, sl % page].cpu().double() - v_want[i]).abs().max().item() <= tol
+        # the rows hold what the pages hold
+        assert torch.equal(qkv[0, nh * hd:(nh + nkv) * hd].reshape(nkv, hd), k_pages[slots[0] // page, :, slots[0] % page, :])
+        # the two kernels it replaces round once more (the product to bfloat16 before the rotation)
+        two = torch.empty_like(qkv)
+        ops.gemm(a_dev, to_dev(w), two, rms=rms)
+        k2, v2 = torch.zeros_like(k_pages), torch.zeros_like(v_pages)
+        ops.rope_store(two, cos, sin, to_dev(slots), k2, v2, nh, nkv, hd)
+        # (a rotated value can be much smaller than the two it is made of, so the bound is absolute)
+        assert (two.float() - qkv.float()).abs().max().item() <= 2 * tol
+        assert (k2.float() - k_pages.float()).abs().max().item() <= 2 * tol
+        assert (v2.float() - v_pages.float()).abs().max().item() <= 2 * tol
+
+
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 @pytest.mark.parametrize("hd,page", [(16, 16), (64, 16), (128, 32), (40, 16)])
 def test_rope_store_writes_values_of_portions_in_tiles(dtype, hd, page):
