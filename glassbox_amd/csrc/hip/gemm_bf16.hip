@@ -4,13 +4,14 @@
 // is the layout MFMA operands want: every lane loads 8 consecutive k as one 16-byte word.
 //
 // Three kernels:
-//  * tiled  (M > 64, prompt portions): a workgroup of 2x2 waves, each wave a block of up to 4x2
-//    v_mfma_f32_32x32x16_bf16 tiles (workgroup tile up to 256x128), operands staged through LDS in
-//    k-steps of 32 with two buffers; the SiLU-multiply of stacked gate/up rows can be its epilogue.
+//  * tiled  (M > 64, prompt portions): a workgroup of 2x2 waves, each wave a block of 2x2 or 2x1
+//    v_mfma_f32_32x32x16_bf16 tiles (workgroup tile 128x128 or 128x64), operands staged through LDS in
+//    k-steps of 64 with two buffers; the SiLU-multiply of stacked gate/up rows can be its epilogue.
 //  * skinny (M <= 64, decoding): bound by reading W once.  A workgroup owns 16 or 32 rows of W; its
 //    waves take interleaved 64-wide k blocks, stream W straight from memory into MFMA operands
 //    (v_mfma_f32_16x16x32_bf16, W as the A operand so that the 16 rows fill the tile) and combine
-//    through LDS in a fixed order; it can norm float32 rows on the way and apply the SiLU-multiply.
+//    through LDS in a fixed order; it can norm float32 rows on the way, apply the SiLU-multiply, or
+//    (the QKV product) rotate the heads and write the key/value cache.
 //  * folded (M <= 8 and few rows of W): the skinny kernel with two k ranges side by side in a tile,
 //    so that a workgroup owns 8 rows of W and there are twice as many workgroups.
 // In all, every output cell is summed in an order fixed by (K, kernel) alone, not by M or by
@@ -71,8 +72,8 @@ template <> __device__ __forceinline__ void store_c<bf16>(bf16* c, float v, int)
 
 // ------------------------------------------------------------------------- tiled
 // A workgroup of 2 x 2 waves; a wave owns WM x WN tiles of 32 x 32, so the workgroup's tile is
-// (64 WM) x (64 WN).  Operands are staged through LDS in k-steps of 32, two buffers; rows are padded
-// to 80 bytes so that the 16-byte operand reads of a wave spread over the banks.
+// (64 WM) x (64 WN).  Operands are staged through LDS in k-steps of 64, two buffers; rows are padded
+// to 144 bytes so that the 16-byte operand reads of a wave spread over the banks.
 //
 // EPI_SILU_MUL (WN = 2): W stacks gate rows [0, N/2) over up rows [N/2, N).  Of a wave's two column
 // tiles the first holds 32 gate columns and the second the 32 up columns that belong to them, so

@@ -251,9 +251,6 @@ def copy_rows(base: torch.Tensor, src: torch.Tensor, dst: torch.Tensor) -> None:
 
 
 # ------------------------------------------------------------------------ products
-SILU_MUL_MAX_ROWS = 64
-
-
 FUSED_NORM_MAX_ROWS = 16   # measured: beyond one 16-row block the re-reading of float32 rows costs more than a norm pass
 
 
@@ -268,7 +265,7 @@ def gemm(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor, accumulate: bool =
     """out (+)= a . w^T with w in the [out features, in features] layout.
     float32 operands take the true 32-bit kernel; bfloat16 operands the matrix-core kernels,
     with out in bfloat16 or float32 (float32 when accumulating into the residual).
-    ``silu_mul`` (bfloat16, at most 64 rows): w stacks gate rows over up rows and out[m, j] =
+    ``silu_mul`` (bfloat16): w stacks gate rows over up rows and out[m, j] =
     silu(a . gate_j) * (a . up_j), of half as many columns.
     ``rms=(gamma, eps)`` (bfloat16 w and out, at most 64 rows): a is the float32 residual and the
     product is that of its RMS-normed rows, the norm computed inside the product's kernel.
