@@ -217,25 +217,51 @@ __global__ __launch_bounds__(WAVES * 64) void decode_kernel(const bf16* __restri
   }
 }
 
-// One block per (request, head): the chunks' partial results, combined in chunk order.
-__global__ void decode_reduce_kernel(const float* __restrict__ ws_acc, const float* __restrict__ ws_ml,
-                                     bf16* __restrict__ out, int out_stride, const int32_t* __restrict__ positions, int nh,
-                                     int hd, int window, int chunk, int splits) {
-  const int s = blockIdx.x / nh, head = blockIdx.x % nh;
+// One block of 256 threads per (request, head): the chunks' partial results, combined in a fixed order.
+// The chunks are dealt to 256 / hd groups of threads, each thread of a group taking one dimension, so
+// that few loads depend on each other; the groups' sums meet in LDS.
+__global__ __launch_bounds__(256) void decode_reduce_kernel(const float* __restrict__ ws_acc, const float* __restrict__ ws_ml,
+                                                            bf16* __restrict__ out, int out_stride,
+                                                            const int32_t* __restrict__ positions, int nh, int hd, int window,
+                                                            int chunk, int splits) {
+  __shared__ float sm_f[256];        // chunk k's weight exp(m_k - M), then times nothing: l_k is kept beside
+  __shared__ float sm_l[256];
+  __shared__ float sm_part[256];     // [group][dimension]
+  __shared__ float sm_top;
+  const int s = blockIdx.x / nh, head = blockIdx.x % nh, tid = threadIdx.x;
   const int pos = positions[s];
   const int lo = window > 0 ? max(0, pos - window + 1) : 0;
-  const int first = lo / chunk, last = pos / chunk;
-  const size_t base = ((size_t)s * nh + head) * splits;
-  float M = -INFINITY;
-  for (int k = first; k <= last; ++k) M = fmaxf(M, ws_ml[(base + k) * 2]);
-  for (int d = threadIdx.x; d < hd; d += blockDim.x) {
-    float val = 0.f, L = 0.f;
-    for (int k = first; k <= last; ++k) {
-      const float f = __expf(ws_ml[(base + k) * 2] - M);
-      val += ws_acc[(base + k) * hd + d] * f;
-      L += ws_ml[(base + k) * 2 + 1] * f;
-    }
-    out[(size_t)s * out_stride + (size_t)head * hd + d] = (bf16)(val / L);
+  const int first = lo / chunk, last = pos / chunk, count = last - first + 1;  // at most 256 chunks hold keys
+  const size_t base = ((size_t)s * nh + head) * splits + first;
+  float mine = -INFINITY;
+  if (tid < count) {
+    mine = ws_ml[(base + tid) * 2];
+    sm_l[tid] = ws_ml[(base + tid) * 2 + 1];
+  }
+  sm_f[tid] = mine;
+  __syncthreads();
+  if (tid == 0) {
+    float top = -INFINITY;
+    for (int k = 0; k < count; ++k) top = fmaxf(top, sm_f[k]);
+    sm_top = top;
+  }
+  __syncthreads();
+  const float top = sm_top;
+  __syncthreads();
+  if (tid < count) sm_f[tid] = __expf(mine - top);
+  __syncthreads();
+  const int groups = 256 / hd;  // hd <= 128: at least two
+  const int d = tid % hd, group = tid / hd;
+  float val = 0.f;
+  if (group < groups)
+    for (int k = group; k < count; k += groups) val += ws_acc[(base + k) * hd + d] * sm_f[k];
+  sm_part[tid] = val;
+  __syncthreads();
+  if (tid < hd) {
+    float total = 0.f, l = 0.f;
+    for (int g = 0; g < groups; ++g) total += sm_part[g * hd + tid];
+    for (int k = 0; k < count; ++k) l += sm_l[k] * sm_f[k];
+    out[(size_t)s * out_stride + (size_t)head * hd + tid] = (bf16)(total / l);
   }
 }
 
@@ -593,7 +619,8 @@ extern "C" int gb_attention_decode_bf16(const void* q, int q_stride, void* out, 
 #undef GB_CASE
   if (int rc = launched("attention_decode")) return rc;
   if (splits > 1) {
-    hipLaunchKernelGGL(decode_reduce_kernel, dim3(n_decode * nh), dim3(64), 0, stream, (const float*)ws_acc,
+    GB_REQUIRE(splits <= 256, "attention_decode: %d chunks are more than the 256 the second pass combines", splits);
+    hipLaunchKernelGGL(decode_reduce_kernel, dim3(n_decode * nh), dim3(256), 0, stream, (const float*)ws_acc,
                        (const float*)ws_ml, (bf16*)out, out_stride, positions, nh, hd, window, chunk, splits);
     return launched("attention_decode_reduce");
   }

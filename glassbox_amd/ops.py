@@ -413,7 +413,7 @@ def decode_chunk(n_decode: int, n_kv_heads: int, max_context: int) -> int:
     unit from requests and kv heads alone, each takes a whole context (and sixteen waves: nothing is
     left to combine afterwards); otherwise small enough that the launch has about a thousand workgroups."""
     groups = max(1, n_decode * n_kv_heads)
-    want_splits = 1 if groups >= 256 else max(1, 1024 // groups)
+    want_splits = 1 if groups >= 256 else min(256, max(1, 1024 // groups))   # the second pass combines up to 256
     chunk = -(-max_context // want_splits)
     return max(256, -(-chunk // 256) * 256)
 
