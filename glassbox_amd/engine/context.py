@@ -22,6 +22,8 @@ class Workspace:
     def __init__(self, device):
         self.device = device
         self._flat: Dict[Tuple[str, torch.dtype], torch.Tensor] = {}
+        #: counts the times a buffer was replaced by a larger one: a captured graph holds the old addresses
+        self.epoch = 0
 
     def buffer(self, name: str, shape: Sequence[int], dtype: torch.dtype) -> torch.Tensor:
         count = 1
@@ -33,6 +35,8 @@ class Workspace:
             if torch.cuda.is_current_stream_capturing():
                 raise RuntimeError(f"workspace buffer {name!r} would have to grow during graph capture")
             grow = max(count, int((flat.numel() if flat is not None else 0) * 1.5), 1)
+            if flat is not None:
+                self.epoch += 1
             flat = torch.empty(grow, dtype=dtype, device=self.device)
             self._flat[key] = flat
         return flat[:count].view(*shape)

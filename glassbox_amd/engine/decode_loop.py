@@ -74,6 +74,7 @@ class DecodeLoop:
         self.use_graph = use_graph
         self.graphs = {}          # context bucket -> captured graph
         self.warm = set()         # buckets that have run once without a graph
+        self.epoch = engine.workspace.epoch
         self.steps = 0
 
     def _run(self) -> None:
@@ -102,6 +103,12 @@ class DecodeLoop:
         # the attention kernel's split of the context is fixed per launch: one graph per bucket of 1,024 tokens
         bucket = min(self.cap, -(-(max(self.lens) + 1) // 1024) * 1024)
         self.ctx.host["max_context"] = bucket
+        if eng.workspace.epoch != self.epoch:
+            # other steps of the engine made a workspace buffer grow since the graphs were captured: they hold
+            # the old buffers' addresses, so they are captured again
+            self.graphs.clear()
+            self.warm.clear()
+            self.epoch = eng.workspace.epoch
         graph = self.graphs.get(bucket)
         if not self.use_graph:
             self._run()

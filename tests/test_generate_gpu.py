@@ -215,3 +215,41 @@ def test_the_command_line(model_dirs, tmp_path):
     toks = [int(t) for t in r.stdout.split()]
     c, w = plain.load_folder(str(out))
     assert toks == plain.greedy(w, c, [5, 17, 3], 8) and "prefill 3 tokens" in r.stderr
+
+
+def test_decode_loop_replays_graphs_like_plain_steps(model_dirs):
+    """The decode loop with HIP graph replay against the same loop without graphs, token by token, over
+    a boundary between context buckets (a second graph is captured), with the engine's own eager steps
+    between the replays: prefills of another request, one of them larger than any step before, so that
+    workspace buffers grow and the graphs have to be captured again."""
+    from glassbox_amd.engine import Engine
+    from glassbox_amd.engine.decode_loop import DecodeLoop
+    folder = model_dirs.get("M")
+    vocab = helpers.TINY["M"]["vocab_size"]
+    prompts = {"p": helpers.random_tokens(vocab, 1000, seed=41), "q": helpers.random_tokens(vocab, 700, seed=42),
+               "r": helpers.random_tokens(vocab, 1015, seed=43)}
+    extra = helpers.random_tokens(vocab, 1500, seed=44)
+    loops = []
+    for use_graph in (True, False):
+        eng = Engine(folder, dtype="bfloat16", max_tokens=8192, max_seqs=8)
+        for name, toks in prompts.items():
+            for at in range(0, len(toks) - 1, 512):
+                eng.step([(name, toks[at:min(at + 512, len(toks) - 1)], [])])
+        loops.append((eng, DecodeLoop(eng, list(prompts), [t[-1] for t in prompts.values()], use_graph=use_graph)))
+    for step in range(48):
+        got = [loop.step() for _, loop in loops]
+        assert got[0] == got[1], f"step {step}: graph replay {got[0]}, plain steps {got[1]}"
+        if step in (9, 20, 33):                       # the engine does other work between replays
+            n = {9: 300, 20: 1500, 33: 64}[step]
+            for eng, _ in loops:
+                eng.step([("other", extra[:n], [n - 1])])
+                eng.end_request("other")
+    graphed = loops[0][1]
+    assert len(graphed.graphs) >= 1 and graphed.epoch > 0           # buffers grew once, graphs were captured again
+    for eng, loop in loops:
+        loop.close()
+        for name in prompts:
+            eng.end_request(name)
+        eng.cache.check_invariants()
+        assert eng.cache.used_pages() == 0
+
