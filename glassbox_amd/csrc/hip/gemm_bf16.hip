@@ -86,9 +86,17 @@ constexpr int TKS = TBK / 16;           // MFMA k-steps per LDS k-step
 
 template <int WM, int WN, int DEPTH, int EPI, bool KFULL, typename CT>
 __global__ __launch_bounds__(256, WN == 2 ? 2 : 1) void gemm_tiled_kernel(const bf16* __restrict__ a, int lda, const bf16* __restrict__ w,
-                                                         int ldw, CT* __restrict__ c, int ldc, int M, int N, int K) {
+                                                         int ldw, CT* __restrict__ c, int ldc, int M, int N, int K,
+                                                         int k_slice) {
   constexpr int BM = 64 * WM, BN = 64 * WN;
   constexpr int CA = BM * TCPR / 256, CW = BN * TCPR / 256;  // chunks a thread moves per k-step
+  if (k_slice > 0) {  // split k: workgroup z of a tile sums its own slice of k into its own copy of C
+    const int z = blockIdx.z;
+    a += (size_t)z * k_slice;
+    w += (size_t)z * k_slice;
+    c += (size_t)z * M * ldc;
+    K = min(k_slice, K - z * k_slice);
+  }
   __shared__ __attribute__((aligned(16))) bf16 As[2][BM][TLD];
   __shared__ __attribute__((aligned(16))) bf16 Ws[2][BN][TLD];
   const int tid = threadIdx.x, lane = tid % 64, wave = tid / 64;
@@ -283,15 +291,85 @@ int launch_tiled(const bf16* a, int lda, const bf16* w, int ldw, CT* c, int ldc,
   if (wn == (B) && depth == (D)) {                                                                                          \
     if (kfull)                                                                                                              \
       hipLaunchKernelGGL((gemm_tiled_kernel<2, (B), (D), EPI, true, CT>), grid, block, 0, stream, a, lda, w, ldw, c, ldc, M, \
-                         N, K);                                                                                             \
+                         N, K, 0);                                                                                          \
     else                                                                                                                    \
       hipLaunchKernelGGL((gemm_tiled_kernel<2, (B), (D), EPI, false, CT>), grid, block, 0, stream, a, lda, w, ldw, c, ldc,   \
-                         M, N, K);                                                                                          \
+                         M, N, K, 0);                                                                                       \
   }
   GB_T(2, 1) GB_T(2, 2)
   if (EPI != EPI_SILU_MUL) { GB_T((EPI == EPI_SILU_MUL ? 2 : 1), 1) GB_T((EPI == EPI_SILU_MUL ? 2 : 1), 2) }
 #undef GB_T
   return launched("gemm_bf16 (tiled)");
+}
+
+// ------------------------------------------------------------------------ split k
+// A product with few tiles (17 to a few hundred rows, or few rows of W) leaves most compute units idle
+// and, as a skinny product, makes every workgroup read all of A.  Here the tiled kernel's workgroups
+// also divide k: workgroup (tile, z) sums slice z of k into copy z of a float32 C in a workspace, and a
+// second kernel adds the copies in the order of z and applies the epilogue.  Tiles of 64 or 128 rows.
+struct SplitPlan {
+  int bm, slices, k_slice;
+  size_t floats;  // of workspace
+};
+
+inline SplitPlan split_plan(int M, int N, int K) {
+  SplitPlan p{M <= 64 ? 64 : 128, 1, 0, 0};
+  const int tiles = ((N + 127) / 128) * ((M + p.bm - 1) / p.bm);
+  if (tiles >= 192 || N % 8 != 0) return p;
+  // measured on SmolLM2-1.7B shapes: a long k (the down projection) always gains; a short one only where
+  // the skinny kernel is at its weakest (33 to 64 rows: every workgroup reads all of A)
+  if (K < 4096 && !(M > 32 && M <= 64)) return p;
+  // a slice keeps at least 8 k-steps (shorter ones cost more in partial sums than they gain)
+  int want = (512 + tiles - 1) / tiles;
+  want = want > 16 ? 16 : want;
+  if (want > K / (8 * TBK)) want = K / (8 * TBK);
+  if (want < 2) return p;
+  p.k_slice = ((K + want - 1) / want + TBK - 1) / TBK * TBK;
+  p.slices = (K + p.k_slice - 1) / p.k_slice;
+  if (p.slices < 2) return SplitPlan{p.bm, 1, 0, 0};
+  p.floats = (size_t)p.slices * M * N;
+  return p;
+}
+
+// ws: [slices][M][N] float32.  Four columns a thread; EPI_SILU_MUL pairs column j with column N/2 + j.
+template <int EPI, typename CT>
+__global__ void splitk_reduce_kernel(const float* __restrict__ ws, int slices, CT* __restrict__ c, int ldc, int M, int N) {
+  const int cols = EPI == EPI_SILU_MUL ? N / 2 : N, groups = cols / 4;
+  const size_t idx = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (idx >= (size_t)M * groups) return;
+  const int m = (int)(idx / groups), j = (int)(idx % groups) * 4;
+  f32x4 sum = {0.f, 0.f, 0.f, 0.f}, up = {0.f, 0.f, 0.f, 0.f};
+  for (int z = 0; z < slices; ++z) {
+    const float* row = ws + ((size_t)z * M + m) * N;
+    sum += *reinterpret_cast<const f32x4*>(row + j);
+    if (EPI == EPI_SILU_MUL) up += *reinterpret_cast<const f32x4*>(row + N / 2 + j);
+  }
+  CT* out = c + (size_t)m * ldc + j;
+#pragma unroll
+  for (int e = 0; e < 4; ++e) {
+    float v = sum[e];
+    if (EPI == EPI_SILU_MUL) v = v / (1.0f + __expf(-v)) * up[e];
+    store_c<CT>(out + e, v, EPI == EPI_ACCUMULATE);
+  }
+}
+
+template <int EPI, typename CT>
+int launch_split(const bf16* a, int lda, const bf16* w, int ldw, CT* c, int ldc, int M, int N, int K, float* ws,
+                 const SplitPlan& plan, hipStream_t stream) {
+  const dim3 grid((N + 127) / 128, (M + plan.bm - 1) / plan.bm, plan.slices), block(256);
+  const bool kfull = K % TBK == 0;
+#define GB_S(WM, FULL)                                                                                                   \
+  if ((plan.bm == 64 * WM) && kfull == FULL)                                                                             \
+    hipLaunchKernelGGL((gemm_tiled_kernel<WM, 2, 1, EPI_STORE, FULL, float>), grid, block, 0, stream, a, lda, w, ldw, ws, \
+                       N, M, N, K, plan.k_slice);
+  GB_S(1, true) GB_S(1, false) GB_S(2, true) GB_S(2, false)
+#undef GB_S
+  if (int rc = launched("gemm_bf16 (split k)")) return rc;
+  const int cols = EPI == EPI_SILU_MUL ? N / 2 : N;
+  const size_t threads = (size_t)M * (cols / 4);
+  hipLaunchKernelGGL((splitk_reduce_kernel<EPI, CT>), dim3((unsigned)((threads + 255) / 256)), dim3(256), 0, stream, ws,
+                     plan.slices, c, ldc, M, N);
+  return launched("gemm_bf16 (split k, second pass)");
 }
 
 // ------------------------------------------------------------------------ skinny
@@ -747,16 +825,23 @@ int launch_skinny(const void* a, int lda, const bf16* w, int ldw, CT* c, int ldc
 // gamma != nullptr (at most 64 rows, bfloat16 C, epilogue 0 or 2): a is the float32 residual and the
 // product is that of its RMS-normed rows: bf16(gamma * x) as the operand, 1/sqrt(mean(x^2) + eps) on
 // the result.
+// split_ws != nullptr: a workspace of split_ws_floats floats that the product may use to divide k over
+// workgroups (gb_gemm_bf16_split_floats says how many it needs; fewer than that is an error).
 // emit_h != nullptr (accumulating product that gb_gemm_bf16_emit_parts accepts): the next norm's operand and
 // partial sums are written beside the residual, see NormExtras.  parts != nullptr (at most 8 rows, no
 // gamma): the rows of a are such an operand and the product is scaled by the norm's factor from n_parts
 // partial sums; eps is that norm's.
 extern "C" int gb_gemm_bf16_emit_parts(int M, int N) { return fold_pays(M, N) ? (N + 7) / 8 : 0; }
 
+// Floats of workspace with which gb_gemm_bf16 would split k for this product (0: it would not).
+extern "C" long long gb_gemm_bf16_split_floats(int M, int N, int K) {
+  return M > 16 ? (long long)split_plan(M, N, K).floats : 0;
+}
+
 extern "C" int gb_gemm_bf16(const void* a, int lda, const void* w, int ldw, void* c, int ldc, int c_dtype, int M, int N,
                             int K, int epilogue, const void* gamma, int gamma_dtype, float eps, const void* emit_gamma,
                             int emit_gamma_dtype, void* emit_h, int emit_ldh, float* emit_ss, const float* parts, int n_parts,
-                            hipStream_t stream) {
+                            float* split_ws, long long split_ws_floats, hipStream_t stream) {
   GB_REQUIRE(M >= 0 && N > 0 && K > 0, "gemm_bf16: bad sizes M=%d N=%d K=%d", M, N, K);
   GB_REQUIRE(K % 8 == 0, "gemm_bf16: the inner size K=%d must be a multiple of 8 (16-byte operand loads)", K);
   GB_REQUIRE(ldw % 8 == 0 && lda % (gamma ? 4 : 8) == 0, "gemm_bf16: row strides (%d, %d) must keep rows 16-byte aligned", lda, ldw);
@@ -778,6 +863,21 @@ extern "C" int gb_gemm_bf16(const void* a, int lda, const void* w, int ldw, void
   const NormExtras extra{emit_gamma, emit_gamma_dtype == kF32, (bf16*)emit_h, emit_ldh, emit_ss, parts, n_parts};
   if (M == 0) return 0;
   const bf16* W = (const bf16*)w;
+  if (split_ws != nullptr && M > 16 && !gamma && !emit_h && !parts) {  // more than the skinny kernels' best range
+    const SplitPlan plan = split_plan(M, N, K);
+    if (plan.slices > 1 && (epilogue != EPI_SILU_MUL || N % 16 == 0) && (uintptr_t)split_ws % 16 == 0) {
+      GB_REQUIRE((long long)plan.floats <= split_ws_floats, "gemm_bf16: the split-k workspace holds %lld floats, %zu are needed",
+                 split_ws_floats, plan.floats);
+      const bf16* A = (const bf16*)a;
+#define GB_SP(EPI, CT) return launch_split<EPI, CT>(A, lda, W, ldw, (CT*)c, ldc, M, N, K, split_ws, plan, stream)
+      if (epilogue == EPI_ACCUMULATE) GB_SP(EPI_ACCUMULATE, float);
+      if (epilogue == EPI_SILU_MUL && c_dtype == kBF16) GB_SP(EPI_SILU_MUL, bf16);
+      if (epilogue == EPI_SILU_MUL) GB_SP(EPI_SILU_MUL, float);
+      if (c_dtype == kF32) GB_SP(EPI_STORE, float);
+      GB_SP(EPI_STORE, bf16);
+#undef GB_SP
+    }
+  }
   if (M <= 64) {
     const int gf = gamma_dtype == kF32;
     if (fold_pays(M, N) && epilogue != EPI_SILU_MUL && !parts) {

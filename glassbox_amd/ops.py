@@ -52,8 +52,10 @@ _SIGS = {
     },
     "gemm_bf16": {
         # a, lda, w, ldw, c, ldc, c_dtype, M, N, K, epilogue, gamma, gamma_dtype, eps,
-        # emit_gamma, emit_gamma_dtype, emit_h, emit_ldh, emit_ss, parts, n_parts, stream
-        "gb_gemm_bf16": [_vp, _i, _vp, _i, _vp, _i, _i, _i, _i, _i, _i, _vp, _i, _f, _vp, _i, _vp, _i, _vp, _vp, _i, _vp],
+        # emit_gamma, emit_gamma_dtype, emit_h, emit_ldh, emit_ss, parts, n_parts, split_ws, split_ws_floats, stream
+        "gb_gemm_bf16": [_vp, _i, _vp, _i, _vp, _i, _i, _i, _i, _i, _i, _vp, _i, _f, _vp, _i, _vp, _i, _vp, _vp, _i, _vp,
+                         C.c_longlong, _vp],
+        "gb_gemm_bf16_split_floats": [_i, _i, _i],
         "gb_gemm_bf16_emit_parts": [_i, _i],
         # a, lda, w, ldw, c, ldc, M, N, K, gamma, gamma_dtype, eps, parts, n_parts, cos, sin, slots, k, v,
         # nh, nkv, hd, page, stream
@@ -260,8 +262,17 @@ def gemm_emit_parts(rows: int, n: int) -> int:
     return int(_lib("gemm_bf16").gb_gemm_bf16_emit_parts(int(rows), int(n)))
 
 
+def gemm_split_floats(rows: int, n: int, k: int) -> int:
+    """Floats of workspace with which a bfloat16 product of these sizes would divide k over workgroups
+    (``gemm(..., workspace=)``); 0 if it would not: only products with few tiles do."""
+    f = _lib("gemm_bf16").gb_gemm_bf16_split_floats
+    f.restype = C.c_longlong
+    return int(f(int(rows), int(n), int(k)))
+
+
 def gemm(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor, accumulate: bool = False, silu_mul: bool = False,
-         rms: Optional[tuple] = None, emit: Optional[tuple] = None, rms_parts: Optional[tuple] = None) -> None:
+         rms: Optional[tuple] = None, emit: Optional[tuple] = None, rms_parts: Optional[tuple] = None,
+         workspace: Optional[torch.Tensor] = None) -> None:
     """out (+)= a . w^T with w in the [out features, in features] layout.
     float32 operands take the true 32-bit kernel; bfloat16 operands the matrix-core kernels,
     with out in bfloat16 or float32 (float32 when accumulating into the residual).
@@ -273,7 +284,9 @@ def gemm(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor, accumulate: bool =
     the new residual r in out, h[m, n] = bf16(gamma[n] r[m, n]) and float32 parts[tile, m] (8 columns a
     tile) of sum(r^2) are written: the work of the RMS norm that reads the residual next.
     ``rms_parts=(parts, n_parts, eps)`` (at most 8 rows): a is such an h, and the product is scaled by
-    1 / sqrt(sum(parts[:, m]) / K + eps) to that of the normed rows."""
+    1 / sqrt(sum(parts[:, m]) / K + eps) to that of the normed rows.
+    ``workspace`` (float32, at least ``gemm_split_floats(M, N, K)`` elements): lets a bfloat16 product of
+    more than 16 rows and few tiles divide k over workgroups; their sums are added in a fixed order."""
     _dev(a, w, out)
     M, K = a.shape
     N = w.shape[0]
@@ -293,7 +306,7 @@ def gemm(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor, accumulate: bool =
         lib = _lib("gemm_bf16")
         _check(lib, lib.gb_gemm_bf16(_p(a), lda, _p(w), ldw, _p(out), ldc, BF16, M, N, K, 2 if silu_mul else 0,
                                      _p(gamma), dtype_code(gamma), float(eps), None, 0, None, 0, None, None, 0,
-                                     _stream()))
+                                     None, 0, _stream()))
     elif a.dtype == torch.float32 and w.dtype == torch.float32:
         if out.dtype != torch.float32:
             raise KernelError("gemm: 32-bit operands need a 32-bit result")
@@ -303,6 +316,10 @@ def gemm(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor, accumulate: bool =
         if accumulate and out.dtype != torch.float32:
             raise KernelError("gemm: accumulation is into a 32-bit result")
         lib = _lib("gemm_bf16")
+        if workspace is not None:
+            _dev(workspace)
+            if workspace.dtype != torch.float32 or not workspace.is_contiguous():
+                raise KernelError("gemm: the workspace must be contiguous float32")
         e_gamma = e_h = e_ss = parts = None
         e_ldh = n_parts = 0
         eps = 0.0
@@ -325,7 +342,8 @@ def gemm(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor, accumulate: bool =
         _check(lib, lib.gb_gemm_bf16(_p(a), lda, _p(w), ldw, _p(out), ldc, dtype_code(out), M, N, K,
                                      2 if silu_mul else (1 if accumulate else 0), None, 0, float(eps),
                                      _p(e_gamma), dtype_code(e_gamma) if e_gamma is not None else 0, _p(e_h), e_ldh,
-                                     _p(e_ss), _p(parts), int(n_parts), _stream()))
+                                     _p(e_ss), _p(parts), int(n_parts), _p(workspace),
+                                     workspace.numel() if workspace is not None else 0, _stream()))
     else:
         raise KernelError(f"gemm: operand types {a.dtype} and {w.dtype} do not match a kernel")
 

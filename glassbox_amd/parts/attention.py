@@ -15,7 +15,7 @@ from typing import Dict, Optional
 import torch
 
 from .. import ops
-from .base import FULL, WINDOW, CacheSpec, LayerCache, Mixer, PositionEncoding, PreNormed, TensorSpec, emit_target
+from .base import FULL, WINDOW, CacheSpec, LayerCache, Mixer, PositionEncoding, PreNormed, TensorSpec, emit_target, split_workspace
 
 
 class PagedAttention(Mixer):
@@ -82,10 +82,12 @@ class PagedAttention(Mixer):
             if pre:
                 ops.gemm(norm.rows, self.wqkv, qkv, rms_parts=norm.as_gemm_arg())
             else:
-                ops.gemm(h, self.wqkv, qkv, rms=norm)
+                ops.gemm(h, self.wqkv, qkv, rms=norm,
+                         workspace=None if norm is not None else split_workspace(ctx, n, rows, self.width))
             self.position.apply_and_store(ctx, qkv, self.n_heads, n_kv, self.head_dim, *store)
         att = ctx.buffer("att", (n, self.q_dim), ctx.dtype)
         ctx.attention(qkv[:, :self.q_dim], att, cache, self.n_heads, self.scale, self.window)
         target, handed_on = emit_target(ctx, n, self.width, emit, "mixer")
-        ops.gemm(att, self.wo, residual, accumulate=True, emit=target)
+        ops.gemm(att, self.wo, residual, accumulate=True, emit=target,
+                 workspace=split_workspace(ctx, n, self.width, self.q_dim))
         return handed_on

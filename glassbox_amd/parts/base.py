@@ -150,6 +150,16 @@ def emit_target(ctx, n: int, width: int, emit, tag: str):
     return (gamma, rows, parts), PreNormed(rows, parts, n_parts, float(eps))
 
 
+def split_workspace(ctx, n: int, out_features: int, in_features: int):
+    """A workspace for ``ops.gemm(..., workspace=)`` if a product of these sizes would divide k over
+    workgroups in this step, else None."""
+    from .. import ops
+    if ctx.dtype != torch.bfloat16 or n <= 16:
+        return None
+    floats = ops.gemm_split_floats(n, out_features, in_features)
+    return ctx.buffer("gemm_split", (floats,), torch.float32) if floats else None
+
+
 class Mixer(Part):
     cache_spec: Optional[CacheSpec] = None
     state_spec: Optional[StateSpec] = None

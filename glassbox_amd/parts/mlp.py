@@ -7,7 +7,7 @@ from typing import Dict, Optional
 import torch
 
 from .. import ops
-from .base import FeedForward, PreNormed, TensorSpec, emit_target
+from .base import FeedForward, PreNormed, TensorSpec, emit_target, split_workspace
 
 
 class SwiGLU(FeedForward):
@@ -38,7 +38,8 @@ class SwiGLU(FeedForward):
             ops.gemm(norm.rows, self.w_gate_up, act, silu_mul=True, rms_parts=norm.as_gemm_arg())
         elif ctx.dtype == torch.bfloat16 and self.intermediate % 8 == 0:
             # the activation is applied where the product's tile is finished: gate_up never reaches memory
-            ops.gemm(h, self.w_gate_up, act, silu_mul=True, rms=norm)
+            ops.gemm(h, self.w_gate_up, act, silu_mul=True, rms=norm,
+                     workspace=None if norm is not None else split_workspace(ctx, n, 2 * self.intermediate, self.width))
         else:
             if norm is not None:   # nothing to fuse it into here: the norm gets its own pass after all
                 normed = ctx.buffer("h", (n, self.width), ctx.dtype)
@@ -48,5 +49,6 @@ class SwiGLU(FeedForward):
             ops.gemm(h, self.w_gate_up, gate_up)
             ops.silu_mul(gate_up, act)
         target, handed_on = emit_target(ctx, n, self.width, emit, "ffn")
-        ops.gemm(act, self.w_down, residual, accumulate=True, emit=target)
+        ops.gemm(act, self.w_down, residual, accumulate=True, emit=target,
+                 workspace=split_workspace(ctx, n, self.width, self.intermediate))
         return handed_on

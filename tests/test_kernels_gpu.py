@@ -154,6 +154,39 @@ def test_gemm_bf16_prepares_the_next_norm(M, N, K, N2, silu, gamma_dtype):
     assert ((out.float() - again.float()).abs() <= 2 ** -6 * (1 + again.float().abs())).all()
 
 
+@pytest.mark.parametrize("M,N,K", [(17, 96, 4096), (33, 2048, 2048), (64, 2048, 8192), (64, 6144, 2048), (100, 2048, 4160),
+                                   (200, 528, 8200), (64, 16384, 2048), (40, 1008, 4104), (512, 2048, 8192)])
+@pytest.mark.parametrize("mode", ["bf16", "f32", "f32+", "silu"])
+def test_gemm_bf16_divides_k_over_workgroups(M, N, K, mode):
+    """With a workspace, a product of few tiles has several workgroups a tile, each over a slice of k,
+    and a second kernel adds their sums in a fixed order and applies the epilogue: against float64, and
+    the same bits on every run."""
+    from glassbox_amd import ops
+    floats = ops.gemm_split_floats(M, N, K)
+    assert floats > 0 and floats % (M * N) == 0 and floats // (M * N) >= 2
+    a, w = rnd(M, K, seed=1).bfloat16(), (rnd(N, K, seed=2) / math.sqrt(K)).bfloat16()
+    c0 = rnd(M, N, seed=3)
+    prod = a.double() @ w.double().T
+    if mode == "silu":
+        want = prod[:, :N // 2] / (1 + torch.exp(-prod[:, :N // 2])) * prod[:, N // 2:]
+    else:
+        want = prod + (c0.double() if mode == "f32+" else 0)
+    ws = torch.full((floats + 3,), float("nan"), device=DEV)[:floats]
+    outs = []
+    for _ in range(2):
+        if mode == "silu":
+            c = torch.full((M, N // 2), 7.0, device=DEV, dtype=torch.bfloat16)
+        else:
+            c = to_dev(c0.clone(), torch.bfloat16 if mode == "bf16" else torch.float32)
+        ops.gemm(to_dev(a), to_dev(w), c, accumulate=(mode == "f32+"), silu_mul=(mode == "silu"), workspace=ws)
+        outs.append(c)
+    tol = 1e-4 * math.sqrt(K) + (2 ** -8) * want.abs().max().item() * (mode in ("bf16", "silu"))
+    assert (outs[0].cpu().double() - want).abs().max().item() <= tol
+    assert torch.equal(outs[0], outs[1])
+    with pytest.raises(ops.KernelError, match="workspace"):
+        ops.gemm(to_dev(a), to_dev(w), outs[0], accumulate=(mode == "f32+"), silu_mul=(mode == "silu"), workspace=ws[:8])
+
+
 def test_gemm_bf16_split_k_is_the_same_on_every_run():
     from glassbox_amd import ops
     a, w = to_dev(rnd(8, 8192, seed=1).bfloat16()), to_dev(rnd(2048, 8192, seed=2).bfloat16())
