@@ -55,6 +55,9 @@ def _host():
             fn = getattr(lib, "gbh_cache_" + name)
             fn.argtypes = [C.c_void_p] + args
             fn.restype = C.c_int
+        lib.gbh_cache_decode_rows.restype = C.c_int
+        lib.gbh_cache_decode_rows.argtypes = [C.c_void_p, C.POINTER(C.c_int64), C.c_int, C.c_int] + [C.c_void_p] * 2 + \
+                                             [C.c_void_p, C.c_int, C.c_void_p, C.c_int]
         lib.gbh_chain_hash.restype = C.c_uint64
         lib.gbh_chain_hash.argtypes = [C.c_uint64, i32p, C.c_int]
         _lib = lib
@@ -159,6 +162,19 @@ class CacheManager:
             self._table_buf = (C.c_int32 * (2 * n))()
             n = self._lib.gbh_cache_table(self._h, seq_id, group, self._table_buf, len(self._table_buf))
         return self._table_buf[:n]
+
+    def decode_rows(self, seq_ids: Sequence[int], stride: int, pos_ptr: int, state_ptr: int, rows_ptr: int,
+                    rows_gap: int, tables_ptr: int, tables_gap: int) -> None:
+        """For requests that bring one token each, writes into the caller's int32 arrays (given as addresses, for
+        instance of a pinned buffer): each request's length and state slot, and per group the cache row of the new
+        token ([group][request], ``rows_gap`` entries between groups) and the block table padded with -1 to
+        ``stride`` entries ([group][request][stride], ``tables_gap`` entries between groups)."""
+        ids = (C.c_int64 * max(1, len(seq_ids)))(*seq_ids)
+        rc = self._lib.gbh_cache_decode_rows(self._h, ids, len(seq_ids), stride, pos_ptr, state_ptr, rows_ptr,
+                                             rows_gap, tables_ptr, tables_gap)
+        if rc:
+            raise CacheError({-1: "unknown request", -2: f"a block table is longer than {stride} pages",
+                              -3: "the page of a new token is not reserved"}.get(rc, f"error {rc}"))
 
     def slot(self, seq_id: int, pos: int, group: int = 0) -> int:
         """Row of (request, position) in a layer's pages (kv.rs:199-201)."""

@@ -22,6 +22,8 @@ USAGE = """usage:
   glassbox batch    --model DIR --prompts FILE [-n 128] ...      (one prompt of ids per line; continuous batching)
   glassbox random   --config FILE.json --out DIR [--seed 0] [--dtype float32|bfloat16] [--norm ones|uniform]
   glassbox bench single --model DIR [--dtype ...] [--label L] [--out FILE]      (pp512 / tg128, as glassbox-bench)
+  glassbox bench serve  --model DIR [--dtype ...] [--workload chat|system|long] [--requests N] [--rates R,R,...]
+                        [--blocks N] [--budget 512] [--max-seqs 32] [--out FILE]    (requests against the clock)
   glassbox replay   --model DIR --dtype D --out DIR --max-tokens N              (same as bin/trace_run)"""
 
 
@@ -170,6 +172,108 @@ def cmd_bench_single(a) -> int:
     return 0
 
 
+def _quantile(values, p):
+    v = sorted(values)
+    return v[round((len(v) - 1) * p)] if v else 0.0
+
+
+def _serve_run(eng, budget, max_seqs, prompts, outputs, rate):
+    """One load through the scheduler in real time (crates/glassbox-bench/src/main.rs:241-288): exponential gaps
+    between arrivals at ``rate`` requests a second (all at once when the rate is infinite), greedy replies of
+    the given lengths."""
+    import math
+    from .engine.scheduler import Scheduler, SchedulerConfig
+    from .sampling import Rng
+    rng, t, times = Rng(42), 0.0, []
+    for _ in prompts:
+        t += 0.0 if math.isinf(rate) else -math.log(1.0 - rng.next_f32()) / rate
+        times.append(t)
+    s = Scheduler(eng, SchedulerConfig(token_budget=budget, max_seqs=max_seqs))
+    t0, nxt = time.perf_counter(), 0
+    while nxt < len(times) or not s.is_idle():
+        now = time.perf_counter() - t0
+        while nxt < len(times) and times[nxt] <= now:
+            s.submit(prompts[nxt], outputs[nxt], arrival=t0 + times[nxt])
+            nxt += 1
+        if s.is_idle():
+            time.sleep(max(0.0, times[nxt] - now))
+            continue
+        s.step()
+    import torch
+    torch.cuda.synchronize()
+    wall = time.perf_counter() - t0
+    m = s.metrics
+    return {"rate_rps": None if math.isinf(rate) else rate, "requests": len(prompts), "wall_s": wall,
+            "throughput_tok_s": m["generated_tokens"] / wall,
+            "total_tok_s": (m["generated_tokens"] + m["prompt_tokens"] - m["prefix_hit_tokens"]) / wall,
+            "ttft_p50_s": _quantile(s.ttft, 0.5), "ttft_p99_s": _quantile(s.ttft, 0.99),
+            "itl_p50_s": _quantile(s.itl, 0.5), "itl_p99_s": _quantile(s.itl, 0.99),
+            "prefix_hit_tokens": m["prefix_hit_tokens"], "prompt_tokens": m["prompt_tokens"],
+            "preemptions": m["preemptions"], "steps": m["steps"],
+            "mean_batch_tokens": m["batch_tokens"] / max(1, m["steps"])}
+
+
+def serve_load(workload: str, n: int, vocab: int):
+    """Prompts and reply lengths of a serving load, as seeded random token ids.  ``chat`` and ``system`` are the
+    reference's two loads (crates/glassbox-bench/src/main.rs:296-318): prompts of 32-320 tokens with replies of
+    32-256; a 384-token prompt that every request shares, 16-64 tokens of its own and replies of 16-64.  ``long``
+    has prompts of 32-2048 tokens and replies of 32-256, every other request starting with one 384-token prefix."""
+    from .sampling import Rng
+    ids, lens = Rng(7), Rng(9)
+    toks = lambda k: [int(ids.next_f32() * vocab) for _ in range(k)]
+    span = lambda lo, width: lo + int(lens.next_f32() * width)
+    if workload == "chat":
+        prompts = [toks(span(32, 288)) for _ in range(n)]
+        return prompts, [span(32, 224) for _ in range(n)]
+    if workload == "system":
+        system = toks(384)
+        prompts = [system + toks(span(16, 48)) for _ in range(n)]
+        return prompts, [span(16, 48) for _ in range(n)]
+    if workload == "long":
+        system, prompts = toks(384), []
+        for i in range(n):
+            k = span(32, 2017)
+            prompts.append((system + toks(max(1, k - 384))) if i % 2 else toks(k))
+        return prompts, [span(32, 225) for _ in range(n)]
+    raise ValueError(f"no serving load is called {workload!r}")
+
+
+def cmd_bench_serve(a) -> int:
+    """Requests that arrive against the clock, through the scheduler (crates/glassbox-bench/src/main.rs:290-371):
+    throughput, time to the first token and between tokens, with and without the prefix cache where prompts
+    share a beginning.  A warm-up pass of a few requests comes first, untimed."""
+    import torch
+    from .engine import Engine
+    rates = [float(r) for r in a.rates.replace(",", " ").split()]
+    runs = []
+    modes = [("prefix cache", True), ("no prefix cache", False)] if a.workload != "chat" else [("continuous batching", False)]
+    for name, prefix in modes:
+        for rate in rates:
+            # a cache of its own for every run, as the reference builds a scheduler for each (main.rs:245): idle
+            # pages keep their prefixes, and a run must not find those of the run before
+            eng = Engine(a.model, dtype=a.dtype, max_tokens=a.blocks * 16, max_seqs=a.max_seqs, prefix_caching=prefix)
+            vocab = eng.model.vocab_size
+            prompts, outputs = serve_load(a.workload, a.requests, vocab)
+            warm = [[(i * 7919 + 13 + j) % vocab for i in range(k)] for j, k in enumerate((700, 40, 300, 90))]
+            _serve_run(eng, a.budget, a.max_seqs, warm, [8] * len(warm), float("inf"))
+            r = _serve_run(eng, a.budget, a.max_seqs, prompts, outputs, rate)
+            print(f"{name:20} {rate:5} req/s: {r['throughput_tok_s']:.0f} tok/s, TTFT p50 {r['ttft_p50_s']:.3f}s "
+                  f"p99 {r['ttft_p99_s']:.3f}s, ITL p50 {r['itl_p50_s'] * 1e3:.2f}ms, {r['prefix_hit_tokens']} prompt "
+                  f"tokens reused, {r['preemptions']} preemptions", file=sys.stderr)
+            runs.append({"workload": a.workload, "mode": name, "result": r})
+            del eng
+    res = {"engine": "glassbox_amd", "model": a.model, "dtype": a.dtype, "token_budget": a.budget,
+           "max_seqs": a.max_seqs, "blocks": a.blocks, "runs": runs,
+           "meta": {"gpu": torch.cuda.get_device_name(0), "date": time.strftime("%Y-%m-%dT%H:%M:%SZ", time.gmtime())}}
+    text = json.dumps(res, indent=2)
+    if a.out:
+        with open(a.out, "w") as fh:
+            fh.write(text + "\n")
+    else:
+        print(text)
+    return 0
+
+
 def main(argv=None) -> int:
     ap = argparse.ArgumentParser(prog="glassbox", usage=USAGE)
     sub = ap.add_subparsers(dest="cmd")
@@ -185,6 +289,12 @@ def main(argv=None) -> int:
     bsub = be.add_subparsers(dest="bench_cmd")
     bs = bsub.add_parser("single"); _add_model(bs)
     bs.add_argument("--label", default=None); bs.add_argument("--out", default=None)
+    bv = bsub.add_parser("serve"); _add_model(bv)
+    bv.add_argument("--workload", default="chat", choices=["chat", "system", "long"])
+    bv.add_argument("--requests", type=int, default=48)
+    bv.add_argument("--rates", default="inf", help="requests a second, several separated by commas; inf = all at once")
+    bv.add_argument("--blocks", type=int, default=4096); bv.add_argument("--budget", type=int, default=512)
+    bv.add_argument("--max-seqs", type=int, default=32); bv.add_argument("--out", default=None)
     rp = sub.add_parser("replay"); _add_model(rp)
     rp.add_argument("--out", required=True); rp.add_argument("--max-tokens", type=int, required=True)
     a = ap.parse_args(argv)
@@ -196,6 +306,8 @@ def main(argv=None) -> int:
         return cmd_random(a)
     if a.cmd == "bench" and a.bench_cmd == "single":
         return cmd_bench_single(a)
+    if a.cmd == "bench" and a.bench_cmd == "serve":
+        return cmd_bench_serve(a)
     if a.cmd == "replay":
         import os
         import subprocess

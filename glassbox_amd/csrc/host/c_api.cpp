@@ -49,6 +49,33 @@ int gbh_cache_table(void* h, int64_t id, int group, int32_t* out, int cap) {
   if (out) std::memcpy(out, t->data(), sizeof(int32_t) * (size_t)(n < cap ? n : cap));
   return n;
 }
+// What a step of one token per request needs, written straight into the caller's (pinned) arrays: per request
+// its length (the new token's position) and state slot, and per group the cache row of the new token and the
+// block table, padded with -1 to `stride` entries.  rows and tables are laid out [group][request] and
+// [group][request][stride], with `group_gap` entries from one group's array to the next.  Returns 0; -1 for an
+// unknown request; -2 if a table is longer than stride; -3 if the page of the new position is not reserved.
+int gbh_cache_decode_rows(void* h, const int64_t* ids, int n, int stride, int32_t* pos, int32_t* state_slot,
+                          int32_t* rows, int rows_gap, int32_t* tables, int tables_gap) {
+  auto* cm = (CacheManager*)h;
+  const int page = cm->page_size(), groups = cm->num_groups();
+  for (int i = 0; i < n; ++i) {
+    int len = cm->seq_len(ids[i]);
+    if (len < 0) return -1;
+    pos[i] = len;
+    state_slot[i] = cm->state_slot(ids[i]);
+    for (int g = 0; g < groups; ++g) {
+      const std::vector<int32_t>& t = *cm->table(ids[i], g);
+      if ((int)t.size() > stride) return -2;
+      int32_t* out = tables + (size_t)g * tables_gap + (size_t)i * stride;
+      std::memcpy(out, t.data(), sizeof(int32_t) * t.size());
+      for (int j = (int)t.size(); j < stride; ++j) out[j] = -1;
+      int lp = len / page;
+      if (lp >= (int)t.size() || t[lp] < 0) return -3;
+      rows[(size_t)g * rows_gap + i] = t[lp] * page + len % page;
+    }
+  }
+  return 0;
+}
 // Pending device copies as triples (group, src, dst); returns how many there were.
 int gbh_cache_take_copies(void* h, int32_t* out, int cap_triples) {
   auto ops = ((CacheManager*)h)->take_copies();

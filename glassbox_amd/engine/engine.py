@@ -16,6 +16,7 @@ from ..cache.manager import FULL, CacheManager, GroupSpec, OutOfPages
 from ..parts.base import LayerCache
 from ..weights.loader import compute_dtype, load_model
 from .context import StepContext, Workspace
+from .decode_graphs import DecodeGraphs
 
 Entry = Tuple[Hashable, Sequence[int], Sequence[int]]  # (request, its next tokens, wanted places among them)
 
@@ -30,10 +31,13 @@ class Engine:
     max_tokens: tokens the cache holds over all live requests (rounded up to whole pages).
     max_seqs: most live requests (= state slots).  page_size: tokens per page (16 as in the
     reference, crates/glassbox-core/src/kv.rs:11).
+    graph_decode: replay steps of one token per request from HIP graphs (engine.decode_graphs); by
+    default where the arithmetic is bfloat16 and every part of the model allows it.
     """
 
     def __init__(self, model, dtype="bfloat16", max_tokens: int = 4096, max_seqs: int = 32, page_size: int = 16,
-                 prefix_caching: bool = False, device: str = "cuda:0", attention_impl: str = "auto"):
+                 prefix_caching: bool = False, device: str = "cuda:0", attention_impl: str = "auto",
+                 graph_decode: Optional[bool] = None):
         ops.require_gpu()
         self.dtype = compute_dtype(dtype)
         self.device = torch.device(device)
@@ -66,19 +70,27 @@ class Engine:
             lc = LayerCache()
             if spec is not None:
                 lc.group = keys.index(spec.group_key)
-                shape = (num_pages, spec.num_kv_heads, self.page_size, spec.head_dim)
+                # one page and one state slot more than the manager hands out: filler rows of a replayed step
+                # write there (engine.decode_graphs)
+                shape = (num_pages + 1, spec.num_kv_heads, self.page_size, spec.head_dim)
                 lc.k_pages = torch.zeros(shape, dtype=self.dtype, device=self.device)
-                lc.v_pages = torch.zeros((num_pages, spec.num_kv_heads, spec.head_dim, self.page_size),
+                lc.v_pages = torch.zeros((num_pages + 1, spec.num_kv_heads, spec.head_dim, self.page_size),
                                          dtype=self.dtype, device=self.device)   # transposed: see ops._check_pages
             if state is not None:
-                lc.state = torch.zeros((self.max_seqs,) + tuple(state.shape), dtype=state.dtype, device=self.device)
+                lc.state = torch.zeros((self.max_seqs + 1,) + tuple(state.shape), dtype=state.dtype, device=self.device)
             self.layers.append(lc)
+        self.spare_page, self.spare_state_slot = num_pages, self.max_seqs
 
         self.workspace = Workspace(self.device)
         self._ids: Dict[Hashable, int] = {}
         self._next_id = 1 << 40   # the scheduler numbers its requests from 1 in the same cache manager
         self._meta_dev: Optional[torch.Tensor] = None
         self.steps = 0
+        if graph_decode is None:
+            graph_decode = self.dtype == torch.bfloat16
+        if graph_decode and not getattr(model, "all_replayable", lambda: False)():
+            graph_decode = False
+        self.decode_graphs = DecodeGraphs(self) if graph_decode else None
 
     # ---------------------------------------------------------------- requests
     def has_request(self, request: Hashable) -> bool:
@@ -185,10 +197,12 @@ class Engine:
             return torch.empty((0, self.model.vocab_size), dtype=torch.float32, device=self.device)
         self._validate(entries)
         self._apply_copies()
-        ctx = self._build_context(entries)
-        logits = self.model.forward(ctx, self.layers)
         self.steps += 1
-        return logits
+        graphs = self.decode_graphs
+        if graphs is not None and graphs.applies(entries):
+            return graphs.run(entries)
+        ctx = self._build_context(entries)
+        return self.model.forward(ctx, self.layers)
 
     def reset_state(self, sid: int) -> None:
         """Empties the state slot of a request that starts (again) from its first token."""

@@ -95,6 +95,11 @@ class Scheduler:
         self.outputs: Dict[int, RequestOutput] = {}
         self.trace: Optional[List[StepRecord]] = [] if trace else None
         self._steps = 0
+        #: seconds from a request's arrival to its first token, and between its later tokens (scheduler.rs:127-129)
+        self.ttft: List[float] = []
+        self.itl: List[float] = []
+        self._arrival: Dict[int, float] = {}
+        self._last_token: Dict[int, float] = {}
 
     def __del__(self):
         h, self._h = getattr(self, "_h", None), None
@@ -103,7 +108,9 @@ class Scheduler:
 
     # ------------------------------------------------------------------ requests
     def submit(self, prompt: Sequence[int], max_tokens: int, sampler: Optional[SamplerConfig] = None,
-               stop: Sequence[int] = ()) -> int:
+               stop: Sequence[int] = (), arrival: Optional[float] = None) -> int:
+        """Queues a request.  ``arrival`` (a ``time.perf_counter`` value) is when it was due, for a load that
+        is replayed against the clock (scheduler.rs:167); by default now."""
         if not prompt:
             raise ValueError("a request needs at least one prompt token")
         vocab = self.engine.model.vocab_size
@@ -115,6 +122,7 @@ class Scheduler:
         rid = self._lib.gbh_sched_submit(self._h, p, len(prompt), max_tokens, s.temperature, s.top_k, s.top_p,
                                          s.min_p, s.repetition_penalty, s.seed, st, len(stop))
         self.outputs[rid] = RequestOutput(prompt_tokens=len(prompt))
+        self._arrival[rid] = time.perf_counter() if arrival is None else arrival
         return rid
 
     def abort(self, rid: int) -> None:
@@ -185,15 +193,24 @@ class Scheduler:
         finished = []
         cap = 4096
         ids, kinds, vals = (C.c_int64 * cap)(), (C.c_int32 * cap)(), (C.c_int32 * cap)()
+        now = time.perf_counter()
         while True:
             n = self._lib.gbh_sched_take_events(self._h, ids, kinds, vals, cap)
             for i in range(min(n, cap)):
                 out = self.outputs.setdefault(ids[i], RequestOutput())
                 if kinds[i] == 0:
                     out.tokens.append(vals[i])
+                    prev = self._last_token.get(ids[i])
+                    if prev is None:
+                        self.ttft.append(now - self._arrival.get(ids[i], now))
+                    else:
+                        self.itl.append(now - prev)
+                    self._last_token[ids[i]] = now
                 else:
                     out.finish = FINISH_NAMES[vals[i]]
                     finished.append(ids[i])
+                    self._arrival.pop(ids[i], None)
+                    self._last_token.pop(ids[i], None)
             if n <= cap:
                 return finished
 

@@ -19,6 +19,8 @@ from .base import FULL, WINDOW, CacheSpec, LayerCache, Mixer, PositionEncoding, 
 
 
 class PagedAttention(Mixer):
+    replayable = True
+
     def __init__(self, width: int, n_heads: int, n_kv_heads: int, head_dim: int, position: PositionEncoding,
                  window: int = 0, shares_kv: bool = False, scale: Optional[float] = None):
         if n_heads % n_kv_heads:
@@ -45,6 +47,9 @@ class PagedAttention(Mixer):
 
     def children(self):
         return {"": self.position} if self.position.tensor_specs() else {}
+
+    def all_replayable(self) -> bool:
+        return self.replayable and self.position.all_replayable()
 
     def load(self, tensors):
         if self.shares_kv:

@@ -18,6 +18,8 @@ Interfaces (all activations are [tokens, width] tensors on the device;
       .state_spec  -> StateSpec | None              fixed-size per-request state it needs
   FeedForward.forward(ctx, h, residual)             adds its output into ``residual`` (float32)
   Block.forward(ctx, x, cache)                      one layer: arrangement of the four above
+  Part.replayable                                   class attribute: the part's launches may be replayed
+                                                    from a HIP graph (see Part)
 
 Optional, for steps of few rows (each part says by a class attribute whether it takes part):
   ``accepts_fused_norm``: forward(..., norm=) takes the un-normed residual and either the norm's
@@ -77,6 +79,16 @@ class LayerCache:
 
 
 class Part:
+    #: True if ``forward`` does nothing but launch kernels, on the current stream, that take every value that
+    #: changes from step to step (token ids, positions, cache rows, block tables, state slots) from the
+    #: context's device tensors, and no host value but the step's shape.  The same launches then serve any
+    #: later step of that shape, and the engine may replay a step of single tokens from a HIP graph.  A
+    #: part that reads the context's host lists, synchronises or allocates leaves this False.
+    replayable = False
+
+    def all_replayable(self) -> bool:
+        return self.replayable and all(c.all_replayable() for c in self.children().values())
+
     def tensor_specs(self) -> Dict[str, TensorSpec]:
         return {}
 

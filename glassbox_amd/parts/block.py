@@ -16,6 +16,8 @@ from .base import FeedForward, LayerCache, Mixer, Norm, Part
 
 
 class PreNormBlock(Part):
+    replayable = True
+
     def __init__(self, mixer_norm: Norm, mixer: Mixer, ffn_norm: Norm, ffn: FeedForward,
                  names=("input_layernorm", "self_attn", "post_attention_layernorm", "mlp")):
         self.mixer_norm, self.mixer, self.ffn_norm, self.ffn = mixer_norm, mixer, ffn_norm, ffn

@@ -12,6 +12,8 @@ from .base import Part, TensorSpec
 
 
 class Embedding(Part):
+    replayable = True
+
     def __init__(self, vocab: int, width: int):
         self.vocab, self.width = vocab, width
         self.table: Optional[torch.Tensor] = None
@@ -28,6 +30,7 @@ class Embedding(Part):
 
 class LMHead(Part):
     """logits = rows . W^T in float32.  ``tied_to`` names an Embedding whose table is the head."""
+    replayable = True
 
     def __init__(self, vocab: int, width: int, tied_to: Optional[Embedding] = None):
         self.vocab, self.width, self.tied_to = vocab, width, tied_to

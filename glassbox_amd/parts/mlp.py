@@ -11,6 +11,8 @@ from .base import FeedForward, PreNormed, TensorSpec, emit_target, split_workspa
 
 
 class SwiGLU(FeedForward):
+    replayable = True
+
     def __init__(self, width: int, intermediate: int):
         self.width, self.intermediate = width, intermediate
         self.w_gate_up: Optional[torch.Tensor] = None

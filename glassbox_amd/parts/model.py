@@ -27,6 +27,8 @@ class LayerCall:
 
 
 class DecoderModel(Part):
+    replayable = True
+
     def __init__(self, config, embedding: Embedding, blocks: Sequence[Part], schedule: Sequence[LayerCall],
                  final_norm: Norm, head: LMHead, names=("model.embed_tokens", "model.layers.{}", "model.norm", "lm_head"),
                  ignorable: Sequence[str] = ()):

@@ -11,6 +11,8 @@ from .base import Norm, TensorSpec
 
 
 class RMSNorm(Norm):
+    replayable = True
+
     def __init__(self, width: int, eps: float):
         self.width = width
         self.eps = float(eps)

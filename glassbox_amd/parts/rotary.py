@@ -17,6 +17,8 @@ from .base import PositionEncoding
 
 
 class Rotary(PositionEncoding):
+    replayable = True
+
     def __init__(self, head_dim: int, theta: float):
         if head_dim % 2:
             raise ValueError(f"rotary pairs need an even head size, got {head_dim}")
@@ -56,6 +58,7 @@ class Rotary(PositionEncoding):
 
 class NoPosition(PositionEncoding):
     """Keys and queries as they are; only the cache write."""
+    replayable = True
 
     def fuse_spec(self, ctx, head_dim: int):
         return (None, None)

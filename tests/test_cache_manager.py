@@ -246,3 +246,34 @@ def test_random_orders_keep_the_invariants(seed, groups):
     assert all(kv.used_pages(g) == 0 for g in range(len(specs))) and kv.free_state_slots() == 6
     kv.remove_seq(12345)   # giving back twice, or something unknown, changes nothing
     kv.check_invariants()
+
+
+def test_decode_rows_fills_the_callers_arrays():
+    """The bulk query that a replayed step uses agrees with the single queries."""
+    import numpy as np
+    cm = CacheManager(16, [GroupSpec(FULL, 0, 12), GroupSpec(WINDOW, 20, 12)], 4, False)
+    lens = {7: 37, 8: 5, 9: 16}
+    for sid, n in lens.items():
+        cm.add_seq(sid)
+        cm.reserve(sid, n)
+        cm.commit(sid, list(range(n)))
+        cm.reserve(sid, 1)
+    ids, stride, rows = [9, 7, 8], 4, 5
+    pos = np.full(rows, -7, np.int32)
+    state = np.full(rows, -7, np.int32)
+    slots = np.full((2, rows), -7, np.int32)
+    tables = np.full((2, rows, stride), -7, np.int32)
+    cm.decode_rows(ids, stride, pos.ctypes.data, state.ctypes.data, slots.ctypes.data, rows, tables.ctypes.data,
+                   rows * stride)
+    for i, sid in enumerate(ids):
+        assert pos[i] == lens[sid] and state[i] == cm.state_slot(sid)
+        for g in range(2):
+            t = cm.table(sid, g)
+            assert list(tables[g, i]) == t + [-1] * (stride - len(t))
+            assert slots[g, i] == cm.slot(sid, lens[sid], g)
+    assert (pos[3:] == -7).all() and (tables[:, 3:] == -7).all() and (slots[:, 3:] == -7).all()
+    with pytest.raises(CacheError):
+        cm.decode_rows(ids, 2, pos.ctypes.data, state.ctypes.data, slots.ctypes.data, rows, tables.ctypes.data, rows * 2)
+    with pytest.raises(CacheError):
+        cm.decode_rows([99], stride, pos.ctypes.data, state.ctypes.data, slots.ctypes.data, rows, tables.ctypes.data,
+                       rows * stride)

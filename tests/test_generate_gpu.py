@@ -253,3 +253,59 @@ def test_decode_loop_replays_graphs_like_plain_steps(model_dirs):
         eng.cache.check_invariants()
         assert eng.cache.used_pages() == 0
 
+
+
+@pytest.mark.parametrize("name,dtype", [("B", "bfloat16"), ("M", "bfloat16"), ("A", "float32")])
+def test_steps_of_single_tokens_replay_graphs_like_plain_steps(model_dirs, name, dtype):
+    """Engine.step replays steps of one token per request from HIP graphs.  The same steps through an engine
+    without graphs give the same logits: with the number of live requests changing (1, 2, 3 and 5 rows, so that
+    filler rows stand beside the live ones), prompts of other requests between the replays (their steps take the
+    general path and their buffers grow), a request ending and its pages going to the next, and a context that
+    crosses from one bucket of 1,024 tokens into the next."""
+    from glassbox_amd.engine import Engine
+    folder = model_dirs.get(name)
+    vocab = helpers.TINY[name]["vocab_size"]
+    long = 1015 if name == "M" else 50
+    lens = {"a": long, "b": 37, "c": 70 if name != "M" else 300, "d": 9, "e": 21, "f": 40}
+    prompts = {r: helpers.random_tokens(vocab, n, seed=60 + i) for i, (r, n) in enumerate(lens.items())}
+    engs = [Engine(folder, dtype=dtype, max_tokens=2048, max_seqs=8, graph_decode=g) for g in (True, False)]
+    assert engs[0].decode_graphs is not None and engs[1].decode_graphs is None
+    nxt = {r: 7 + i for i, r in enumerate(prompts)}
+    tol = 2e-5 if dtype == "float32" else 8e-3
+
+    def both(entries, what):
+        outs = [e.step(entries).float().cpu() for e in engs]
+        if outs[0].numel():
+            scale = max(1.0, float(outs[1].abs().max()))
+            err = float((outs[0] - outs[1]).abs().max())
+            assert err <= tol * scale, f"{what}: graphs and plain steps differ by {err:.3e} (largest logit {scale:.2f})"
+        return outs[1]
+
+    def decode(live, steps, what):
+        for s in range(steps):
+            logits = both([(r, [nxt[r]], [0]) for r in live], f"{what}, step {s}, requests {live}")
+            for r, row in zip(live, logits):
+                nxt[r] = int(row.argmax())
+
+    both([("a", prompts["a"], [])], "prompt a")
+    decode(["a"], 4, "one request")
+    both([("b", prompts["b"], [len(prompts["b"]) - 1])], "prompt b")
+    decode(["a", "b"], 5, "two requests")
+    both([("c", prompts["c"], []), ("a", [nxt["a"]], [0]), ("b", [nxt["b"]], [0])], "prompt c beside single tokens")
+    decode(["b", "c", "a"], 6, "three requests and a filler")
+    for e in engs:
+        e.end_request("b")
+    both([("d", prompts["d"], []), ("e", prompts["e"], [3])], "prompts d and e")
+    decode(["a", "c", "d", "e"], 3, "four requests")
+    both([("f", prompts["f"], [])], "prompt f")
+    decode(["f", "a", "c", "d", "e"], 7, "five requests and three fillers")
+    decode(["a"], 3, "one request again")
+    graphs = engs[0].decode_graphs
+    assert graphs.replays >= 12 and len({rows for rows, _ in graphs.shapes}) >= 4
+    if name == "M":
+        assert len({bucket for _, bucket in graphs.shapes}) == 2
+    for e in engs:
+        for r in ("a", "c", "d", "e", "f"):
+            e.end_request(r)
+        e.cache.check_invariants()
+        assert e.cache.used_pages() == 0
