@@ -58,6 +58,9 @@ def _host():
         lib.gbh_cache_decode_rows.restype = C.c_int
         lib.gbh_cache_decode_rows.argtypes = [C.c_void_p, C.POINTER(C.c_int64), C.c_int, C.c_int] + [C.c_void_p] * 2 + \
                                              [C.c_void_p, C.c_int, C.c_void_p, C.c_int]
+        lib.gbh_cache_step_rows.restype = C.c_int
+        lib.gbh_cache_step_rows.argtypes = [C.c_void_p, C.POINTER(C.c_int64), C.POINTER(C.c_int32), C.c_int, C.c_int] + \
+                                           [C.c_void_p] * 5 + [C.c_void_p, C.c_int, C.c_void_p, C.c_int]
         lib.gbh_chain_hash.restype = C.c_uint64
         lib.gbh_chain_hash.argtypes = [C.c_uint64, i32p, C.c_int]
         _lib = lib
@@ -175,6 +178,22 @@ class CacheManager:
         if rc:
             raise CacheError({-1: "unknown request", -2: f"a block table is longer than {stride} pages",
                               -3: "the page of a new token is not reserved"}.get(rc, f"error {rc}"))
+
+    def step_rows(self, seq_ids: Sequence[int], counts: Sequence[int], stride: int, positions_ptr: int, tok_seq_ptr: int,
+                  q_start_ptr: int, pos0_ptr: int, state_ptr: int, rows_ptr: int, rows_gap: int, tables_ptr: int,
+                  tables_gap: int) -> int:
+        """The metadata of a step in which request i brings ``counts[i]`` tokens, written into the caller's int32
+        arrays (addresses): per token its position, the index of its request and per group its cache row
+        ([group][token], ``rows_gap`` between groups); per request its first token's index, first position, state
+        slot and per group the block table padded to ``stride`` ([group][request][stride], ``tables_gap`` between
+        groups).  Returns 0, or the stride that is needed if ``stride`` is too small (nothing is written then)."""
+        ids = (C.c_int64 * max(1, len(seq_ids)))(*seq_ids)
+        cnt = (C.c_int32 * max(1, len(counts)))(*counts)
+        rc = self._lib.gbh_cache_step_rows(self._h, ids, cnt, len(seq_ids), stride, positions_ptr, tok_seq_ptr, q_start_ptr,
+                                           pos0_ptr, state_ptr, rows_ptr, rows_gap, tables_ptr, tables_gap)
+        if rc < 0:
+            raise CacheError({-1: "unknown request", -3: "a position of the step is not reserved"}.get(rc, f"error {rc}"))
+        return rc
 
     def slot(self, seq_id: int, pos: int, group: int = 0) -> int:
         """Row of (request, position) in a layer's pages (kv.rs:199-201)."""

@@ -302,6 +302,206 @@ int launch_tiled(const bf16* a, int lda, const bf16* w, int ldw, CT* c, int ldc,
   return launched("gemm_bf16 (tiled)");
 }
 
+// ------------------------------------------------------------------------- ring
+// Large products (many rows, many 256 x 256 tiles): a workgroup of 2 x 4 waves with a 256 x 256 tile, a wave
+// 4 x 2 tiles of 32 x 32.  The larger tile halves the operand bytes a flop needs, which is what bounds the
+// 128-wide kernel.  Operands go from memory straight into LDS (global_load_lds, 16 bytes a lane: a wave's
+// instruction fills 1 KB of LDS in lane order, so the lane decides which piece of memory lands where), in
+// k-steps of 32 through a ring of RING_STAGES buffers: nothing waits in registers, and a load has
+// RING_STAGES - 1 k-steps to arrive in.  A row of a k-step is 64 bytes = 4 pieces; piece c of row r lies at
+// position c ^ ((r >> 2) & 3), which spreads the 16-byte operand reads of a wave over all banks.
+//
+// The compiler knows nothing of what those loads write: before every LDS read it would wait for all of them.
+// So the operand reads are inline assembly, and the waits are written here by hand:
+//   * vmcnt before the barrier of k-step s: this wave's loads of stage s have landed (loads retire in order);
+//   * the barrier: every wave's have, and every wave has finished reading stage s - 1 (its reads were
+//     waited for before its last MFMAs), so the loads issued after it may overwrite that buffer;
+//   * lgkmcnt before the MFMAs that use an operand.
+constexpr int RBK = 32, RING_STAGES = 4;
+constexpr int RGM = 2, RGN = 4, RTM = 4, RTN = 2;          // waves along m, n; 32 x 32 tiles of a wave along m, n
+constexpr int RBM = RGM * RTM * 32, RBN = RGN * RTN * 32;  // 256 x 256
+constexpr int RLA = RBM / 16 / (RGM * RGN), RLW = RBN / 16 / (RGM * RGN), RLPS = RLA + RLW;  // loads of a wave per stage
+typedef __attribute__((address_space(3))) void lds_void;
+typedef __attribute__((address_space(1))) const void glb_void;
+
+__device__ __forceinline__ bf16x8 lds_read16(uint32_t addr) {
+  bf16x8 v;
+  asm volatile("ds_read_b128 %0, %1" : "=v"(v) : "v"(addr) : "memory");
+  return v;
+}
+// waits until at most LEFT LDS reads are outstanding; the operands named become usable
+template <int LEFT, int NA, int NB>
+__device__ __forceinline__ void lds_wait(bf16x8 (&fa)[NA], bf16x8 (&fb)[NB]) {
+  asm volatile("s_waitcnt lgkmcnt(%0)" ::"n"(LEFT) : "memory");
+#pragma unroll
+  for (int i = 0; i < NA; ++i) asm volatile("" : "+v"(fa[i]));
+#pragma unroll
+  for (int j = 0; j < NB; ++j) asm volatile("" : "+v"(fb[j]));
+}
+template <int LEFT> __device__ __forceinline__ void vm_wait() { __builtin_amdgcn_s_waitcnt(0x0F70 | LEFT); }
+
+template <int EPI, typename CT>
+__global__ __launch_bounds__(512, 1) void gemm_ring_kernel(const bf16* __restrict__ a, int lda, const bf16* __restrict__ w, int ldw,
+                                                           CT* __restrict__ c, int ldc, int M, int N, int K) {
+  __shared__ __attribute__((aligned(16))) bf16 As[RING_STAGES][RBM * RBK];
+  __shared__ __attribute__((aligned(16))) bf16 Ws[RING_STAGES][RBN * RBK];
+  const int tid = threadIdx.x, lane = tid % 64, wave = tid / 64;
+  const int wm = wave / RGN, wn = wave % RGN;
+  const int m0 = blockIdx.y * RBM;
+  const int half = N / 2;  // EPI_SILU_MUL: number of gate rows
+  // row of W behind row r of the workgroup's W tile (r = wn * 64 + j * 32 + column); with EPI_SILU_MUL a wave's
+  // first column tile holds gate rows and its second the up rows that belong to them
+  auto w_row = [&](int r) -> int {
+    if (EPI == EPI_SILU_MUL) {
+      const int n = blockIdx.x * (RBN / 2) + (r / 64) * 32 + r % 32;
+      return n < half ? ((r % 64) / 32 ? half + n : n) : 0;
+    }
+    return min(blockIdx.x * RBN + r, N - 1);
+  };
+  // a wave's load instruction moves 16 rows x 4 pieces; rows beyond M or N are read from a row that exists
+  const bf16* asrc[RLA];
+  const bf16* wsrc[RLW];
+#pragma unroll
+  for (int t = 0; t < RLA; ++t) {
+    const int row = (wave * RLA + t) * 16 + lane / 4, piece = (lane % 4) ^ ((row >> 2) & 3);
+    asrc[t] = a + (size_t)min(m0 + row, M - 1) * lda + piece * 8;
+  }
+#pragma unroll
+  for (int t = 0; t < RLW; ++t) {
+    const int row = (wave * RLW + t) * 16 + lane / 4, piece = (lane % 4) ^ ((row >> 2) & 3);
+    wsrc[t] = w + (size_t)w_row(row) * ldw + piece * 8;
+  }
+  auto load_a = [&](int t, int stage, int k0) {
+    __builtin_amdgcn_global_load_lds((glb_void*)(asrc[t] + k0), (lds_void*)&As[stage][(wave * RLA + t) * 16 * RBK], 16, 0, 0);
+  };
+  auto load_w = [&](int t, int stage, int k0) {
+    __builtin_amdgcn_global_load_lds((glb_void*)(wsrc[t] + k0), (lds_void*)&Ws[stage][(wave * RLW + t) * 16 * RBK], 16, 0, 0);
+  };
+  f32x16 acc[RTM][RTN];
+#pragma unroll
+  for (int i = 0; i < RTM; ++i)
+#pragma unroll
+    for (int j = 0; j < RTN; ++j)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
+
+  // operand of MFMA step ks (0, 1): row lane % 32 of a 32-row tile, piece 2 ks + lane / 32
+  uint32_t off[2];
+#pragma unroll
+  for (int ks = 0; ks < 2; ++ks) off[ks] = 2 * ((lane % 32) * RBK + (((2 * ks + lane / 32) ^ ((lane >> 2) & 3)) * 8));
+  const uint32_t abase = (uint32_t)(uintptr_t)(lds_void*)&As[0][0] + 2 * wm * RTM * 32 * RBK;
+  const uint32_t wbase = (uint32_t)(uintptr_t)(lds_void*)&Ws[0][0] + 2 * wn * RTN * 32 * RBK;
+  constexpr uint32_t A_STAGE = 2 * RBM * RBK, W_STAGE = 2 * RBN * RBK, TILE = 2 * 32 * RBK;
+
+  const int steps = K / RBK;
+  // k-step s: MORE = stage s + RING_STAGES - 1 exists and is requested during this step, one load after each
+  // row of MFMAs (requests and arithmetic side by side, not in bursts)
+  auto step = [&](int s, auto more) {
+    const int stage = s % RING_STAGES, nstage = (s + RING_STAGES - 1) % RING_STAGES, nk0 = (s + RING_STAGES - 1) * RBK;
+    const int ahead = steps - 1 - s;  // stages after s that are on their way
+    if (ahead >= RING_STAGES - 2)
+      vm_wait<(RING_STAGES - 2) * RLPS>();
+    else if (ahead == 1)
+      vm_wait<RLPS>();
+    else
+      vm_wait<0>();
+    __builtin_amdgcn_s_barrier();
+    bf16x8 fa[2][RTM], fw[2][RTN];
+#pragma unroll
+    for (int ks = 0; ks < 2; ++ks) {
+#pragma unroll
+      for (int i = 0; i < RTM; ++i) fa[ks][i] = lds_read16(abase + stage * A_STAGE + i * TILE + off[ks]);
+#pragma unroll
+      for (int j = 0; j < RTN; ++j) fw[ks][j] = lds_read16(wbase + stage * W_STAGE + j * TILE + off[ks]);
+    }
+#pragma unroll
+    for (int ks = 0; ks < 2; ++ks) {
+      if (ks == 0)
+        lds_wait<RTM + RTN>(fa[0], fw[0]);
+      else
+        lds_wait<0>(fa[1], fw[1]);
+#pragma unroll
+      for (int i = 0; i < RTM; ++i) {
+#pragma unroll
+        for (int j = 0; j < RTN; ++j)
+          acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa[ks][i], fw[ks][j], acc[i][j], 0, 0, 0);
+        if (decltype(more)::value) {
+          constexpr int SLOTS = 2 * RTM;
+          const int slot = ks * RTM + i;
+#pragma unroll
+          for (int t = 0; t < RLA; ++t)
+            if ((t * SLOTS) / RLPS == slot) load_a(t, nstage, nk0);
+#pragma unroll
+          for (int t = 0; t < RLW; ++t)
+            if (((RLA + t) * SLOTS) / RLPS == slot) load_w(t, nstage, nk0);
+        }
+        __builtin_amdgcn_sched_barrier(0);
+      }
+    }
+  };
+  using Yes = std::true_type;
+  using No = std::false_type;
+  static_assert(RING_STAGES == 4, "the tail below is written for four stages");
+#pragma unroll
+  for (int s = 0; s < RING_STAGES - 1; ++s)
+    if (s < steps) {
+#pragma unroll
+      for (int t = 0; t < RLA; ++t) load_a(t, s, s * RBK);
+#pragma unroll
+      for (int t = 0; t < RLW; ++t) load_w(t, s, s * RBK);
+    }
+  int s = 0;
+  for (; s + RING_STAGES - 1 < steps; ++s) step(s, Yes{});
+  for (; s < steps; ++s) step(s, No{});  // the last stages are on their way or have landed: nothing more is requested
+
+  // accumulator layout of a 32x32 tile: lane holds column lane%32, rows 8*(r/4) + 4*(lane/32) + r%4
+  if (EPI == EPI_SILU_MUL) {
+    const int gn = blockIdx.x * (RBN / 2) + wn * 32 + lane % 32;
+    if (gn >= half) return;
+#pragma unroll
+    for (int i = 0; i < RTM; ++i)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) {
+        const int gm = m0 + wm * RTM * 32 + i * 32 + 8 * (r / 4) + 4 * (lane / 32) + r % 4;
+        const float g = acc[i][0][r], u = acc[i][1][r];
+        if (gm < M) c[(size_t)gm * ldc + gn] = (CT)(g / (1.0f + __expf(-g)) * u);
+      }
+    return;
+  }
+#pragma unroll
+  for (int i = 0; i < RTM; ++i)
+#pragma unroll
+    for (int j = 0; j < RTN; ++j) {
+      const int gn = blockIdx.x * RBN + wn * RTN * 32 + j * 32 + lane % 32;
+      if (gn >= N) continue;
+#pragma unroll
+      for (int r = 0; r < 16; ++r) {
+        const int gm = m0 + wm * RTM * 32 + i * 32 + 8 * (r / 4) + 4 * (lane / 32) + r % 4;
+        if (gm < M) store_c<CT>(c + (size_t)gm * ldc + gn, acc[i][j][r], EPI == EPI_ACCUMULATE);
+      }
+    }
+}
+
+// The ring kernel pays where its tiles fill the chip about twice over (fewer leave compute units idle in the
+// last round) and the loads are whole 16-byte pieces.  GB_RING=0 switches it off (for measurements).
+inline bool ring_pays(int epi, const void* a, int lda, const void* w, int ldw, int M, int N, int K) {
+  static const bool on = [] { const char* e = getenv("GB_RING"); return !(e && e[0] == '0'); }();
+  if (!on || K % RBK != 0 || K < RBK * RING_STAGES || lda % 8 != 0 || ldw % 8 != 0 || (uintptr_t)a % 16 != 0 || (uintptr_t)w % 16 != 0)
+    return false;
+  const int cols = epi == EPI_SILU_MUL ? N / 2 : N, bn = epi == EPI_SILU_MUL ? RBN / 2 : RBN;
+  const long long tiles = (long long)((M + RBM - 1) / RBM) * ((cols + bn - 1) / bn);
+  return M >= 1024 && tiles >= 448;
+}
+
+template <int EPI, typename CT>
+int launch_ring(const bf16* a, int lda, const bf16* w, int ldw, CT* c, int ldc, int M, int N, int K, hipStream_t stream) {
+  const int cols = EPI == EPI_SILU_MUL ? N / 2 : N, bn = EPI == EPI_SILU_MUL ? RBN / 2 : RBN;
+  const dim3 grid((cols + bn - 1) / bn, (M + RBM - 1) / RBM), block(512);
+  GB_REQUIRE(grid.y <= 65535, "gemm_bf16: M=%d needs more than 65535 row tiles", M);
+  hipLaunchKernelGGL((gemm_ring_kernel<EPI, CT>), grid, block, 0, stream, a, lda, w, ldw, c, ldc, M, N, K);
+  return launched("gemm_bf16 (ring)");
+}
+
 // ------------------------------------------------------------------------ split k
 // A product with few tiles (17 to a few hundred rows, or few rows of W) leaves most compute units idle
 // and, as a skinny product, makes every workgroup read all of A.  Here the tiled kernel's workgroups
@@ -899,6 +1099,15 @@ extern "C" int gb_gemm_bf16(const void* a, int lda, const void* w, int ldw, void
 #undef GB_SK
   }
   const bf16* A = (const bf16*)a;
+  if (ring_pays(epilogue, a, lda, w, ldw, M, N, K) && (epilogue != EPI_SILU_MUL || N % 2 == 0)) {
+#define GB_RG(EPI, CT) return launch_ring<EPI, CT>(A, lda, W, ldw, (CT*)c, ldc, M, N, K, stream)
+    if (epilogue == EPI_ACCUMULATE) GB_RG(EPI_ACCUMULATE, float);
+    if (epilogue == EPI_SILU_MUL && c_dtype == kBF16) GB_RG(EPI_SILU_MUL, bf16);
+    if (epilogue == EPI_SILU_MUL) GB_RG(EPI_SILU_MUL, float);
+    if (c_dtype == kF32) GB_RG(EPI_STORE, float);
+    GB_RG(EPI_STORE, bf16);
+#undef GB_RG
+  }
 #define GB_TL(EPI, CT) return launch_tiled<EPI, CT>(A, lda, W, ldw, (CT*)c, ldc, M, N, K, stream)
   if (epilogue == EPI_ACCUMULATE) GB_TL(EPI_ACCUMULATE, float);
   if (epilogue == EPI_SILU_MUL && c_dtype == kBF16) GB_TL(EPI_SILU_MUL, bf16);

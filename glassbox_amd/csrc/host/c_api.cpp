@@ -1,5 +1,6 @@
 // C interface of the host runtime (cache manager, scheduler, sampler), loaded
 // from Python through ctypes.  Every object is an opaque handle.
+#include <algorithm>
 #include <cstring>
 #include <string>
 #include <vector>
@@ -73,6 +74,47 @@ int gbh_cache_decode_rows(void* h, const int64_t* ids, int n, int stride, int32_
       if (lp >= (int)t.size() || t[lp] < 0) return -3;
       rows[(size_t)g * rows_gap + i] = t[lp] * page + len % page;
     }
+  }
+  return 0;
+}
+// The same for a step of any mix: request i brings counts[i] tokens at positions len .. len + counts[i] - 1.
+// Per token (requests in the order given, their tokens in order): position, index of its request, and per group
+// the cache row ([group][token], rows_gap entries between groups).  Per request: first token's index, first
+// position, state slot, and per group the block table padded with -1 to `stride` entries.  Returns 0; -1 for an
+// unknown request; -3 if a position is not reserved; the stride that is needed if `stride` is too small.
+int gbh_cache_step_rows(void* h, const int64_t* ids, const int32_t* counts, int n, int stride, int32_t* positions,
+                        int32_t* tok_seq, int32_t* q_start, int32_t* pos0, int32_t* state_slot, int32_t* rows,
+                        int rows_gap, int32_t* tables, int tables_gap) {
+  auto* cm = (CacheManager*)h;
+  const int page = cm->page_size(), groups = cm->num_groups();
+  int need = 0;
+  for (int i = 0; i < n; ++i) {
+    if (cm->seq_len(ids[i]) < 0) return -1;
+    for (int g = 0; g < groups; ++g) need = std::max(need, (int)cm->table(ids[i], g)->size());
+  }
+  if (need > stride) return need;
+  int at = 0;
+  for (int i = 0; i < n; ++i) {
+    const int len = cm->seq_len(ids[i]);
+    q_start[i] = at;
+    pos0[i] = len;
+    state_slot[i] = cm->state_slot(ids[i]);
+    for (int j = 0; j < counts[i]; ++j) {
+      positions[at + j] = len + j;
+      tok_seq[at + j] = i;
+    }
+    for (int g = 0; g < groups; ++g) {
+      const std::vector<int32_t>& t = *cm->table(ids[i], g);
+      int32_t* out = tables + (size_t)g * tables_gap + (size_t)i * stride;
+      std::memcpy(out, t.data(), sizeof(int32_t) * t.size());
+      for (int j = (int)t.size(); j < stride; ++j) out[j] = -1;
+      for (int j = 0; j < counts[i]; ++j) {
+        const int p = len + j, lp = p / page;
+        if (lp >= (int)t.size() || t[lp] < 0) return -3;
+        rows[(size_t)g * rows_gap + at + j] = t[lp] * page + p % page;
+      }
+    }
+    at += counts[i];
   }
   return 0;
 }

@@ -55,7 +55,8 @@ class StepContext:
         self.slots, self.tables = slots, tables          # one entry per page group
         self.q_start, self.q_len, self.pos0, self.state_slots = q_start, q_len, pos0, state_slots
         self.want = want
-        #: the same metadata as Python lists, for kernel selection and for parts written in Python
+        #: per request, as Python lists: first row, rows, first position, state slot; and the step's shape
+        #: (n_decode, max_q_len, max_context): for kernel selection and for parts written in Python
         self.host = host
         self.attention_impl = attention_impl
         #: whether norms may be computed inside the next matrix product (steps of few rows); "plain" turns

@@ -213,75 +213,55 @@ class Engine:
 
     # ---------------------------------------------------------------- metadata
     def _build_context(self, entries) -> StepContext:
-        P = self.page_size
+        """The step's metadata: one pinned buffer, filled by the cache manager in one call, and one copy."""
+        P, G, S = self.page_size, len(self.group_keys), len(entries)
         # single-token requests first: the tuned attention kernels take the two kinds in two launches
-        order = sorted(range(len(entries)), key=lambda i: len(entries[i][1]) > 1)
-        S = len(entries)
-        G = len(self.group_keys)
-        token_ids: List[int] = []
-        positions: List[int] = []
-        tok_seq: List[int] = []
-        q_start, q_len, pos0, state_slots = [], [], [], []
-        tables_host: List[List[List[int]]] = [[] for _ in range(G)]
-        slots_host: List[List[int]] = [[] for _ in range(G)]
-        want_flat: List[Tuple[int, int, int]] = []   # (entry index, place, flat row)
+        order = sorted(range(S), key=lambda i: len(entries[i][1]) > 1)
+        sids = [entries[i][0] for i in order]
+        q_len = [len(entries[i][1]) for i in order]
+        n = sum(q_len)
+        pos0 = [self.cache.seq_len(sid) for sid in sids]
+        q_start, at = [], 0
+        for l in q_len:
+            q_start.append(at)
+            at += l
+        first_row = dict(zip(order, q_start))
+        # logits come out in the order of the wanted rows: that is the order of the entries
+        want_rows = [first_row[ei] + w for ei in range(S) for w in entries[ei][2]]
+        W = len(want_rows)
+        stride = max(1, max(-(-(p + l) // P) for p, l in zip(pos0, q_len)))
+        while True:
+            # token ids, positions, request of each token | first row, rows, first position, state slot of each
+            # request | wanted rows | cache rows [G][n] | block tables [G][S][stride]
+            total = 3 * n + 4 * S + W + G * n + G * S * stride
+            # a fresh pinned buffer per step: the host allocator hands it out again only after the copy ran
+            staged = torch.empty(total, dtype=torch.int32, pin_memory=True)
+            base, o_rows = staged.data_ptr(), 3 * n + 4 * S + W
+            at = lambda off: base + 4 * off
+            need = self.cache.step_rows(sids, q_len, stride, at(n), at(2 * n), at(3 * n), at(3 * n + 2 * S),
+                                        at(3 * n + 3 * S), at(o_rows), n, at(o_rows + G * n), S * stride)
+            if need == 0:
+                break
+            stride = need   # a request holds more pages than its tokens need
+        hv = staged.numpy()
+        tok = hv[:n]
         for s, ei in enumerate(order):
-            sid, tokens, want = entries[ei]
-            start = self.cache.seq_len(sid)
-            q_start.append(len(token_ids))
-            q_len.append(len(tokens))
-            pos0.append(start)
-            state_slots.append(self.cache.state_slot(sid))
-            for g in range(G):
-                table = self.cache.table(sid, g)
-                tables_host[g].append(table)
-                for j in range(len(tokens)):
-                    p = start + j
-                    slots_host[g].append(table[p // P] * P + p % P)
-            for k, w in enumerate(want):
-                want_flat.append((ei, k, len(token_ids) + w))
-            token_ids.extend(tokens)
-            positions.extend(range(start, start + len(tokens)))
-            tok_seq.extend([s] * len(tokens))
-        n = len(token_ids)
-        # logits come out in the order of the wanted rows: make that the order of the entries
-        want_flat.sort(key=lambda w: (w[0], w[1]))
-        want_rows = [w[2] for w in want_flat]
-        maxp = [max(1, max(len(t) for t in tables_host[g])) for g in range(G)]
-
-        pieces: List[List[int]] = [token_ids, positions, tok_seq, q_start, q_len, pos0, state_slots, want_rows]
-        for g in range(G):
-            pieces.append(slots_host[g])
-            flat: List[int] = []
-            for t in tables_host[g]:
-                flat.extend(t)
-                flat.extend([-1] * (maxp[g] - len(t)))
-            pieces.append(flat)
-        total = sum(len(p) for p in pieces)
+            tok[q_start[s]:q_start[s] + q_len[s]] = entries[ei][1]
+        hv[3 * n + S:3 * n + 2 * S] = q_len
+        hv[3 * n + 4 * S:o_rows] = want_rows
+        state_slots = hv[3 * n + 3 * S:3 * n + 4 * S].tolist()
         if self._meta_dev is None or self._meta_dev.numel() < total:
             self._meta_dev = torch.empty(max(total * 2, 4096), dtype=torch.int32, device=self.device)
-        flat_all: List[int] = []
-        for p in pieces:
-            flat_all.extend(p)
-        # a fresh pinned buffer per step: the host allocator hands it out again only after the copy ran
-        staged = torch.empty(total, dtype=torch.int32, pin_memory=True)
-        staged.copy_(torch.tensor(flat_all, dtype=torch.int32))
-        self._meta_dev[:total].copy_(staged, non_blocking=True)
-        views: List[torch.Tensor] = []
-        off = 0
-        for p in pieces:
-            views.append(self._meta_dev[off:off + len(p)])
-            off += len(p)
-        d_tok, d_pos, d_seq, d_qs, d_ql, d_p0, d_ss, d_want = views[:8]
-        slots = [views[8 + 2 * g] for g in range(G)]
-        tables = [views[9 + 2 * g].view(S, maxp[g]) for g in range(G)]
+        dev = self._meta_dev
+        dev[:total].copy_(staged, non_blocking=True)
+        cut = lambda off, count: dev[off:off + count]
+        slots = [cut(o_rows + g * n, n) for g in range(G)]
+        tables = [cut(o_rows + G * n + g * S * stride, S * stride).view(S, stride) for g in range(G)]
         n_decode = sum(1 for l in q_len if l == 1)
-        host = {"q_start": q_start, "q_len": q_len, "pos0": pos0, "state_slots": state_slots,
-                "positions": positions, "tok_seq": tok_seq, "token_ids": token_ids, "tables": tables_host,
-                "n_decode": n_decode, "max_q_len": max(q_len),
-                "max_context": max(p + l for p, l in zip(pos0, q_len)), "want_rows": want_rows}
-        ctx = StepContext(device=self.device, dtype=self.dtype, page_size=P, workspace=self.workspace, n=n,
-                          num_seqs=S, token_ids=d_tok, positions=d_pos, tok_seq=d_seq, slots=slots, tables=tables,
-                          q_start=d_qs, q_len=d_ql, pos0=d_p0, state_slots=d_ss, want=d_want, host=host,
-                          attention_impl=self.attention_impl)
-        return ctx
+        host = {"q_start": q_start, "q_len": q_len, "pos0": pos0, "state_slots": state_slots, "n_decode": n_decode,
+                "max_q_len": max(q_len), "max_context": max(p + l for p, l in zip(pos0, q_len))}
+        return StepContext(device=self.device, dtype=self.dtype, page_size=P, workspace=self.workspace, n=n,
+                           num_seqs=S, token_ids=cut(0, n), positions=cut(n, n), tok_seq=cut(2 * n, n), slots=slots,
+                           tables=tables, q_start=cut(3 * n, S), q_len=cut(3 * n + S, S), pos0=cut(3 * n + 2 * S, S),
+                           state_slots=cut(3 * n + 3 * S, S), want=cut(3 * n + 4 * S, W), host=host,
+                           attention_impl=self.attention_impl)

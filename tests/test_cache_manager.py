@@ -277,3 +277,42 @@ def test_decode_rows_fills_the_callers_arrays():
     with pytest.raises(CacheError):
         cm.decode_rows([99], stride, pos.ctypes.data, state.ctypes.data, slots.ctypes.data, rows, tables.ctypes.data,
                        rows * stride)
+
+
+def test_step_rows_fills_the_callers_arrays():
+    """The bulk query behind a step's metadata agrees with the single queries, for a mix of portions and single
+    tokens over a full and a windowed group."""
+    import numpy as np
+    cm = CacheManager(16, [GroupSpec(FULL, 0, 16), GroupSpec(WINDOW, 20, 16)], 4, False)
+    lens, counts = {7: 37, 8: 0, 9: 16}, {7: 1, 8: 21, 9: 3}
+    for sid, n in lens.items():
+        cm.add_seq(sid)
+        if n:
+            cm.reserve(sid, n)
+            cm.commit(sid, list(range(n)))
+        cm.reserve(sid, counts[sid])
+    ids = [9, 7, 8]
+    cnt = [counts[i] for i in ids]
+    n, S, stride = sum(cnt), 3, 3
+    i32 = lambda *shape: np.full(shape, -7, np.int32)
+    pos, seq, q_start, pos0, state = i32(n), i32(n), i32(S), i32(S), i32(S)
+    rows, tables = i32(2, n), i32(2, S, stride)
+    args = lambda st, tb: (ids, cnt, st, pos.ctypes.data, seq.ctypes.data, q_start.ctypes.data, pos0.ctypes.data,
+                           state.ctypes.data, rows.ctypes.data, n, tb.ctypes.data, S * st)
+    assert cm.step_rows(*args(2, tables)) == 3 and (pos == -7).all()        # too narrow: says what it needs, writes nothing
+    assert cm.step_rows(*args(stride, tables)) == 0
+    at = 0
+    for i, sid in enumerate(ids):
+        assert q_start[i] == at and pos0[i] == lens[sid] and state[i] == cm.state_slot(sid)
+        for j in range(cnt[i]):
+            assert pos[at + j] == lens[sid] + j and seq[at + j] == i
+            for g in range(2):
+                assert rows[g, at + j] == cm.slot(sid, lens[sid] + j, g)
+        for g in range(2):
+            t = cm.table(sid, g)
+            assert list(tables[g, i]) == t + [-1] * (stride - len(t))
+        at += cnt[i]
+    with pytest.raises(CacheError):
+        cm.step_rows([5], [1], stride, *args(stride, tables)[3:])
+    with pytest.raises(CacheError):   # two tokens where one is reserved
+        cm.step_rows([7], [18], stride + 1, *args(stride, i32(2, S, stride + 1))[3:-1], S * (stride + 1))

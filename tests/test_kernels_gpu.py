@@ -83,6 +83,37 @@ def test_gemm_bf16_fused_silu_mul(I, K, M):
     assert torch.equal(out2, out)
 
 
+@pytest.mark.parametrize("M,N,K", [(2100, 14000, 160), (1024, 28672, 128), (2048, 16384, 2048), (4000, 7200, 352),
+                                   (2049, 14080, 128 + 32)])
+@pytest.mark.parametrize("mode", ["bf16", "f32", "f32+", "silu"])
+def test_gemm_bf16_large_products_through_the_lds_ring(M, N, K, mode):
+    """Products of a thousand rows and more with some hundred 256 x 256 tiles take the kernel whose operands go
+    from memory straight into a ring of LDS buffers: rows and columns that do not fill the last tiles, k-steps
+    from the ring's depth upwards, every epilogue; twice in a row gives the same bits."""
+    from glassbox_amd import ops
+    a, w = rnd(M, K, seed=11).bfloat16(), rnd(N, K, seed=12).bfloat16()
+    if mode == "silu":
+        a, w = a * 0.25, w * 0.25
+    full = a.double() @ w.double().T
+    c0 = rnd(M, N, seed=13)
+    if mode == "silu":
+        g, u = full[:, :N // 2], full[:, N // 2:]
+        want = g / (1 + torch.exp(-g)) * u
+    else:
+        want = full + (c0.double() if mode == "f32+" else 0)
+    outs = []
+    for _ in range(2):
+        if mode == "silu":
+            c = torch.full((M, N // 2), 7.0, device=DEV, dtype=torch.bfloat16)
+        else:
+            c = to_dev(c0.clone(), torch.bfloat16 if mode == "bf16" else torch.float32)
+        ops.gemm(to_dev(a), to_dev(w), c, accumulate=(mode == "f32+"), silu_mul=(mode == "silu"))
+        outs.append(c)
+    tol = 1e-4 * math.sqrt(K) + (2 ** -8) * want.abs().max().item() * (mode in ("bf16", "silu"))
+    assert (outs[0].cpu().double() - want).abs().max().item() <= tol
+    assert torch.equal(outs[0], outs[1])
+
+
 @pytest.mark.parametrize("N,K,M,silu", [(96, 64, 1, False), (6144, 2048, 8, False), (352, 176, 5, True),
                                         (16384, 2048, 8, True), (480, 80, 33, False), (512, 4104, 64, True)])
 @pytest.mark.parametrize("gamma_dtype", [torch.float32, torch.bfloat16])
