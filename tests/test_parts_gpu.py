@@ -1,7 +1,8 @@
 """Each part alone against its plain formula, and what the composition allows: a toy architecture
 defined here (a mixer with state of its own, windowed and full attention in different layers, a
 layer named twice, a layer that reads another layer's cache) is registered, built, loaded and
-stepped without a change to the package's files.  The toy stands for no real model."""
+stepped without a change to the package's files; a second toy has a feed-forward that routes rows to
+experts and a position encoding with a table of its own.  The toys stand for no real model."""
 import math
 from dataclasses import dataclass
 from typing import Dict
@@ -246,3 +247,153 @@ def test_toy_architecture_registers_builds_and_steps(tmp_path, dtype):
     eng.step([("w", requests["t2"], [])])
     sid = eng._ids["w"]
     assert eng.cache.table(sid, 1)[:3] == [-1, -1, -1] and all(p >= 0 for p in eng.cache.table(sid, 0))
+
+
+# ------------------------------------------------- a second toy: routing and learned positions
+def register_routed_toy():
+    """A feed-forward that routes each row to one of a few experts and a position encoding with a table of its
+    own, both defined here with tensor operations (toys, not kernels)."""
+    from glassbox_amd import ops
+    from glassbox_amd.config import LlamaConfig, register_architecture
+    from glassbox_amd.parts.attention import PagedAttention
+    from glassbox_amd.parts.base import FeedForward, PositionEncoding, TensorSpec
+    from glassbox_amd.parts.block import PreNormBlock
+    from glassbox_amd.parts.embedding import Embedding, LMHead
+    from glassbox_amd.parts.mlp import SwiGLU
+    from glassbox_amd.parts.model import DecoderModel, LayerCall
+    from glassbox_amd.parts.norm import RMSNorm
+    from glassbox_amd.parts.rotary import Rotary
+
+    @dataclass(frozen=True)
+    class RoutedConfig(LlamaConfig):
+        architecture = "ToyRoutedForCausalLM"
+        num_experts: int = 3
+        expert_size: int = 40
+
+    class RoutedFFN(FeedForward):
+        """Each row goes to the expert with the largest router logit; the expert's output is weighted with that
+        logit's softmax probability.  Router logits and probabilities in 32-bit."""
+
+        def __init__(self, width, experts, size):
+            self.width, self.experts, self.size = width, experts, size
+
+        def tensor_specs(self) -> Dict[str, TensorSpec]:
+            specs = {"router.weight": TensorSpec((self.experts, self.width), kind="f32")}
+            for e in range(self.experts):
+                specs[f"experts.{e}.gate.weight"] = TensorSpec((self.size, self.width))
+                specs[f"experts.{e}.up.weight"] = TensorSpec((self.size, self.width))
+                specs[f"experts.{e}.down.weight"] = TensorSpec((self.width, self.size))
+            return specs
+
+        def load(self, tensors):
+            self.t = {k: v.float() for k, v in tensors.items()}
+
+        def forward(self, ctx, h, residual):
+            h = h.float()
+            prob = torch.softmax(h @ self.t["router.weight"].T, dim=-1)
+            top, choice = prob.max(dim=-1)
+            for e in range(self.experts):
+                rows = (choice == e).nonzero().flatten()
+                if rows.numel():
+                    x = h[rows]
+                    g, u = x @ self.t[f"experts.{e}.gate.weight"].T, x @ self.t[f"experts.{e}.up.weight"].T
+                    y = (g / (1 + torch.exp(-g)) * u) @ self.t[f"experts.{e}.down.weight"].T
+                    residual[rows] += top[rows, None] * y
+
+    class LearnedPosition(PositionEncoding):
+        """A table row per position is added to every query and key head; then the cache write."""
+
+        def __init__(self, head_dim, positions):
+            self.head_dim, self.positions = head_dim, positions
+
+        def tensor_specs(self) -> Dict[str, TensorSpec]:
+            return {"position_table": TensorSpec((self.positions, self.head_dim), kind="f32")}
+
+        def load(self, tensors):
+            self.table = tensors["position_table"]
+
+        def apply_and_store(self, ctx, qkv, n_heads, n_kv_heads, head_dim, slots, k_pages, v_pages):
+            rows = self.table[ctx.positions.long()]
+            heads = qkv.view(qkv.shape[0], -1, head_dim)
+            moved = n_heads + (n_kv_heads if slots is not None else 0)
+            heads[:, :moved] = (heads[:, :moved].float() + rows[:, None, :]).to(qkv.dtype)
+            if slots is not None:
+                ops.rope_store(qkv, None, None, slots, k_pages, v_pages, n_heads, n_kv_heads, head_dim, rotate=False,
+                               portions=ctx.portions())
+
+    def build(cfg):
+        d, hd = cfg.hidden_size, cfg.head_size
+        norm = lambda: RMSNorm(d, cfg.rms_norm_eps)
+        attn = lambda pos: PagedAttention(d, cfg.num_attention_heads, cfg.num_key_value_heads, hd, position=pos)
+        blocks = [
+            PreNormBlock(norm(), attn(LearnedPosition(hd, cfg.max_position_embeddings)), norm(),
+                         RoutedFFN(d, cfg.num_experts, cfg.expert_size)),
+            PreNormBlock(norm(), attn(Rotary(hd, cfg.rope_theta)), norm(), SwiGLU(d, cfg.intermediate_size)),
+            PreNormBlock(norm(), attn(Rotary(hd, cfg.rope_theta)), norm(), RoutedFFN(d, cfg.num_experts, cfg.expert_size)),
+        ]
+        emb = Embedding(cfg.vocab_size, d)
+        return DecoderModel(cfg, emb, blocks, [LayerCall(i, cache=i) for i in range(3)], norm(),
+                            LMHead(cfg.vocab_size, d, tied_to=emb))
+
+    register_architecture("ToyRoutedForCausalLM", RoutedConfig, build)
+
+
+def routed_plain(w, cfg, tokens):
+    d, nh, nkv, hd = cfg["hidden_size"], cfg["num_attention_heads"], cfg["num_key_value_heads"], cfg["head_dim"]
+    eps, theta, T = cfg["rms_norm_eps"], cfg["rope_theta"], len(tokens)
+    W = {k: v.double() for k, v in w.items()}
+    x = W["model.embed_tokens.weight"][torch.tensor(tokens)]
+    for i in range(3):
+        p = f"model.layers.{i}."
+        h = plain.rms_norm(x, W[p + "input_layernorm.weight"], eps)
+        q = (h @ W[p + "self_attn.q_proj.weight"].T).reshape(T, nh, hd)
+        k = (h @ W[p + "self_attn.k_proj.weight"].T).reshape(T, nkv, hd)
+        v = (h @ W[p + "self_attn.v_proj.weight"].T).reshape(T, nkv, hd)
+        if i == 0:
+            table = W[p + "self_attn.position_table"][:T]
+            q, k = q + table[:, None, :], k + table[:, None, :]
+        else:
+            q, k = plain.rope(q, list(range(T)), theta), plain.rope(k, list(range(T)), theta)
+        x = x + plain.attention(q, k, v, 0).reshape(T, nh * hd) @ W[p + "self_attn.o_proj.weight"].T
+        h = plain.rms_norm(x, W[p + "post_attention_layernorm.weight"], eps)
+        if i == 1:
+            x = x + plain.swiglu(h, W[p + "mlp.gate_proj.weight"], W[p + "mlp.up_proj.weight"], W[p + "mlp.down_proj.weight"])
+            continue
+        prob = torch.softmax(h @ W[p + "mlp.router.weight"].T, dim=-1)
+        out = torch.zeros_like(x)
+        for t in range(T):
+            e = int(prob[t].argmax())
+            out[t] = prob[t, e] * plain.swiglu(h[t:t + 1], W[p + f"mlp.experts.{e}.gate.weight"],
+                                               W[p + f"mlp.experts.{e}.up.weight"], W[p + f"mlp.experts.{e}.down.weight"])[0]
+        x = x + out
+    return plain.rms_norm(x, W["model.norm.weight"], eps) @ W["model.embed_tokens.weight"].T
+
+
+def test_toy_with_routing_and_learned_positions(tmp_path):
+    """A feed-forward with routing and a position encoding with a table of its own are parts like any other:
+    declared, loaded by name, chosen layer by layer.  In 32-bit, where a row's expert is the same here and in the
+    plain formulas; whole, in portions, and mixed with few pages."""
+    from glassbox_amd import Engine
+    from glassbox_amd.config import config_from_dict
+    from glassbox_amd.weights import write_random_model
+    register_routed_toy()
+    raw = dict(architectures=["ToyRoutedForCausalLM"], hidden_size=48, intermediate_size=80, num_hidden_layers=3,
+               num_attention_heads=3, num_key_value_heads=1, head_dim=16, vocab_size=89, rope_theta=7000.0,
+               rms_norm_eps=1e-6, tie_word_embeddings=True, max_position_embeddings=128, num_experts=3, expert_size=40)
+    folder = write_random_model(config_from_dict(raw), str(tmp_path / "routed"), seed=5, norm_init="uniform", std=0.08)
+    w = plain.read_safetensors(folder + "/model.safetensors")
+    assert w["model.layers.0.self_attn.position_table"].shape == (128, 16)
+    assert w["model.layers.2.mlp.experts.2.down.weight"].shape == (48, 40) and "model.layers.1.mlp.router.weight" not in w
+    requests = {f"r{i}": helpers.random_tokens(89, n, seed=20 + i) for i, n in enumerate((44, 19, 61, 8))}
+    want = {r: routed_plain(w, raw, t).numpy() for r, t in requests.items()}
+    steps_mixed, peak = helpers.schedule_mixed(requests, seed=4, live=3, tail=6)
+    for steps, pool in ((helpers.schedule_whole(requests), 512), (helpers.schedule_chunks(requests, sizes=(7, 2, 11, 3)), 512),
+                        (steps_mixed, peak)):
+        eng = Engine(folder, dtype="float32", max_tokens=pool, max_seqs=3)
+        assert eng.decode_graphs is None
+        got = helpers.replay(eng, steps)
+        for r in requests:
+            bad = helpers.first_bad(got[r], want[r], 1e-4)
+            assert bad is None, f"{r}: first wrong position {bad}"
+        eng.cache.check_invariants()
+        assert eng.cache.used_pages(0) == 0
