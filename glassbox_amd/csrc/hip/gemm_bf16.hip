@@ -313,10 +313,11 @@ int launch_tiled(const bf16* a, int lda, const bf16* w, int ldw, CT* c, int ldc,
 //
 // The compiler knows nothing of what those loads write: before every LDS read it would wait for all of them.
 // So the operand reads are inline assembly, and the waits are written here by hand:
-//   * vmcnt before the barrier of k-step s: this wave's loads of stage s have landed (loads retire in order);
-//   * the barrier: every wave's have, and every wave has finished reading stage s - 1 (its reads were
-//     waited for before its last MFMAs), so the loads issued after it may overwrite that buffer;
-//   * lgkmcnt before the MFMAs that use an operand.
+//   * lgkmcnt before the MFMAs that use an operand;
+//   * the barrier of k-step s stands between its two MFMA steps.  Before it a wave waits for its last operand
+//     reads of stage s (lgkmcnt) and for its own loads of stage s + 1 (vmcnt: loads retire in order).  After
+//     it, every wave's loads of stage s + 1 have landed, so its operands may be read (they arrive under the
+//     second MFMA step), and every wave is done with stage s, so the loads of k-step s + 1 may overwrite it.
 constexpr int RBK = 32, RING_STAGES = 4;
 constexpr int RGM = 2, RGN = 4, RTM = 4, RTN = 2;          // waves along m, n; 32 x 32 tiles of a wave along m, n
 constexpr int RBM = RGM * RTM * 32, RBN = RGN * RTN * 32;  // 256 x 256
@@ -342,7 +343,14 @@ template <int LEFT> __device__ __forceinline__ void vm_wait() { __builtin_amdgcn
 
 template <int EPI, typename CT>
 __global__ __launch_bounds__(512, 1) void gemm_ring_kernel(const bf16* __restrict__ a, int lda, const bf16* __restrict__ w, int ldw,
-                                                           CT* __restrict__ c, int ldc, int M, int N, int K) {
+                                                           CT* __restrict__ c, int ldc, int M, int N, int K, int k_slice) {
+  if (k_slice > 0) {  // split k: workgroup z of a tile sums its own slice of k into its own copy of C
+    const int z = blockIdx.z;
+    a += (size_t)z * k_slice;
+    w += (size_t)z * k_slice;
+    c += (size_t)z * M * ldc;
+    K = min(k_slice, K - z * k_slice);
+  }
   __shared__ __attribute__((aligned(16))) bf16 As[RING_STAGES][RBM * RBK];
   __shared__ __attribute__((aligned(16))) bf16 Ws[RING_STAGES][RBN * RBK];
   const int tid = threadIdx.x, lane = tid % 64, wave = tid / 64;
@@ -394,54 +402,60 @@ __global__ __launch_bounds__(512, 1) void gemm_ring_kernel(const bf16* __restric
   constexpr uint32_t A_STAGE = 2 * RBM * RBK, W_STAGE = 2 * RBN * RBK, TILE = 2 * 32 * RBK;
 
   const int steps = K / RBK;
-  // k-step s: MORE = stage s + RING_STAGES - 1 exists and is requested during this step, one load after each
-  // row of MFMAs (requests and arithmetic side by side, not in bursts)
+  bf16x8 fa[2][RTM], fw[2][RTN];
+  auto read_operands = [&](int stage, int ks) {
+#pragma unroll
+    for (int i = 0; i < RTM; ++i) fa[ks][i] = lds_read16(abase + stage * A_STAGE + i * TILE + off[ks]);
+#pragma unroll
+    for (int j = 0; j < RTN; ++j) fw[ks][j] = lds_read16(wbase + stage * W_STAGE + j * TILE + off[ks]);
+  };
+  // the MFMAs of MFMA step ks; with MORE, half of the loads of stage s + RING_STAGES - 1 are requested among them,
+  // one after a row of MFMAs (requests and arithmetic side by side, not in bursts)
+  auto multiply = [&](int ks, auto more, int nstage, int nk0) {
+#pragma unroll
+    for (int i = 0; i < RTM; ++i) {
+#pragma unroll
+      for (int j = 0; j < RTN; ++j)
+        acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa[ks][i], fw[ks][j], acc[i][j], 0, 0, 0);
+      if (decltype(more)::value) {
+        constexpr int SLOTS = 2 * RTM;
+        const int slot = ks * RTM + i;
+#pragma unroll
+        for (int t = 0; t < RLA; ++t)
+          if ((t * SLOTS) / RLPS == slot) load_a(t, nstage, nk0);
+#pragma unroll
+        for (int t = 0; t < RLW; ++t)
+          if (((RLA + t) * SLOTS) / RLPS == slot) load_w(t, nstage, nk0);
+      }
+      __builtin_amdgcn_sched_barrier(0);
+    }
+  };
+  // k-step s.  On entry the operands of its first MFMA step are on their way into registers.  The barrier stands
+  // between the two MFMA steps: by then this wave has read all it needs of stage s, and once every wave has,
+  // stage s + 1 (whose loads were waited for) may be read and the buffer of stage s overwritten (by the loads of
+  // k-step s + 1).  So the first operands of k-step s + 1 arrive under the second MFMA step of k-step s.
+  static_assert(RLPS == 4 && RING_STAGES == 4, "the wait counts below are written for four loads a stage, four stages");
   auto step = [&](int s, auto more) {
     const int stage = s % RING_STAGES, nstage = (s + RING_STAGES - 1) % RING_STAGES, nk0 = (s + RING_STAGES - 1) * RBK;
-    const int ahead = steps - 1 - s;  // stages after s that are on their way
-    if (ahead >= RING_STAGES - 2)
-      vm_wait<(RING_STAGES - 2) * RLPS>();
-    else if (ahead == 1)
-      vm_wait<RLPS>();
-    else
-      vm_wait<0>();
-    __builtin_amdgcn_s_barrier();
-    bf16x8 fa[2][RTM], fw[2][RTN];
-#pragma unroll
-    for (int ks = 0; ks < 2; ++ks) {
-#pragma unroll
-      for (int i = 0; i < RTM; ++i) fa[ks][i] = lds_read16(abase + stage * A_STAGE + i * TILE + off[ks]);
-#pragma unroll
-      for (int j = 0; j < RTN; ++j) fw[ks][j] = lds_read16(wbase + stage * W_STAGE + j * TILE + off[ks]);
-    }
-#pragma unroll
-    for (int ks = 0; ks < 2; ++ks) {
-      if (ks == 0)
-        lds_wait<RTM + RTN>(fa[0], fw[0]);
+    read_operands(stage, 1);
+    lds_wait<RTM + RTN>(fa[0], fw[0]);
+    multiply(0, more, nstage, nk0);
+    lds_wait<0>(fa[1], fw[1]);
+    if (s + 1 < steps) {
+      // loads of this wave that may still be on their way: those of stage s + 2, and the half of stage s + 3 just asked for
+      if (decltype(more)::value)
+        vm_wait<RLPS + RLPS / 2>();
+      else if (s + 2 < steps)
+        vm_wait<RLPS>();
       else
-        lds_wait<0>(fa[1], fw[1]);
-#pragma unroll
-      for (int i = 0; i < RTM; ++i) {
-#pragma unroll
-        for (int j = 0; j < RTN; ++j)
-          acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa[ks][i], fw[ks][j], acc[i][j], 0, 0, 0);
-        if (decltype(more)::value) {
-          constexpr int SLOTS = 2 * RTM;
-          const int slot = ks * RTM + i;
-#pragma unroll
-          for (int t = 0; t < RLA; ++t)
-            if ((t * SLOTS) / RLPS == slot) load_a(t, nstage, nk0);
-#pragma unroll
-          for (int t = 0; t < RLW; ++t)
-            if (((RLA + t) * SLOTS) / RLPS == slot) load_w(t, nstage, nk0);
-        }
-        __builtin_amdgcn_sched_barrier(0);
-      }
+        vm_wait<0>();
+      __builtin_amdgcn_s_barrier();
+      read_operands((s + 1) % RING_STAGES, 0);
     }
+    multiply(1, more, nstage, nk0);
   };
   using Yes = std::true_type;
   using No = std::false_type;
-  static_assert(RING_STAGES == 4, "the tail below is written for four stages");
 #pragma unroll
   for (int s = 0; s < RING_STAGES - 1; ++s)
     if (s < steps) {
@@ -450,6 +464,14 @@ __global__ __launch_bounds__(512, 1) void gemm_ring_kernel(const bf16* __restric
 #pragma unroll
       for (int t = 0; t < RLW; ++t) load_w(t, s, s * RBK);
     }
+  if (steps >= 3)
+    vm_wait<2 * RLPS>();
+  else if (steps == 2)
+    vm_wait<RLPS>();
+  else
+    vm_wait<0>();
+  __builtin_amdgcn_s_barrier();
+  read_operands(0, 0);
   int s = 0;
   for (; s + RING_STAGES - 1 < steps; ++s) step(s, Yes{});
   for (; s < steps; ++s) step(s, No{});  // the last stages are on their way or have landed: nothing more is requested
@@ -482,15 +504,21 @@ __global__ __launch_bounds__(512, 1) void gemm_ring_kernel(const bf16* __restric
     }
 }
 
-// The ring kernel pays where its tiles fill the chip about twice over (fewer leave compute units idle in the
-// last round) and the loads are whole 16-byte pieces.  GB_RING=0 switches it off (for measurements).
-inline bool ring_pays(int epi, const void* a, int lda, const void* w, int ldw, int M, int N, int K) {
+// The ring kernel pays where its tiles occupy at least three quarters of the compute units and the loads are whole
+// 16-byte pieces.  GB_RING=0 switches it off (for measurements).
+inline bool ring_on() {
   static const bool on = [] { const char* e = getenv("GB_RING"); return !(e && e[0] == '0'); }();
-  if (!on || K % RBK != 0 || K < RBK * RING_STAGES || lda % 8 != 0 || ldw % 8 != 0 || (uintptr_t)a % 16 != 0 || (uintptr_t)w % 16 != 0)
-    return false;
+  return on;
+}
+inline bool ring_takes(const void* a, int lda, const void* w, int ldw, int K) {
+  return ring_on() && K % RBK == 0 && K >= RBK * RING_STAGES && lda % 8 == 0 && ldw % 8 == 0 && (uintptr_t)a % 16 == 0 &&
+         (uintptr_t)w % 16 == 0;
+}
+inline bool ring_pays(int epi, const void* a, int lda, const void* w, int ldw, int M, int N, int K) {
+  if (!ring_takes(a, lda, w, ldw, K)) return false;
   const int cols = epi == EPI_SILU_MUL ? N / 2 : N, bn = epi == EPI_SILU_MUL ? RBN / 2 : RBN;
   const long long tiles = (long long)((M + RBM - 1) / RBM) * ((cols + bn - 1) / bn);
-  return M >= 1024 && tiles >= 448;
+  return M >= 1024 && tiles >= 192;
 }
 
 template <int EPI, typename CT>
@@ -498,7 +526,7 @@ int launch_ring(const bf16* a, int lda, const bf16* w, int ldw, CT* c, int ldc, 
   const int cols = EPI == EPI_SILU_MUL ? N / 2 : N, bn = EPI == EPI_SILU_MUL ? RBN / 2 : RBN;
   const dim3 grid((cols + bn - 1) / bn, (M + RBM - 1) / RBM), block(512);
   GB_REQUIRE(grid.y <= 65535, "gemm_bf16: M=%d needs more than 65535 row tiles", M);
-  hipLaunchKernelGGL((gemm_ring_kernel<EPI, CT>), grid, block, 0, stream, a, lda, w, ldw, c, ldc, M, N, K);
+  hipLaunchKernelGGL((gemm_ring_kernel<EPI, CT>), grid, block, 0, stream, a, lda, w, ldw, c, ldc, M, N, K, 0);
   return launched("gemm_bf16 (ring)");
 }
 
@@ -506,14 +534,33 @@ int launch_ring(const bf16* a, int lda, const bf16* w, int ldw, CT* c, int ldc, 
 // A product with few tiles (17 to a few hundred rows, or few rows of W) leaves most compute units idle
 // and, as a skinny product, makes every workgroup read all of A.  Here the tiled kernel's workgroups
 // also divide k: workgroup (tile, z) sums slice z of k into copy z of a float32 C in a workspace, and a
-// second kernel adds the copies in the order of z and applies the epilogue.  Tiles of 64 or 128 rows.
+// second kernel adds the copies in the order of z and applies the epilogue.  Tiles of 64 or 128 rows; with
+// a thousand rows and more and a long k, the ring kernel's tiles of 256.
 struct SplitPlan {
   int bm, slices, k_slice;
   size_t floats;  // of workspace
+  bool ring;      // the ring kernel's 256 x 256 tiles, if the operands allow (else the tiled kernel's, same slices)
 };
 
 inline SplitPlan split_plan(int M, int N, int K) {
-  SplitPlan p{M <= 64 ? 64 : 128, 1, 0, 0};
+  SplitPlan p{M <= 64 ? 64 : 128, 1, 0, 0, false};
+  // many rows, a long k and few 256 x 256 tiles (the down projection of a prompt portion): slices of k fill the
+  // chip with the ring kernel's tiles once; a slice keeps 1,024 of k or more
+  if (ring_on() && M >= 1024 && K >= 4096 && K % TBK == 0 && N % 8 == 0) {
+    const int tiles = ((M + RBM - 1) / RBM) * ((N + RBN - 1) / RBN);
+    int want = tiles < 192 ? 256 / tiles : 1;
+    if (want > K / 1024) want = K / 1024;
+    if (want >= 2) {
+      p.k_slice = ((K + want - 1) / want + TBK - 1) / TBK * TBK;
+      p.slices = (K + p.k_slice - 1) / p.k_slice;
+      if (p.slices >= 2 && K - (p.slices - 1) * p.k_slice >= RBK * RING_STAGES) {
+        p.floats = (size_t)p.slices * M * N;
+        p.ring = true;
+        return p;
+      }
+      p.slices = 1, p.k_slice = 0;
+    }
+  }
   const int tiles = ((N + 127) / 128) * ((M + p.bm - 1) / p.bm);
   if (tiles >= 192 || N % 8 != 0) return p;
   // measured on SmolLM2-1.7B shapes: a long k (the down projection) always gains; a short one only where
@@ -526,7 +573,7 @@ inline SplitPlan split_plan(int M, int N, int K) {
   if (want < 2) return p;
   p.k_slice = ((K + want - 1) / want + TBK - 1) / TBK * TBK;
   p.slices = (K + p.k_slice - 1) / p.k_slice;
-  if (p.slices < 2) return SplitPlan{p.bm, 1, 0, 0};
+  if (p.slices < 2) return SplitPlan{p.bm, 1, 0, 0, false};
   p.floats = (size_t)p.slices * M * N;
   return p;
 }
@@ -558,8 +605,12 @@ int launch_split(const bf16* a, int lda, const bf16* w, int ldw, CT* c, int ldc,
                  const SplitPlan& plan, hipStream_t stream) {
   const dim3 grid((N + 127) / 128, (M + plan.bm - 1) / plan.bm, plan.slices), block(256);
   const bool kfull = K % TBK == 0;
+  const bool ring = plan.ring && ring_takes(a, lda, w, ldw, K);
+  if (ring)
+    hipLaunchKernelGGL((gemm_ring_kernel<EPI_STORE, float>), dim3((N + RBN - 1) / RBN, (M + RBM - 1) / RBM, plan.slices), dim3(512),
+                       0, stream, a, lda, w, ldw, ws, N, M, N, K, plan.k_slice);
 #define GB_S(WM, FULL)                                                                                                   \
-  if ((plan.bm == 64 * WM) && kfull == FULL)                                                                             \
+  if (!ring && (plan.bm == 64 * WM) && kfull == FULL)                                                                    \
     hipLaunchKernelGGL((gemm_tiled_kernel<WM, 2, 1, EPI_STORE, FULL, float>), grid, block, 0, stream, a, lda, w, ldw, ws, \
                        N, M, N, K, plan.k_slice);
   GB_S(1, true) GB_S(1, false) GB_S(2, true) GB_S(2, false)

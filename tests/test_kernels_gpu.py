@@ -84,7 +84,7 @@ def test_gemm_bf16_fused_silu_mul(I, K, M):
 
 
 @pytest.mark.parametrize("M,N,K", [(2100, 14000, 160), (1024, 28672, 128), (2048, 16384, 2048), (4000, 7200, 352),
-                                   (2049, 14080, 128 + 32)])
+                                   (2049, 14080, 128 + 32), (2048, 6144, 128)])
 @pytest.mark.parametrize("mode", ["bf16", "f32", "f32+", "silu"])
 def test_gemm_bf16_large_products_through_the_lds_ring(M, N, K, mode):
     """Products of a thousand rows and more with some hundred 256 x 256 tiles take the kernel whose operands go
@@ -186,7 +186,9 @@ def test_gemm_bf16_prepares_the_next_norm(M, N, K, N2, silu, gamma_dtype):
 
 
 @pytest.mark.parametrize("M,N,K", [(17, 96, 4096), (33, 2048, 2048), (64, 2048, 8192), (64, 6144, 2048), (100, 2048, 4160),
-                                   (200, 528, 8200), (64, 16384, 2048), (40, 1008, 4104), (512, 2048, 8192)])
+                                   (200, 528, 8200), (64, 16384, 2048), (40, 1008, 4104), (512, 2048, 8192),
+                                   # a thousand rows and more: slices of k through the 256 x 256 tiles
+                                   (2048, 2048, 8192), (1100, 1008, 4160), (1024, 528, 5120)])
 @pytest.mark.parametrize("mode", ["bf16", "f32", "f32+", "silu"])
 def test_gemm_bf16_divides_k_over_workgroups(M, N, K, mode):
     """With a workspace, a product of few tiles has several workgroups a tile, each over a slice of k,
