@@ -3,10 +3,12 @@
 // (crates/glassbox-core/src/kernels.rs:381,586).  Both operands are contiguous along k, which
 // is the layout MFMA operands want: every lane loads 8 consecutive k as one 16-byte word.
 //
-// Three kernels:
+// Four kernels:
 //  * tiled  (M > 64, prompt portions): a workgroup of 2x2 waves, each wave a block of 2x2 or 2x1
 //    v_mfma_f32_32x32x16_bf16 tiles (workgroup tile 128x128 or 128x64), operands staged through LDS in
 //    k-steps of 64 with two buffers; the SiLU-multiply of stacked gate/up rows can be its epilogue.
+//  * ring   (a thousand rows and more, enough 256x256 tiles to fill the chip): 2x4 waves, a wave 4x2 such
+//    tiles; operands go from memory straight into a ring of LDS buffers in k-steps of 32.
 //  * skinny (M <= 64, decoding): bound by reading W once.  A workgroup owns 16 or 32 rows of W; its
 //    waves take interleaved 64-wide k blocks, stream W straight from memory into MFMA operands
 //    (v_mfma_f32_16x16x32_bf16, W as the A operand so that the 16 rows fill the tile) and combine
