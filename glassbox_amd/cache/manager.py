@@ -58,6 +58,8 @@ def _host():
         lib.gbh_cache_decode_rows.restype = C.c_int
         lib.gbh_cache_decode_rows.argtypes = [C.c_void_p, C.POINTER(C.c_int64), C.c_int, C.c_int] + [C.c_void_p] * 2 + \
                                              [C.c_void_p, C.c_int, C.c_void_p, C.c_int]
+        lib.gbh_cache_max_len.restype = C.c_int
+        lib.gbh_cache_max_len.argtypes = [C.c_void_p, C.POINTER(C.c_int64), C.c_int]
         lib.gbh_cache_step_rows.restype = C.c_int
         lib.gbh_cache_step_rows.argtypes = [C.c_void_p, C.POINTER(C.c_int64), C.POINTER(C.c_int32), C.c_int, C.c_int] + \
                                            [C.c_void_p] * 5 + [C.c_void_p, C.c_int, C.c_void_p, C.c_int]
@@ -165,6 +167,14 @@ class CacheManager:
             self._table_buf = (C.c_int32 * (2 * n))()
             n = self._lib.gbh_cache_table(self._h, seq_id, group, self._table_buf, len(self._table_buf))
         return self._table_buf[:n]
+
+    def max_len(self, seq_ids: Sequence[int]) -> int:
+        """The longest of the requests' lengths."""
+        ids = (C.c_int64 * max(1, len(seq_ids)))(*seq_ids)
+        n = self._lib.gbh_cache_max_len(self._h, ids, len(seq_ids))
+        if n < 0:
+            raise CacheError("unknown request")
+        return n
 
     def decode_rows(self, seq_ids: Sequence[int], stride: int, pos_ptr: int, state_ptr: int, rows_ptr: int,
                     rows_gap: int, tables_ptr: int, tables_gap: int) -> None:

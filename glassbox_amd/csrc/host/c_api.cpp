@@ -204,6 +204,43 @@ void gbh_sched_plan_entry(void* h, int i, int64_t* id, int* start, int* n, int* 
 }
 // Copies the tokens of plan entry i (n of them) into out.
 void gbh_sched_plan_entry_tokens(void* h, int i, int32_t* out) { ((gb::Scheduler*)h)->copy_entry_tokens(i, out); }
+// The whole plan in one call: per entry id, start, count, wants, decode (arrays of plan_size entries) and all
+// entries' tokens one after the other (plan_tokens of them).
+void gbh_sched_plan_all(void* h, int64_t* ids, int32_t* starts, int32_t* counts, int32_t* wants, int32_t* decodes,
+                        int32_t* tokens) {
+  auto* s = (gb::Scheduler*)h;
+  const auto& plan = s->planned();
+  int at = 0;
+  for (size_t i = 0; i < plan.size(); ++i) {
+    ids[i] = plan[i].id;
+    starts[i] = plan[i].start;
+    counts[i] = plan[i].n;
+    wants[i] = plan[i].wants ? 1 : 0;
+    decodes[i] = plan[i].decode ? 1 : 0;
+    s->copy_entry_tokens((int)i, tokens + at);
+    at += plan[i].n;
+  }
+}
+// Sampling parameters of the wanted rows 0 .. n-1 in one call (arrays of n entries; see gbh_sched_row_params).
+void gbh_sched_rows_params(void* h, int n, float* temperature, int32_t* top_k, float* top_p, float* min_p,
+                           float* repetition_penalty, float* uniform, int32_t* skip) {
+  for (int j = 0; j < n; ++j) {
+    int k = 0, sk = 0;
+    ((gb::Scheduler*)h)->row_params(j, temperature + j, &k, top_p + j, min_p + j, repetition_penalty + j, uniform + j, &sk);
+    top_k[j] = k;
+    skip[j] = sk;
+  }
+}
+// The longest of the requests' lengths (-1 for an unknown request).
+int gbh_cache_max_len(void* h, const int64_t* ids, int n) {
+  int longest = 0;
+  for (int i = 0; i < n; ++i) {
+    const int len = ((CacheManager*)h)->seq_len(ids[i]);
+    if (len < 0) return -1;
+    longest = std::max(longest, len);
+  }
+  return longest;
+}
 // Sampling parameters of the j-th wanted row, with a uniform number drawn ahead from a copy of
 // the request's generator (the draw is kept only if the device reports more than one candidate).
 void gbh_sched_row_params(void* h, int j, float* temperature, int* top_k, float* top_p, float* min_p,

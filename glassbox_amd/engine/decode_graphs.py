@@ -97,7 +97,7 @@ class DecodeGraphs:
         eng, cache = self.engine, self.engine.cache
         n = len(entries)
         sids = [e[0] for e in entries]
-        longest = max(cache.seq_len(s) for s in sids) + 1
+        longest = cache.max_len(sids) + 1
         key = (padded_rows(n), -(-longest // BUCKET) * BUCKET)
         shape = self.shapes.get(key)
         if shape is None:

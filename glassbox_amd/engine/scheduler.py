@@ -11,6 +11,8 @@ from __future__ import annotations
 
 import ctypes as C
 import time
+
+import numpy as np
 from dataclasses import dataclass, field
 from typing import Dict, List, Optional, Sequence, Tuple
 
@@ -39,6 +41,8 @@ def _host():
             "plan": (C.c_int, [vp]), "plan_size": (C.c_int, [vp]), "plan_tokens": (C.c_int, [vp]),
             "plan_entry": (None, [vp, C.c_int, i64p, ip, ip, ip, ip]),
             "plan_entry_tokens": (None, [vp, C.c_int, i32p]),
+            "plan_all": (None, [vp] + [vp] * 6),
+            "rows_params": (None, [vp, C.c_int] + [vp] * 7),
             "row_params": (None, [vp, C.c_int, fp, ip, fp, fp, fp, fp, ip]),
             "row_context": (C.c_int, [vp, C.c_int, i32p, C.c_int]),
             "finish": (None, [vp, i32p, i32p, C.c_int]),
@@ -95,6 +99,7 @@ class Scheduler:
         self.outputs: Dict[int, RequestOutput] = {}
         self.trace: Optional[List[StepRecord]] = [] if trace else None
         self._steps = 0
+        self._greedy = [SamplerConfig()] * 256   # what a step of greedy rows hands the sampler
         #: seconds from a request's arrival to its first token, and between its later tokens (scheduler.rs:127-129)
         self.ttft: List[float] = []
         self.itl: List[float] = []
@@ -149,33 +154,41 @@ class Scheduler:
             self._record(t0, [], finished)
             return rc == 2
         n = lib.gbh_sched_plan_size(h)
-        entries, batch_desc = [], []
-        rid, start, cnt, wants, dec = C.c_int64(), C.c_int(), C.c_int(), C.c_int(), C.c_int()
+        # the whole plan in one call: ids | starts, counts, wants, decodes | the entries' tokens
+        ids = np.empty(n, np.int64)
+        meta = np.empty((4, n), np.int32)
+        flat = np.empty(max(1, lib.gbh_sched_plan_tokens(h)), np.int32)
+        lib.gbh_sched_plan_all(h, ids.ctypes.data, meta[0].ctypes.data, meta[1].ctypes.data, meta[2].ctypes.data,
+                               meta[3].ctypes.data, flat.ctypes.data)
+        ids, (starts, counts, wants, decodes), flat = ids.tolist(), meta.tolist(), flat.tolist()
+        entries, batch_desc, at = [], [], 0
         for i in range(n):
-            lib.gbh_sched_plan_entry(h, i, C.byref(rid), C.byref(start), C.byref(cnt), C.byref(wants), C.byref(dec))
-            buf = (C.c_int32 * cnt.value)()
-            lib.gbh_sched_plan_entry_tokens(h, i, buf)
-            if start.value == 0:
-                self.engine.reset_state(rid.value)
-            entries.append((rid.value, list(buf), [cnt.value - 1] if wants.value else []))
-            batch_desc.append((rid.value, "decode" if dec.value else "prefill", cnt.value))
+            if starts[i] == 0:
+                self.engine.reset_state(ids[i])
+            entries.append((ids[i], flat[at:at + counts[i]], [counts[i] - 1] if wants[i] else []))
+            batch_desc.append((ids[i], "decode" if decodes[i] else "prefill", counts[i]))
+            at += counts[i]
         logits = self.engine.run_reserved(entries)
         rows = logits.shape[0]
-        configs, uniforms, contexts, skip = [], [], [], []
-        t, k, tp, mp, rp, u, sk = C.c_float(), C.c_int(), C.c_float(), C.c_float(), C.c_float(), C.c_float(), C.c_int()
-        for j in range(rows):
-            lib.gbh_sched_row_params(h, j, C.byref(t), C.byref(k), C.byref(tp), C.byref(mp), C.byref(rp), C.byref(u),
-                                     C.byref(sk))
-            configs.append(SamplerConfig(t.value, k.value, tp.value, mp.value, rp.value))
-            uniforms.append(u.value)
-            skip.append(sk.value)
-            if rp.value != 1.0:
-                m = lib.gbh_sched_row_context(h, j, None, 0)
-                cb = (C.c_int32 * max(1, m))()
-                lib.gbh_sched_row_context(h, j, cb, m)
-                contexts.append(list(cb[:m]))
-            else:
-                contexts.append([])
+        # sampling parameters of every wanted row: temperature, top_p, min_p, penalty, uniform | top_k, skip
+        fl, it = np.empty((5, max(1, rows)), np.float32), np.empty((2, max(1, rows)), np.int32)
+        lib.gbh_sched_rows_params(h, rows, fl[0].ctypes.data, it[0].ctypes.data, fl[1].ctypes.data, fl[2].ctypes.data,
+                                  fl[3].ctypes.data, fl[4].ctypes.data, it[1].ctypes.data)
+        temp, top_p, min_p, penalty, uniforms = (a[:rows] for a in fl.tolist())
+        top_k = it[0].tolist()[:rows]
+        if self.sample_fn is sample_rows and rows and max(temp) <= 0.0 and all(p == 1.0 for p in penalty):
+            configs, contexts = self._greedy[:rows] if rows <= len(self._greedy) else [SamplerConfig()] * rows, None
+        else:
+            configs = [SamplerConfig(temp[j], top_k[j], top_p[j], min_p[j], penalty[j]) for j in range(rows)]
+            contexts = []
+            for j in range(rows):
+                if penalty[j] != 1.0:
+                    m = lib.gbh_sched_row_context(h, j, None, 0)
+                    cb = (C.c_int32 * max(1, m))()
+                    lib.gbh_sched_row_context(h, j, cb, m)
+                    contexts.append(list(cb[:m]))
+                else:
+                    contexts.append([])
         tokens, cands = self.sample_fn(logits, configs, uniforms, contexts) if rows else ([], [])
         lib.gbh_sched_finish(h, (C.c_int32 * max(1, rows))(*tokens), (C.c_int32 * max(1, rows))(*cands), rows)
         finished = self._drain_events()
