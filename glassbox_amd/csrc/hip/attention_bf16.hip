@@ -301,15 +301,15 @@ struct PageSource {
   }
 };
 
-template <int HD>
-__device__ __forceinline__ void load_keys(bf16x8 (&kf)[2][HD / 16], const PageSource& src, int kbase, int lane) {
+template <int HD, int T>
+__device__ __forceinline__ void load_keys(bf16x8 (&kf)[T][HD / 16], const PageSource& src, int kbase, int lane) {
   const int col = lane & 31, g = lane >> 5;
   // row r of a group of 16 rows of the score tile takes key 8*((r>>2)&1) + 4*(r>>3) + (r&3) of the group:
   // the probabilities a lane then holds for a value product are those of 8 neighbouring keys
   const int r16 = col & 15, key16 = ((r16 >> 2) & 1) * 8 + (r16 >> 3) * 4 + (r16 & 3);
   const int mine = key16 * HD + 8 * g;
 #pragma unroll
-  for (int t = 0; t < 2; ++t) {
+  for (int t = 0; t < T; ++t) {
     int s0, s1;  // a tile of 32 keys is two groups of 16, each within one page
     const size_t p0 = src.page_of(kbase + 32 * t, &s0), p1 = src.page_of(kbase + 32 * t + 16, &s1);
     const bf16* b0 = src.kp + ((p0 << src.shift) + s0) * HD;
@@ -320,12 +320,12 @@ __device__ __forceinline__ void load_keys(bf16x8 (&kf)[2][HD / 16], const PageSo
   }
 }
 
-template <int HD>
-__device__ __forceinline__ void load_values(bf16x8 (&vf)[(HD + 31) / 32][4], const PageSource& src, int kbase, int lane) {
+template <int HD, int T>
+__device__ __forceinline__ void load_values(bf16x8 (&vf)[(HD + 31) / 32][2 * T], const PageSource& src, int kbase, int lane) {
   const int col = lane & 31, g = lane >> 5;
   const int mine = (col << src.shift) + 8 * g;
 #pragma unroll
-  for (int u = 0; u < 4; ++u) {
+  for (int u = 0; u < 2 * T; ++u) {
     int slot;
     const size_t pg = src.page_of(kbase + 16 * u, &slot);
     const bf16* vb = src.vp + ((pg * HD) << src.shift) + slot + mine;
@@ -335,15 +335,16 @@ __device__ __forceinline__ void load_values(bf16x8 (&vf)[(HD + 31) / 32][4], con
   }
 }
 
-// One step over the 64 keys from kbase, whose fragments kf and vf hold.  The live blocks take their
+// One step over the 32 T keys from kbase (T = 2; T = 1 for the head sizes whose fragments of 64 keys do not
+// fit the registers), whose fragments kf and vf hold.  The live blocks take their
 // turn one after the other (scores, softmax, values), so that only one block's scores are in
 // registers at a time; as soon as the last block's score products have read kf it is loaded again
 // for the keys from `next`, and vf likewise after the last value products, so that those loads are
 // in flight during the arithmetic in between.
-template <int HD, int QB, int ACT>
+template <int HD, int QB, int ACT, int T = 2>
 __device__ __forceinline__ void attend64_q32(float (&m)[QB], float (&l)[QB], f32x16 (&acc)[QB][(HD + 31) / 32],
-                                             const bf16x8* __restrict__ q_lds, int q_at, bf16x8 (&kf)[2][HD / 16],
-                                             bf16x8 (&vf)[(HD + 31) / 32][4], const PageSource& src, int kbase, int next,
+                                             const bf16x8* __restrict__ q_lds, int q_at, bf16x8 (&kf)[T][HD / 16],
+                                             bf16x8 (&vf)[(HD + 31) / 32][2 * T], const PageSource& src, int kbase, int next,
                                              const int (&lo)[QB], const int (&hi)[QB], bool mask, float c, int lane) {
   constexpr int KS = HD / 16, DB = (HD + 31) / 32;
   constexpr int LAST = (ACT & 2) ? 1 : 0;
@@ -355,9 +356,9 @@ __device__ __forceinline__ void attend64_q32(float (&m)[QB], float (&l)[QB], f32
 #pragma unroll
   for (int qb = 0; qb < QB; ++qb) {
     if (!((ACT >> qb) & 1)) continue;
-    f32x16 s[2];
+    f32x16 s[T];
 #pragma unroll
-    for (int t = 0; t < 2; ++t) {
+    for (int t = 0; t < T; ++t) {
 #pragma unroll
       for (int r = 0; r < 16; ++r) s[t][r] = 0.f;
 #pragma unroll
@@ -367,11 +368,11 @@ __device__ __forceinline__ void attend64_q32(float (&m)[QB], float (&l)[QB], f32
     if (qb == LAST) {
       // not earlier: above the score products the old and the new fragments would both need registers
       __builtin_amdgcn_sched_barrier(0);
-      load_keys<HD>(kf, src, next, lane);
+      load_keys<HD, T>(kf, src, next, lane);
     }
     if (mask) {  // the same for the whole wave
 #pragma unroll
-      for (int t = 0; t < 2; ++t)
+      for (int t = 0; t < T; ++t)
 #pragma unroll
         for (int r = 0; r < 16; ++r) {
           const int key = kbase + 32 * t + 16 * (r >> 3) + 8 * g + 4 * ((r >> 2) & 1) + (r & 3);
@@ -380,7 +381,7 @@ __device__ __forceinline__ void attend64_q32(float (&m)[QB], float (&l)[QB], f32
     }
     float mx = -INFINITY;
 #pragma unroll
-    for (int t = 0; t < 2; ++t)
+    for (int t = 0; t < T; ++t)
 #pragma unroll
       for (int r = 0; r < 16; ++r) mx = fmaxf(mx, s[t][r]);
     mx = fmaxf(mx, __shfl_xor(mx, 32, kWave));
@@ -390,7 +391,7 @@ __device__ __forceinline__ void attend64_q32(float (&m)[QB], float (&l)[QB], f32
     const float mc = m_ref * c;
     float sum = 0.f;
 #pragma unroll
-    for (int t = 0; t < 2; ++t)
+    for (int t = 0; t < T; ++t)
 #pragma unroll
       for (int r = 0; r < 16; ++r) {
         s[t][r] = __builtin_amdgcn_exp2f(fmaf(s[t][r], c, -mc));
@@ -405,7 +406,7 @@ __device__ __forceinline__ void attend64_q32(float (&m)[QB], float (&l)[QB], f32
         for (int r = 0; r < 16; ++r) acc[qb][b][r] *= alpha;
     }
 #pragma unroll
-    for (int u = 0; u < 4; ++u) {
+    for (int u = 0; u < 2 * T; ++u) {
       bf16x8 pf;
 #pragma unroll
       for (int e = 0; e < 8; ++e) pf[e] = (bf16)s[u >> 1][8 * (u & 1) + e];
@@ -414,7 +415,7 @@ __device__ __forceinline__ void attend64_q32(float (&m)[QB], float (&l)[QB], f32
     }
   }
   __builtin_amdgcn_sched_barrier(0);
-  load_values<HD>(vf, src, next, lane);
+  load_values<HD, T>(vf, src, next, lane);
 }
 
 // What a wave knows of one block of 32 tokens: the keys [first, last] that any of its tokens sees, and
@@ -422,8 +423,8 @@ __device__ __forceinline__ void attend64_q32(float (&m)[QB], float (&l)[QB], f32
 struct BlockRange {
   int first, last, free_lo, free_hi;
   bool whole;
-  __device__ bool live(int kb) const { return kb <= last && kb + 63 >= first; }
-  __device__ bool unmasked(int kb) const { return whole && kb >= free_lo && kb + 63 <= free_hi; }
+  // of the keys kb .. kb + span - 1
+  __device__ bool unmasked(int kb, int span = 64) const { return whole && kb >= free_lo && kb + span - 1 <= free_hi; }
 };
 
 __device__ __forceinline__ BlockRange block_range(int t0, int qlen, int p0, int window) {
@@ -485,8 +486,10 @@ __global__ __launch_bounds__(256, 2) void prefill_kernel(const bf16* __restrict_
   PageSource src{kp, vp, tables + (size_t)seq * table_stride, nkv, kvh, page_shift, 0, 0};
   const size_t row0 = (size_t)q_start[seq];
   const float c = scale * 1.4426950408889634f;
-  bf16x8 kf[2][KS];
-  bf16x8 vf[DB][4];
+  constexpr int T = QB == 2 ? 2 : 1;  // tiles of 32 keys a step: with one block live at a time (the larger head
+                                      // sizes) the fragments of 64 keys would not fit the registers
+  bf16x8 kf[T][KS];
+  bf16x8 vf[DB][2 * T];
   // The query fragments wait in LDS, each lane's own in a place of its own (no lane reads another's):
   // they are needed once per step over 64 keys, and the registers are better spent on the accumulators.
   __shared__ bf16x8 q_lds[4 * QB * KS * 64];
@@ -523,8 +526,8 @@ __global__ __launch_bounds__(256, 2) void prefill_kernel(const bf16* __restrict_
     src.tlo = range[0].first & ~15;
     src.thi = end & ~15;
     int kb = range[0].first & ~63;
-    load_keys<HD>(kf, src, kb, lane);
-    load_values<HD>(vf, src, kb, lane);
+    load_keys<HD, T>(kf, src, kb, lane);
+    load_values<HD, T>(vf, src, kb, lane);
     if (has_second) {
       // both blocks as far as the earlier one's keys reach (with a window the later one may see none of
       // them yet: they are masked), then the later block alone
@@ -566,10 +569,12 @@ __global__ __launch_bounds__(256, 2) void prefill_kernel(const bf16* __restrict_
       const BlockRange range = block_range(start[which], qlen, p0, window);
       src.tlo = range.first & ~15;
       src.thi = range.last & ~15;
-      load_keys<HD>(kf, src, range.first & ~63, lane);
-      load_values<HD>(vf, src, range.first & ~63, lane);
-      for (int kb = range.first & ~63; kb <= range.last; kb += 64)
-        attend64_q32<HD, 1, 1>(m, l, acc, q_lds, q_at, kf, vf, src, kb, kb + 64, lo, hi, !range.unmasked(kb), c, lane);
+      constexpr int SPAN = 32 * T;
+      load_keys<HD, T>(kf, src, range.first & ~(SPAN - 1), lane);
+      load_values<HD, T>(vf, src, range.first & ~(SPAN - 1), lane);
+      for (int kb = range.first & ~(SPAN - 1); kb <= range.last; kb += SPAN)
+        attend64_q32<HD, 1, 1, T>(m, l, acc, q_lds, q_at, kf, vf, src, kb, kb + SPAN, lo, hi, !range.unmasked(kb, SPAN), c,
+                                  lane);
       const float total = l[0] + __shfl_xor(l[0], 32, kWave);
       if (valid) store_block<HD>(acc[0], total, out + (row0 + tok) * out_stride + (size_t)head * HD, g);
     }

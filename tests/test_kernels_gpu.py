@@ -535,6 +535,7 @@ class BareContext:
 
 
 @pytest.mark.parametrize("nh,nkv,hd,window", [(4, 2, 16, 0), (3, 1, 32, 0), (6, 2, 48, 0), (8, 8, 64, 0), (8, 2, 128, 0),
+                                              (6, 3, 96, 0), (4, 4, 112, 0), (4, 2, 128, 70),
                                               (16, 1, 64, 0), (5, 5, 80, 0), (4, 2, 64, 37), (4, 4, 64, 300), (2, 1, 112, 0)])
 @pytest.mark.parametrize("page", [16, 64])
 def test_tuned_attention_against_the_plain_kernel(nh, nkv, hd, window, page):
