@@ -1024,10 +1024,11 @@ int launch_fold(const void* a, int lda, const bf16* w, int ldw, CT* c, int ldc, 
 // GB_SKINNY="waves,iters,rowtiles" overrides (for measurements).
 inline void skinny_plan(int tiles, int K, int mt, int* waves, int* iters, int* rt) {
   // measured on SmolLM2-1.7B and Llama-3-8B shapes: sixteen waves a workgroup keep the most loads in
-  // flight; two row tiles a workgroup halve the re-reading of A once there are tiles enough
+  // flight; two row tiles a workgroup halve the re-reading of A once that still leaves workgroups for
+  // three quarters of the compute units (384 tiles: better with two; 256 tiles: better with one)
   const int blocks = (K + 63) / 64;               // 64-wide k blocks
   *waves = blocks >= 16 ? 16 : 4;
-  *rt = tiles >= 256 ? 2 : 1;
+  *rt = tiles >= 384 ? 2 : 1;
   const int per_wave = (blocks + *waves - 1) / *waves;
   *iters = (mt == 1 && per_wave >= 2) ? 2 : 1;
   if (const char* env = getenv("GB_SKINNY")) {
