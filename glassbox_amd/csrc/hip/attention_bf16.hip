@@ -455,10 +455,45 @@ __device__ __forceinline__ void store_block(const f32x16 (&acc)[(HD + 31) / 32],
     }
 }
 
-// grid (groups of four waves, query heads, requests from seq_base on); wave w of a request takes its
-// blocks w and n-1-w of 32 tokens.
-template <int HD, int QB>
-__global__ __launch_bounds__(256, 2) void prefill_kernel(const bf16* __restrict__ q, int q_stride, bf16* __restrict__ out,
+// The waves 1 .. SPLIT-1 that shared a block's keys hand their maximum, sum and accumulators to wave 0 of their
+// group through LDS (`handed`: DB*16*64 floats, `handed_ml`: 2*64, both the group's own), one wave at a time.
+// Every wave of the workgroup calls this (it holds barriers); `again` is false only at the workgroup's first call.
+template <int DB, int SPLIT>
+__device__ __forceinline__ void hand_over(float& m, float& l, f32x16 (&acc)[DB], float* handed, float* handed_ml, int half,
+                                          int lane, float c, bool again) {
+  for (int giver = 1; giver < SPLIT; ++giver) {
+    if (again || giver > 1) __syncthreads();  // what was handed over before has been taken
+    if (half == giver) {
+      handed_ml[lane] = m;
+      handed_ml[64 + lane] = l;
+#pragma unroll
+      for (int b = 0; b < DB; ++b)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) handed[(b * 16 + r) * 64 + lane] = acc[b][r];
+    }
+    __syncthreads();
+    if (half == 0) {
+      const float m1 = handed_ml[lane], l1 = handed_ml[64 + lane];
+      const float top = fmaxf(m, m1);
+      const float ref = top == -INFINITY ? 0.f : top;
+      const float a0 = m == -INFINITY ? 0.f : __builtin_amdgcn_exp2f((m - ref) * c);
+      const float a1 = m1 == -INFINITY ? 0.f : __builtin_amdgcn_exp2f((m1 - ref) * c);
+      m = top;
+      l = l * a0 + l1 * a1;
+#pragma unroll
+      for (int b = 0; b < DB; ++b)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) acc[b][r] = acc[b][r] * a0 + handed[(b * 16 + r) * 64 + lane] * a1;
+    }
+  }
+}
+
+// grid (groups of PAIRS pairs of blocks, query heads, requests from seq_base on); pair w of a request is its
+// blocks w and n-1-w of 32 tokens.  SPLIT waves share a pair: they take its tiles of 64 keys in turn, and at the
+// end the others hand their sums to the first through LDS.  One wave a pair is best when the pairs alone give
+// every SIMD a wave; short portions and few heads do not, and then the keys are what is left to divide.
+template <int HD, int QB, int PAIRS, int SPLIT>
+__global__ __launch_bounds__(64 * PAIRS * SPLIT, 2) void prefill_kernel(const bf16* __restrict__ q, int q_stride, bf16* __restrict__ out,
                                                       int out_stride, const int32_t* __restrict__ q_start,
                                                       const int32_t* __restrict__ q_len, const int32_t* __restrict__ pos0,
                                                       int seq_base, const int32_t* __restrict__ tables, int table_stride,
@@ -474,12 +509,17 @@ __global__ __launch_bounds__(256, 2) void prefill_kernel(const bf16* __restrict_
   const int die = linear % kDies;
   const int unit = die * (total / kDies) + min(die, total % kDies) + linear / kDies;
   const int seq = seq_base + unit / (gx * gy), head = unit / gx % gy, group = unit % gx;
+  static_assert(QB == 2 || PAIRS == 1 || SPLIT == 1, "one block at a time: waves share keys only if the workgroup is one pair");
+  static_assert(PAIRS * SPLIT <= 8, "two waves a SIMD have the registers this kernel needs");
   const int tid = threadIdx.x, lane = tid & 63;
-  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);  // the same in all lanes: what follows from it is scalar
+  const int wave_of_all = __builtin_amdgcn_readfirstlane(tid >> 6);  // the same in all lanes: what follows from it is scalar
+  const int wave = wave_of_all / SPLIT, half = wave_of_all % SPLIT;  // which pair; which of its tiles of keys
   const int qlen = q_len[seq];
   const int blocks = (qlen + 31) / 32;
-  const int w = group * 4 + wave;
-  if (2 * w >= blocks) return;
+  const int w = group * PAIRS + wave;
+  const bool works = 2 * w < blocks;
+  if (SPLIT == 1 && !works) return;
+  if (2 * group * PAIRS >= blocks) return;  // the whole workgroup; with SPLIT > 1 every wave left goes to the barriers below
   const int col = lane & 31, g = lane >> 5;
   const int p0 = pos0[seq];
   const int kvh = head / (nh / nkv);
@@ -492,7 +532,9 @@ __global__ __launch_bounds__(256, 2) void prefill_kernel(const bf16* __restrict_
   bf16x8 vf[DB][2 * T];
   // The query fragments wait in LDS, each lane's own in a place of its own (no lane reads another's):
   // they are needed once per step over 64 keys, and the registers are better spent on the accumulators.
-  __shared__ bf16x8 q_lds[4 * QB * KS * 64];
+  __shared__ bf16x8 q_lds[PAIRS * QB * KS * 64];
+  __shared__ float handed[SPLIT > 1 ? PAIRS : 1][SPLIT > 1 ? DB * 16 * 64 : 1];  // see hand_over
+  __shared__ float handed_ml[PAIRS][2 * 64];
   const int q_at = wave * (QB * KS * 64) + lane;
   bf16x8* qf = q_lds + q_at;
   // the wave's two blocks start at these tokens; the later one is absent when it is the earlier one itself
@@ -507,7 +549,7 @@ __global__ __launch_bounds__(256, 2) void prefill_kernel(const bf16* __restrict_
 #pragma unroll
     for (int qb = 0; qb < 2; ++qb) {
       const int tok = start[qb] + col;
-      const bool valid = tok < qlen && (qb == 0 || has_second);
+      const bool valid = works && tok < qlen && (qb == 0 || has_second);
       const int p = p0 + tok;
       lo[qb] = valid ? (window > 0 ? max(0, p - window + 1) : 0) : 1;
       hi[qb] = valid ? p : 0;
@@ -525,24 +567,47 @@ __global__ __launch_bounds__(256, 2) void prefill_kernel(const bf16* __restrict_
     const int end = has_second ? range[1].last : range[0].last;
     src.tlo = range[0].first & ~15;
     src.thi = end & ~15;
+    // the tiles of 64 keys in order: both blocks as far as the earlier one's keys reach (with a window the later
+    // one may see none of them yet: they are masked), then, with a window after a gap, the later block alone
+    auto after = [&](int kb) {
+      int next = kb + 64;
+      if (has_second && kb <= range[0].last && next > range[0].last && next + 63 < range[1].first) next = range[1].first & ~63;
+      return next;
+    };
+    auto my_next = [&](int kb) {  // the waves of a pair take the tiles in turn
+#pragma unroll
+      for (int i = 0; i < SPLIT; ++i) kb = after(kb);
+      return kb;
+    };
     int kb = range[0].first & ~63;
+    for (int i = 0; i < half; ++i) kb = after(kb);
+    if (!works) kb = end + 1;  // (a pair beyond the request's last block only goes to the barriers)
     load_keys<HD, T>(kf, src, kb, lane);
     load_values<HD, T>(vf, src, kb, lane);
     if (has_second) {
-      // both blocks as far as the earlier one's keys reach (with a window the later one may see none of
-      // them yet: they are masked), then the later block alone
       while (kb <= range[0].last) {
-        int next = kb + 64;
-        if (next > range[0].last && next + 63 < range[1].first) next = range[1].first & ~63;
+        const int next = my_next(kb);
         const bool mask = !(range[0].unmasked(kb) && range[1].unmasked(kb));
         attend64_q32<HD, 2, 3>(m, l, acc, q_lds, q_at, kf, vf, src, kb, next, lo, hi, mask, c, lane);
         kb = next;
       }
-      for (; kb <= range[1].last; kb += 64)
-        attend64_q32<HD, 2, 2>(m, l, acc, q_lds, q_at, kf, vf, src, kb, kb + 64, lo, hi, !range[1].unmasked(kb), c, lane);
+      while (kb <= range[1].last) {
+        const int next = my_next(kb);
+        attend64_q32<HD, 2, 2>(m, l, acc, q_lds, q_at, kf, vf, src, kb, next, lo, hi, !range[1].unmasked(kb), c, lane);
+        kb = next;
+      }
     } else {
-      for (; kb <= range[0].last; kb += 64)
-        attend64_q32<HD, 2, 1>(m, l, acc, q_lds, q_at, kf, vf, src, kb, kb + 64, lo, hi, !range[0].unmasked(kb), c, lane);
+      while (kb <= range[0].last) {
+        const int next = my_next(kb);
+        attend64_q32<HD, 2, 1>(m, l, acc, q_lds, q_at, kf, vf, src, kb, next, lo, hi, !range[0].unmasked(kb), c, lane);
+        kb = next;
+      }
+    }
+    if constexpr (SPLIT > 1) {
+#pragma unroll
+      for (int qb = 0; qb < 2; ++qb)
+        hand_over<DB, SPLIT>(m[qb], l[qb], acc[qb], handed[wave], handed_ml[wave], half, lane, c, qb > 0);
+      if (half != 0 || !works) return;
     }
 #pragma unroll
     for (int qb = 0; qb < 2; ++qb) {
@@ -569,12 +634,17 @@ __global__ __launch_bounds__(256, 2) void prefill_kernel(const bf16* __restrict_
       const BlockRange range = block_range(start[which], qlen, p0, window);
       src.tlo = range.first & ~15;
       src.thi = range.last & ~15;
-      constexpr int SPAN = 32 * T;
-      load_keys<HD, T>(kf, src, range.first & ~(SPAN - 1), lane);
-      load_values<HD, T>(vf, src, range.first & ~(SPAN - 1), lane);
-      for (int kb = range.first & ~(SPAN - 1); kb <= range.last; kb += SPAN)
-        attend64_q32<HD, 1, 1, T>(m, l, acc, q_lds, q_at, kf, vf, src, kb, kb + SPAN, lo, hi, !range.unmasked(kb, SPAN), c,
-                                  lane);
+      constexpr int SPAN = 32 * T;  // the waves of the pair take the steps of SPAN keys in turn
+      const int kb0 = (range.first & ~(SPAN - 1)) + half * SPAN;
+      load_keys<HD, T>(kf, src, kb0, lane);
+      load_values<HD, T>(vf, src, kb0, lane);
+      for (int kb = kb0; kb <= range.last; kb += SPAN * SPLIT)
+        attend64_q32<HD, 1, 1, T>(m, l, acc, q_lds, q_at, kf, vf, src, kb, kb + SPAN * SPLIT, lo, hi,
+                                  !range.unmasked(kb, SPAN), c, lane);
+      if constexpr (SPLIT > 1) {
+        hand_over<DB, SPLIT>(m[0], l[0], acc[0], handed[wave], handed_ml[wave], half, lane, c, which > 0);
+        if (half != 0) continue;
+      }
       const float total = l[0] + __shfl_xor(l[0], 32, kWave);
       if (valid) store_block<HD>(acc[0], total, out + (row0 + tok) * out_stride + (size_t)head * HD, g);
     }
@@ -632,11 +702,13 @@ extern "C" int gb_attention_decode_bf16(const void* q, int q_stride, void* out, 
   return 0;
 }
 
-// Requests seq_base .. seq_base+n_seqs-1 of the step (prompt portions); max_q_len is the longest portion.
+// Requests seq_base .. seq_base+n_seqs-1 of the step (prompt portions); max_q_len is the longest portion and
+// max_context the longest context any of them reaches (both only shape the launch).
 extern "C" int gb_attention_prefill_bf16(const void* q, int q_stride, void* out, int out_stride, const int32_t* q_start,
                                          const int32_t* q_len, const int32_t* pos0, int seq_base, int n_seqs, int max_q_len,
-                                         const int32_t* tables, int table_stride, const void* k_pages, const void* v_pages,
-                                         int nh, int nkv, int hd, int page_size, float scale, int window, hipStream_t stream) {
+                                         int max_context, const int32_t* tables, int table_stride, const void* k_pages,
+                                         const void* v_pages, int nh, int nkv, int hd, int page_size, float scale, int window,
+                                         hipStream_t stream) {
   GB_REQUIRE(n_seqs >= 0 && nh > 0 && nkv > 0 && nh % nkv == 0, "attention_prefill: bad head counts nh=%d nkv=%d", nh, nkv);
   GB_REQUIRE(gb_attention_supported_head_size(hd), "attention_prefill: head size %d is not a multiple of 16 up to 128", hd);
   GB_REQUIRE(page_size >= 16 && (page_size & (page_size - 1)) == 0, "attention_prefill: page size %d is not a power of two from 16 up", page_size);
@@ -646,14 +718,42 @@ extern "C" int gb_attention_prefill_bf16(const void* q, int q_stride, void* out,
              "attention_prefill: q rows must be 16-byte aligned and out rows 8-byte aligned");
   GB_REQUIRE(n_seqs <= 65535 && nh <= 65535, "attention_prefill: too many requests or heads for one launch");
   if (n_seqs == 0 || max_q_len <= 0) return 0;
-  // a wave takes two blocks of 32 tokens, a workgroup four waves
-  const dim3 grid((max_q_len + 255) / 256, nh, n_seqs), block(256);
-#define GB_CASE(HD)                                                                                                        \
-  if (hd == HD)                                                                                                            \
-    hipLaunchKernelGGL((prefill_kernel<HD, (HD <= 64 ? 2 : 1)>), grid, block, 0, stream, (const bf16*)q, q_stride,          \
-                       (bf16*)out, out_stride, q_start, q_len, pos0, seq_base, tables, table_stride, (const bf16*)k_pages, \
-                       (const bf16*)v_pages, nh, nkv, page_shift, scale, window);
+  // A pair of blocks of 32 tokens is the unit of work.  A compute unit is what a workgroup's waves share, and
+  // what bounds them together: so the pairs are spread over workgroups first (four a workgroup only if that still
+  // gives every compute unit one), and then, up to head size 64, a pair's keys over waves, four waves a workgroup
+  // (eight where even single pairs leave compute units idle).  Waves that find no tile of keys left only merge.
+  static const int forced = [] { const char* e = getenv("GB_PREFILL_SPLIT"); return e ? atoi(e) : 0; }();
+  const long long pairs = (long long)((max_q_len + 63) / 64) * nh * n_seqs;
+  int per_group = pairs >= 1024 ? 4 : pairs >= 512 ? 2 : 1, split = 1;
+  if (hd <= 64) {
+    split = 4 / per_group;
+    if (per_group == 1 && pairs <= 128) split = 8;
+    if (forced == 1 || forced == 2 || forced == 4 || forced == 8) split = forced, per_group = forced == 8 ? 1 : 4 / forced;
+  } else if (per_group < 4) {  // one block at a time: waves share keys only in a workgroup of one pair
+    per_group = 1;
+    split = pairs <= 128 ? 8 : 4;
+  }
+  (void)max_context;
+  const dim3 grid((max_q_len + 64 * per_group - 1) / (64 * per_group), nh, n_seqs), block(64 * per_group * split);
+#define GB_LAUNCH(HD, QB, PAIRS, SPLIT)                                                                                     \
+  hipLaunchKernelGGL((prefill_kernel<HD, QB, PAIRS, SPLIT>), grid, block, 0, stream, (const bf16*)q, q_stride, (bf16*)out, \
+                     out_stride, q_start, q_len, pos0, seq_base, tables, table_stride, (const bf16*)k_pages,               \
+                     (const bf16*)v_pages, nh, nkv, page_shift, scale, window)
+#define GB_CASE(HD)                                        \
+  if (hd == HD) {                                          \
+    if constexpr (HD <= 64) {                              \
+      if (split == 1) GB_LAUNCH(HD, 2, 4, 1);              \
+      if (split == 2) GB_LAUNCH(HD, 2, 2, 2);              \
+      if (split == 4) GB_LAUNCH(HD, 2, 1, 4);              \
+      if (split == 8) GB_LAUNCH(HD, 2, 1, 8);              \
+    } else {                                               \
+      if (per_group == 4) GB_LAUNCH(HD, 1, 4, 1);          \
+      if (per_group == 1 && split == 4) GB_LAUNCH(HD, 1, 1, 4); \
+      if (per_group == 1 && split == 8) GB_LAUNCH(HD, 1, 1, 8); \
+    }                                                      \
+  }
   GB_FOR_HEAD_SIZES(GB_CASE)
 #undef GB_CASE
+#undef GB_LAUNCH
   return launched("attention_prefill");
 }

@@ -70,9 +70,9 @@ _SIGS = {
         # n_decode, nh, nkv, hd, page, scale, window, chunk, max_context, stream
         "gb_attention_decode_bf16": [_vp, _i, _vp, _i, _vp, _vp, _vp, _vp, _i, _vp, _vp, _i, _i, _i, _i, _i, _f, _i,
                                      _i, _i, _vp],
-        # q, q_stride, out, out_stride, q_start, q_len, pos0, seq_base, n_seqs, max_q_len, tables, table_stride,
-        # k, v, nh, nkv, hd, page, scale, window, stream
-        "gb_attention_prefill_bf16": [_vp, _i, _vp, _i, _vp, _vp, _vp, _i, _i, _i, _vp, _i, _vp, _vp, _i, _i, _i, _i,
+        # q, q_stride, out, out_stride, q_start, q_len, pos0, seq_base, n_seqs, max_q_len, max_context, tables,
+        # table_stride, k, v, nh, nkv, hd, page, scale, window, stream
+        "gb_attention_prefill_bf16": [_vp, _i, _vp, _i, _vp, _vp, _vp, _i, _i, _i, _i, _vp, _i, _vp, _vp, _i, _i, _i, _i,
                                       _f, _i, _vp],
     },
     "sampling": {
@@ -477,7 +477,7 @@ def attention_prefill(q: torch.Tensor, out: torch.Tensor, ctx, cache, n_heads: i
     lib = _lib("attention_bf16")
     _check(lib, lib.gb_attention_prefill_bf16(_p(q), _rows(q, "q"), _p(out), _rows(out, "out"), _p(ctx.q_start),
                                               _p(ctx.q_len), _p(ctx.pos0), n_dec, S - n_dec, int(ctx.host["max_q_len"]),
-                                              _p(tables), tables.stride(0), _p(k_pages), _p(v_pages), n_heads, nkv, hd,
+                                              int(ctx.host["max_context"]), _p(tables), tables.stride(0), _p(k_pages), _p(v_pages), n_heads, nkv, hd,
                                               page, float(scale), int(window), _stream()))
 
 

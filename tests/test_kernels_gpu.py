@@ -568,7 +568,8 @@ def test_tuned_attention_against_the_plain_kernel(nh, nkv, hd, window, page):
 
 
 @pytest.mark.parametrize("nh,nkv,hd,window", [(32, 32, 64, 0), (32, 8, 48, 0), (32, 4, 16, 100), (32, 32, 64, 200),
-                                              (32, 16, 32, 0)])
+                                              (32, 16, 32, 0), (32, 8, 128, 0), (8, 8, 96, 0), (40, 8, 64, 0), (16, 4, 64, 0),
+                                              (16, 16, 64, 150)])
 def test_tuned_prefill_long_portions(nh, nkv, hd, window):
     """Portions long enough, and heads enough, that a wave takes 64 tokens: one portion starts in the
     middle of its request and ends off every tile edge, the other is a whole short prompt."""
