@@ -565,9 +565,10 @@ inline SplitPlan split_plan(int M, int N, int K) {
   }
   const int tiles = ((N + 127) / 128) * ((M + p.bm - 1) / p.bm);
   if (tiles >= 192 || N % 8 != 0) return p;
-  // measured on SmolLM2-1.7B shapes: a long k (the down projection) always gains; a short one only where
-  // the skinny kernel is at its weakest (33 to 64 rows: every workgroup reads all of A)
-  if (K < 4096 && !(M > 32 && M <= 64)) return p;
+  // measured on SmolLM2-1.7B shapes: a long k (the down projection) always gains; a short one where the
+  // skinny kernel is at its weakest (33 to 64 rows: every workgroup reads all of A) and where the tiles are
+  // very few (the O projection of a portion of some hundred rows: 16 to 64 tiles)
+  if (K < 4096 && !(M > 32 && M <= 64) && !(M > 64 && K >= 2048 && tiles <= 128)) return p;
   // a slice keeps at least 8 k-steps (shorter ones cost more in partial sums than they gain)
   int want = (512 + tiles - 1) / tiles;
   want = want > 16 ? 16 : want;

@@ -188,7 +188,9 @@ def test_gemm_bf16_prepares_the_next_norm(M, N, K, N2, silu, gamma_dtype):
 @pytest.mark.parametrize("M,N,K", [(17, 96, 4096), (33, 2048, 2048), (64, 2048, 8192), (64, 6144, 2048), (100, 2048, 4160),
                                    (200, 528, 8200), (64, 16384, 2048), (40, 1008, 4104), (512, 2048, 8192),
                                    # a thousand rows and more: slices of k through the 256 x 256 tiles
-                                   (2048, 2048, 8192), (1100, 1008, 4160), (1024, 528, 5120)])
+                                   (2048, 2048, 8192), (1100, 1008, 4160), (1024, 528, 5120),
+                                   # some hundred rows, a k of 2,048 and very few tiles
+                                   (128, 2048, 2048), (512, 2048, 2048), (300, 1008, 2112)])
 @pytest.mark.parametrize("mode", ["bf16", "f32", "f32+", "silu"])
 def test_gemm_bf16_divides_k_over_workgroups(M, N, K, mode):
     """With a workspace, a product of few tiles has several workgroups a tile, each over a slice of k,
