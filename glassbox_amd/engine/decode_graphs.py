@@ -19,13 +19,15 @@ every part must declare ``replayable`` (parts.base.Part).
 """
 from __future__ import annotations
 
-from typing import Dict, List, Sequence, Tuple
+from collections import OrderedDict
+from typing import List, Sequence, Tuple
 
 import torch
 
 from .context import StepContext, Workspace
 
 BUCKET = 1024
+MAX_SHAPES = 64   # shapes kept (buffers and a graph each); the least recently used one goes first
 
 
 def padded_rows(n: int) -> int:
@@ -85,7 +87,7 @@ class DecodeGraphs:
         self.engine = engine
         #: buffers of its own: steps of other shapes make the engine's buffers grow, and a graph holds addresses
         self.workspace = Workspace(engine.device)
-        self.shapes: Dict[Tuple[int, int], _Shape] = {}
+        self.shapes: "OrderedDict[Tuple[int, int], _Shape]" = OrderedDict()
         self.epoch = 0
         self.replays = 0
 
@@ -101,7 +103,12 @@ class DecodeGraphs:
         key = (padded_rows(n), -(-longest // BUCKET) * BUCKET)
         shape = self.shapes.get(key)
         if shape is None:
+            if len(self.shapes) >= MAX_SHAPES:
+                torch.cuda.synchronize()         # its last replay may still be running
+                self.shapes.popitem(last=False)
             shape = self.shapes[key] = _Shape(eng, self.workspace, *key)
+        else:
+            self.shapes.move_to_end(key)
         shape.copied.synchronize()           # the last copy out of the pinned buffer has run
         hv = shape.host.numpy()
         hv[:] = shape.filler

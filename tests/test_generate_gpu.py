@@ -309,3 +309,26 @@ def test_steps_of_single_tokens_replay_graphs_like_plain_steps(model_dirs, name,
             e.end_request(r)
         e.cache.check_invariants()
         assert e.cache.used_pages() == 0
+
+
+def test_decode_graph_shapes_are_kept_up_to_a_limit(model_dirs, monkeypatch):
+    """Only so many shapes keep their buffers and graph; the least recently used one makes room, and a shape that
+    comes back is warmed and captured again.  The logits stay those of an engine without graphs."""
+    from glassbox_amd.engine import Engine, decode_graphs
+    monkeypatch.setattr(decode_graphs, "MAX_SHAPES", 2)
+    folder = model_dirs.get("A")
+    vocab = helpers.TINY["A"]["vocab_size"]
+    prompts = {r: helpers.random_tokens(vocab, n, seed=80 + i) for i, (r, n) in enumerate({"a": 20, "b": 9, "c": 31}.items())}
+    engs = [Engine(folder, dtype="bfloat16", max_tokens=1024, max_seqs=4, graph_decode=g) for g in (True, False)]
+    nxt = {"a": 3, "b": 4, "c": 5}
+    for r, toks in prompts.items():
+        for e in engs:
+            e.step([(r, toks, [])])
+    for live in (["a"], ["a", "b"], ["a", "b", "c"], ["a"], ["b", "c"], ["c", "a", "b"]):
+        for _ in range(4):
+            outs = [e.step([(r, [nxt[r]], [0]) for r in live]).float().cpu() for e in engs]
+            assert float((outs[0] - outs[1]).abs().max()) <= 8e-3 * max(1.0, float(outs[1].abs().max())), live
+            for r, row in zip(live, outs[1]):
+                nxt[r] = int(row.argmax())
+        assert len(engs[0].decode_graphs.shapes) <= 2
+    assert engs[0].decode_graphs.replays >= 6
