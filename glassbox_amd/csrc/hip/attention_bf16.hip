@@ -455,6 +455,47 @@ __device__ __forceinline__ void store_block(const f32x16 (&acc)[(HD + 31) / 32],
     }
 }
 
+// A block's sums as they stand (not divided by l), for the pass that adds the parts of workgroups that shared its
+// keys: part_acc [part][row][head][HD], part_ml [part][row][head][2] = the maximum and l.
+template <int HD>
+__device__ __forceinline__ void store_part(const f32x16 (&acc)[(HD + 31) / 32], float m, float l, float* __restrict__ acc_row,
+                                           float* __restrict__ ml, int g) {
+#pragma unroll
+  for (int b = 0; b < (HD + 31) / 32; ++b)
+#pragma unroll
+    for (int jj = 0; jj < 4; ++jj) {
+      const int d0 = 32 * b + 8 * jj + 4 * g;
+      if (32 * b + 32 <= HD || d0 < HD) {
+        f32x4 o;
+#pragma unroll
+        for (int r = 0; r < 4; ++r) o[r] = acc[b][4 * jj + r];
+        *reinterpret_cast<f32x4*>(acc_row + d0) = o;
+      }
+    }
+  if (g == 0) {
+    ml[0] = m;
+    ml[1] = l;
+  }
+}
+
+// Adds the parts in their order: one workgroup of HD threads per (row, head).
+__global__ void prefill_parts_kernel(const float* __restrict__ part_acc, const float* __restrict__ part_ml, bf16* __restrict__ out,
+                                     int out_stride, int first_row, int n_rows, int nh, int hd, int parts, float c) {
+  const int row = blockIdx.x / nh, head = blockIdx.x % nh, d = threadIdx.x;
+  if (d >= hd) return;
+  const size_t cell = (size_t)row * nh + head, stride = (size_t)n_rows * nh;
+  float top = -INFINITY;
+  for (int k = 0; k < parts; ++k) top = fmaxf(top, part_ml[(k * stride + cell) * 2]);
+  float val = 0.f, l = 0.f;
+  for (int k = 0; k < parts; ++k) {
+    const float mk = part_ml[(k * stride + cell) * 2];
+    const float f = mk == -INFINITY ? 0.f : __builtin_amdgcn_exp2f((mk - top) * c);
+    val += part_acc[(k * stride + cell) * hd + d] * f;
+    l += part_ml[(k * stride + cell) * 2 + 1] * f;
+  }
+  out[(size_t)(first_row + row) * out_stride + (size_t)head * hd + d] = (bf16)(val / l);
+}
+
 // The waves 1 .. SPLIT-1 that shared a block's keys hand their maximum, sum and accumulators to wave 0 of their
 // group through LDS (`handed`: DB*16*64 floats, `handed_ml`: 2*64, both the group's own), one wave at a time.
 // Every wave of the workgroup calls this (it holds barriers); `again` is false only at the workgroup's first call.
@@ -498,7 +539,10 @@ __global__ __launch_bounds__(64 * PAIRS * SPLIT, 2) void prefill_kernel(const bf
                                                       const int32_t* __restrict__ q_len, const int32_t* __restrict__ pos0,
                                                       int seq_base, const int32_t* __restrict__ tables, int table_stride,
                                                       const bf16* __restrict__ kp, const bf16* __restrict__ vp, int nh, int nkv,
-                                                      int page_shift, float scale, int window) {
+                                                      int page_shift, float scale, int window, float* __restrict__ part_acc,
+                                                      float* __restrict__ part_ml, int parts, int first_row, int n_rows) {
+  // parts > 1: `parts` workgroups share a group's pairs, taking the tiles of keys in turn like the waves of a pair
+  // do; each writes its sums to part_acc / part_ml (rows counted from first_row), and prefill_parts_kernel adds them.
   constexpr int KS = HD / 16, DB = (HD + 31) / 32;
   // Workgroups go to the chip's eight dies in turn, each die with an L2 of its own.  The ones that
   // land on one die are given consecutive units of work, so that a head's keys and values, which all
@@ -508,7 +552,7 @@ __global__ __launch_bounds__(64 * PAIRS * SPLIT, 2) void prefill_kernel(const bf
   const int linear = blockIdx.x + gx * (blockIdx.y + gy * blockIdx.z);
   const int die = linear % kDies;
   const int unit = die * (total / kDies) + min(die, total % kDies) + linear / kDies;
-  const int seq = seq_base + unit / (gx * gy), head = unit / gx % gy, group = unit % gx;
+  const int seq = seq_base + unit / (gx * gy), head = unit / gx % gy, group = unit % gx / parts, part = unit % gx % parts;
   static_assert(QB == 2 || PAIRS == 1 || SPLIT == 1, "one block at a time: waves share keys only if the workgroup is one pair");
   static_assert(PAIRS * SPLIT <= 8, "two waves a SIMD have the registers this kernel needs");
   const int tid = threadIdx.x, lane = tid & 63;
@@ -574,13 +618,12 @@ __global__ __launch_bounds__(64 * PAIRS * SPLIT, 2) void prefill_kernel(const bf
       if (has_second && kb <= range[0].last && next > range[0].last && next + 63 < range[1].first) next = range[1].first & ~63;
       return next;
     };
-    auto my_next = [&](int kb) {  // the waves of a pair take the tiles in turn
-#pragma unroll
-      for (int i = 0; i < SPLIT; ++i) kb = after(kb);
+    auto my_next = [&](int kb) {  // the waves of a pair (in all the workgroups that share it) take the tiles in turn
+      for (int i = 0; i < SPLIT * parts; ++i) kb = after(kb);
       return kb;
     };
     int kb = range[0].first & ~63;
-    for (int i = 0; i < half; ++i) kb = after(kb);
+    for (int i = 0; i < part * SPLIT + half; ++i) kb = after(kb);
     if (!works) kb = end + 1;  // (a pair beyond the request's last block only goes to the barriers)
     load_keys<HD, T>(kf, src, kb, lane);
     load_values<HD, T>(vf, src, kb, lane);
@@ -614,6 +657,11 @@ __global__ __launch_bounds__(64 * PAIRS * SPLIT, 2) void prefill_kernel(const bf
       const float total = l[qb] + __shfl_xor(l[qb], 32, kWave);
       const int tok = start[qb] + col;
       if (tok >= qlen || (qb == 1 && !has_second)) continue;
+      if (parts > 1) {
+        const size_t cell = ((size_t)part * n_rows + (row0 + tok - first_row)) * nh + head;
+        store_part<HD>(acc[qb], m[qb], total, part_acc + cell * HD, part_ml + cell * 2, g);
+        continue;
+      }
       store_block<HD>(acc[qb], total, out + (row0 + tok) * out_stride + (size_t)head * HD, g);
     }
   } else {
@@ -635,18 +683,23 @@ __global__ __launch_bounds__(64 * PAIRS * SPLIT, 2) void prefill_kernel(const bf
       src.tlo = range.first & ~15;
       src.thi = range.last & ~15;
       constexpr int SPAN = 32 * T;  // the waves of the pair take the steps of SPAN keys in turn
-      const int kb0 = (range.first & ~(SPAN - 1)) + half * SPAN;
+      const int kb0 = (range.first & ~(SPAN - 1)) + (part * SPLIT + half) * SPAN, stride = SPAN * SPLIT * parts;
       load_keys<HD, T>(kf, src, kb0, lane);
       load_values<HD, T>(vf, src, kb0, lane);
-      for (int kb = kb0; kb <= range.last; kb += SPAN * SPLIT)
-        attend64_q32<HD, 1, 1, T>(m, l, acc, q_lds, q_at, kf, vf, src, kb, kb + SPAN * SPLIT, lo, hi,
-                                  !range.unmasked(kb, SPAN), c, lane);
+      for (int kb = kb0; kb <= range.last; kb += stride)
+        attend64_q32<HD, 1, 1, T>(m, l, acc, q_lds, q_at, kf, vf, src, kb, kb + stride, lo, hi, !range.unmasked(kb, SPAN), c,
+                                  lane);
       if constexpr (SPLIT > 1) {
         hand_over<DB, SPLIT>(m[0], l[0], acc[0], handed[wave], handed_ml[wave], half, lane, c, which > 0);
         if (half != 0) continue;
       }
       const float total = l[0] + __shfl_xor(l[0], 32, kWave);
-      if (valid) store_block<HD>(acc[0], total, out + (row0 + tok) * out_stride + (size_t)head * HD, g);
+      if (valid && parts > 1) {
+        const size_t cell = ((size_t)part * n_rows + (row0 + tok - first_row)) * nh + head;
+        store_part<HD>(acc[0], m[0], total, part_acc + cell * HD, part_ml + cell * 2, g);
+      } else if (valid) {
+        store_block<HD>(acc[0], total, out + (row0 + tok) * out_stride + (size_t)head * HD, g);
+      }
     }
   }
 }
@@ -702,12 +755,54 @@ extern "C" int gb_attention_decode_bf16(const void* q, int q_stride, void* out, 
   return 0;
 }
 
+// How the prompt portions of a step are spread over the chip.  A pair of blocks of 32 tokens is the unit of work.
+// A compute unit is what a workgroup's waves share, and what bounds them together: so the pairs are spread over
+// workgroups first (four a workgroup only if that still gives every compute unit one), then a pair's keys over
+// waves (four a workgroup; eight where even single pairs leave compute units idle), and where the pairs are fewer
+// than half the compute units and the contexts long, over `parts` workgroups whose sums a second pass adds.
+struct PrefillPlan {
+  int per_group, split, parts;
+};
+inline PrefillPlan prefill_plan(int max_q_len, int max_context, int nh, int n_seqs, int hd) {
+  static const int forced = [] { const char* e = getenv("GB_PREFILL_SPLIT"); return e ? atoi(e) : 0; }();
+  static const int forced_parts = [] { const char* e = getenv("GB_PREFILL_PARTS"); return e ? atoi(e) : 0; }();
+  const long long pairs = (long long)((max_q_len + 63) / 64) * nh * n_seqs;
+  PrefillPlan p{pairs >= 1024 ? 4 : pairs >= 512 ? 2 : 1, 1, 1};
+  if (hd <= 64) {
+    p.split = 4 / p.per_group;
+    if (p.per_group == 1 && pairs <= 128) p.split = 8;
+    if (forced == 1 || forced == 2 || forced == 4 || forced == 8) p.split = forced, p.per_group = forced == 8 ? 1 : 4 / forced;
+  } else if (p.per_group < 4) {  // one block at a time: waves share keys only in a workgroup of one pair
+    p.per_group = 1;
+    p.split = pairs <= 128 ? 8 : 4;
+  }
+  if (p.per_group == 1 && pairs <= 128) {
+    // a wave keeps at least four tiles of 64 keys; four waves a workgroup then, and up to eight workgroups a pair
+    const int tiles = (max(max_context, max_q_len) + 63) / 64;
+    int parts = (int)(256 / (pairs > 0 ? pairs : 1));
+    parts = parts > 8 ? 8 : parts;
+    while (parts > 1 && parts * 4 * 4 > tiles) --parts;
+    if (forced_parts >= 1 && forced_parts <= 8) parts = forced_parts;
+    if (parts > 1) p.parts = parts, p.split = 4;
+  }
+  return p;
+}
+
+// Workgroups that would share a pair's keys with these sizes (1: none do); the caller then provides
+// parts * rows * nh * (hd + 2) floats for their sums, rows being all rows of the portions.
+extern "C" int gb_attention_prefill_parts(int max_q_len, int max_context, int nh, int n_seqs, int hd) {
+  return prefill_plan(max_q_len, max_context, nh, n_seqs, hd).parts;
+}
+
 // Requests seq_base .. seq_base+n_seqs-1 of the step (prompt portions); max_q_len is the longest portion and
-// max_context the longest context any of them reaches (both only shape the launch).
+// max_context the longest context any of them reaches (both only shape the launch).  first_row, n_rows: the rows of
+// q and out that the portions occupy (contiguous); part_ws: float32 workspace of part_floats elements, needed if
+// gb_attention_prefill_parts says so.
 extern "C" int gb_attention_prefill_bf16(const void* q, int q_stride, void* out, int out_stride, const int32_t* q_start,
                                          const int32_t* q_len, const int32_t* pos0, int seq_base, int n_seqs, int max_q_len,
                                          int max_context, const int32_t* tables, int table_stride, const void* k_pages,
                                          const void* v_pages, int nh, int nkv, int hd, int page_size, float scale, int window,
+                                         int first_row, int n_rows, float* part_ws, long long part_floats,
                                          hipStream_t stream) {
   GB_REQUIRE(n_seqs >= 0 && nh > 0 && nkv > 0 && nh % nkv == 0, "attention_prefill: bad head counts nh=%d nkv=%d", nh, nkv);
   GB_REQUIRE(gb_attention_supported_head_size(hd), "attention_prefill: head size %d is not a multiple of 16 up to 128", hd);
@@ -718,27 +813,22 @@ extern "C" int gb_attention_prefill_bf16(const void* q, int q_stride, void* out,
              "attention_prefill: q rows must be 16-byte aligned and out rows 8-byte aligned");
   GB_REQUIRE(n_seqs <= 65535 && nh <= 65535, "attention_prefill: too many requests or heads for one launch");
   if (n_seqs == 0 || max_q_len <= 0) return 0;
-  // A pair of blocks of 32 tokens is the unit of work.  A compute unit is what a workgroup's waves share, and
-  // what bounds them together: so the pairs are spread over workgroups first (four a workgroup only if that still
-  // gives every compute unit one), and then, up to head size 64, a pair's keys over waves, four waves a workgroup
-  // (eight where even single pairs leave compute units idle).  Waves that find no tile of keys left only merge.
-  static const int forced = [] { const char* e = getenv("GB_PREFILL_SPLIT"); return e ? atoi(e) : 0; }();
-  const long long pairs = (long long)((max_q_len + 63) / 64) * nh * n_seqs;
-  int per_group = pairs >= 1024 ? 4 : pairs >= 512 ? 2 : 1, split = 1;
-  if (hd <= 64) {
-    split = 4 / per_group;
-    if (per_group == 1 && pairs <= 128) split = 8;
-    if (forced == 1 || forced == 2 || forced == 4 || forced == 8) split = forced, per_group = forced == 8 ? 1 : 4 / forced;
-  } else if (per_group < 4) {  // one block at a time: waves share keys only in a workgroup of one pair
-    per_group = 1;
-    split = pairs <= 128 ? 8 : 4;
+  const PrefillPlan plan = prefill_plan(max_q_len, max_context, nh, n_seqs, hd);
+  const int per_group = plan.per_group, split = plan.split, parts = plan.parts;
+  float *part_acc = nullptr, *part_ml = nullptr;
+  if (parts > 1) {
+    const long long cells = (long long)parts * n_rows * nh;
+    GB_REQUIRE(part_ws && part_floats >= cells * (hd + 2) && n_rows > 0 && first_row >= 0 && ((uintptr_t)part_ws % 16 == 0),
+               "attention_prefill: %d workgroups share a pair's keys: a workspace of %lld floats is needed", parts,
+               cells * (hd + 2));
+    part_acc = part_ws;
+    part_ml = part_ws + cells * hd;
   }
-  (void)max_context;
-  const dim3 grid((max_q_len + 64 * per_group - 1) / (64 * per_group), nh, n_seqs), block(64 * per_group * split);
+  const dim3 grid((max_q_len + 64 * per_group - 1) / (64 * per_group) * parts, nh, n_seqs), block(64 * per_group * split);
 #define GB_LAUNCH(HD, QB, PAIRS, SPLIT)                                                                                     \
   hipLaunchKernelGGL((prefill_kernel<HD, QB, PAIRS, SPLIT>), grid, block, 0, stream, (const bf16*)q, q_stride, (bf16*)out, \
                      out_stride, q_start, q_len, pos0, seq_base, tables, table_stride, (const bf16*)k_pages,               \
-                     (const bf16*)v_pages, nh, nkv, page_shift, scale, window)
+                     (const bf16*)v_pages, nh, nkv, page_shift, scale, window, part_acc, part_ml, parts, first_row, n_rows)
 #define GB_CASE(HD)                                        \
   if (hd == HD) {                                          \
     if constexpr (HD <= 64) {                              \
@@ -755,5 +845,11 @@ extern "C" int gb_attention_prefill_bf16(const void* q, int q_stride, void* out,
   GB_FOR_HEAD_SIZES(GB_CASE)
 #undef GB_CASE
 #undef GB_LAUNCH
-  return launched("attention_prefill");
+  if (int rc = launched("attention_prefill")) return rc;
+  if (parts > 1) {
+    hipLaunchKernelGGL(prefill_parts_kernel, dim3((unsigned)(n_rows * nh)), dim3((hd + 63) / 64 * 64), 0, stream, part_acc, part_ml,
+                       (bf16*)out, out_stride, first_row, n_rows, nh, hd, parts, scale * 1.4426950408889634f);
+    return launched("attention_prefill (second pass)");
+  }
+  return 0;
 }

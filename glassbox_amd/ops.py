@@ -71,9 +71,10 @@ _SIGS = {
         "gb_attention_decode_bf16": [_vp, _i, _vp, _i, _vp, _vp, _vp, _vp, _i, _vp, _vp, _i, _i, _i, _i, _i, _f, _i,
                                      _i, _i, _vp],
         # q, q_stride, out, out_stride, q_start, q_len, pos0, seq_base, n_seqs, max_q_len, max_context, tables,
-        # table_stride, k, v, nh, nkv, hd, page, scale, window, stream
+        # table_stride, k, v, nh, nkv, hd, page, scale, window, first_row, n_rows, part_ws, part_floats, stream
         "gb_attention_prefill_bf16": [_vp, _i, _vp, _i, _vp, _vp, _vp, _i, _i, _i, _i, _vp, _i, _vp, _vp, _i, _i, _i, _i,
-                                      _f, _i, _vp],
+                                      _f, _i, _i, _i, _vp, C.c_longlong, _vp],
+        "gb_attention_prefill_parts": [_i, _i, _i, _i, _i],
     },
     "sampling": {
         "gb_argmax": [_vp, _vp, _i, _i, _vp],
@@ -475,10 +476,17 @@ def attention_prefill(q: torch.Tensor, out: torch.Tensor, ctx, cache, n_heads: i
         raise KernelError("attention_prefill: q and out must be bfloat16 [n, heads * head size]")
     tables = ctx.tables[cache.group]
     lib = _lib("attention_bf16")
+    max_q, max_ctx = int(ctx.host["max_q_len"]), int(ctx.host["max_context"])
+    # the portions' rows follow the single-token requests' rows; few and short portions over long contexts share
+    # their keys among workgroups, which need room for their sums
+    first_row, n_rows = n_dec, q.shape[0] - n_dec
+    parts = lib.gb_attention_prefill_parts(max_q, max_ctx, n_heads, S - n_dec, hd)
+    ws = ctx.buffer("attn_parts", (parts * n_rows * n_heads * (hd + 2),), torch.float32) if parts > 1 else None
     _check(lib, lib.gb_attention_prefill_bf16(_p(q), _rows(q, "q"), _p(out), _rows(out, "out"), _p(ctx.q_start),
-                                              _p(ctx.q_len), _p(ctx.pos0), n_dec, S - n_dec, int(ctx.host["max_q_len"]),
-                                              int(ctx.host["max_context"]), _p(tables), tables.stride(0), _p(k_pages), _p(v_pages), n_heads, nkv, hd,
-                                              page, float(scale), int(window), _stream()))
+                                              _p(ctx.q_len), _p(ctx.pos0), n_dec, S - n_dec, max_q, max_ctx, _p(tables),
+                                              tables.stride(0), _p(k_pages), _p(v_pages), n_heads, nkv, hd, page,
+                                              float(scale), int(window), first_row, n_rows, _p(ws),
+                                              ws.numel() if ws is not None else 0, _stream()))
 
 
 # ------------------------------------------------------------------------ sampling

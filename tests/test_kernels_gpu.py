@@ -646,6 +646,39 @@ def test_tuned_decode_finds_one_far_key_in_every_chunk_position():
             assert (out.cpu().float()[0] - want).abs().max().item() < 2e-2, f"key at {target} was not found"
 
 
+@pytest.mark.parametrize("nh,nkv,hd,window", [(8, 2, 64, 0), (4, 4, 128, 0), (6, 3, 32, 700), (8, 8, 96, 0)])
+def test_tuned_prefill_short_portions_over_long_contexts(nh, nkv, hd, window):
+    """Few pairs of blocks and long contexts: several workgroups share a pair's keys and a second pass adds their
+    sums.  Two short portions at the ends of long requests, beside a request of a single token."""
+    from types import SimpleNamespace
+    from glassbox_amd import ops
+    q_lens, ctx_lens = [1, 100, 37], [400, 2150, 1301]
+    k_pages, v_pages, tables, ks, vs = paged_setup(ctx_lens, nkv, hd, 16, seed=hd + nh, dtype=torch.bfloat16)
+    ctx = BareContext(q_lens, ctx_lens, tables)
+    lib = ops._lib("attention_bf16")
+    assert lib.gb_attention_prefill_parts(max(q_lens), max(ctx_lens), nh, 2, hd) > 1
+    n = sum(q_lens)
+    q = (rnd(n, nh * hd, seed=14) * 0.7).bfloat16()
+    scale = 1 / math.sqrt(hd)
+    cache = SimpleNamespace(k_pages=to_dev(k_pages), v_pages=to_dev(v_pages), group=0)
+    out = torch.zeros(n, nh * hd, device=DEV, dtype=torch.bfloat16)
+    qd = to_dev(q)
+    ops.attention_decode(qd, out, ctx, cache, nh, scale, window)
+    ops.attention_prefill(qd, out, ctx, cache, nh, scale, window)
+    twin = torch.zeros_like(out)
+    ops.attention_plain(qd, twin, ctx.positions, torch.tensor(ctx.tok_seq, dtype=torch.int32, device=DEV), ctx.tables[0],
+                        cache.k_pages, cache.v_pages, nh, scale, window)
+    close = (out.float() - twin.float()).abs() <= 2 ** -7 * (1 + twin.float().abs())
+    bad = torch.nonzero(~close.all(dim=1)).flatten().tolist()
+    assert not bad, f"rows {bad[:8]} (request, position) {[(ctx.tok_seq[i], ctx.pos_list[i]) for i in bad[:8]]}"
+    want = plain_attention_rows(q, ks, vs, ctx.tok_seq, ctx.pos_list, nh, scale, window)
+    assert (out.cpu().double() - want).abs().max().item() < 2 ** -6
+    again = torch.zeros_like(out)
+    ops.attention_decode(qd, again, ctx, cache, nh, scale, window)
+    ops.attention_prefill(qd, again, ctx, cache, nh, scale, window)
+    assert torch.equal(out, again)
+
+
 @pytest.mark.parametrize("nh,ctxlen,qlen", [(2, 200, 90), (64, 1200, 1090)])   # 32 and 64 tokens a wave
 def test_tuned_prefill_sees_exactly_the_causal_keys(nh, ctxlen, qlen):
     """A portion in the middle of a request (it starts at position 110): token t must find a marked
