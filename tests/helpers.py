@@ -28,7 +28,11 @@ TINY_C = dict(architectures=["LlamaForCausalLM"], hidden_size=80, intermediate_s
 MID_M = dict(architectures=["LlamaForCausalLM"], hidden_size=960, intermediate_size=2560, num_hidden_layers=2,
              num_attention_heads=15, num_key_value_heads=5, vocab_size=1000, rope_theta=100000.0,
              rms_norm_eps=1e-5, tie_word_embeddings=True, max_position_embeddings=8192)
-TINY = {"A": TINY_A, "B": TINY_B, "C": TINY_C, "M": MID_M}
+# one layer of SmolLM2-1.7B's widths (the benchmark's shapes: 2,048 wide, 32 heads, 8,192 in the feed-forward)
+WIDE_W = dict(architectures=["LlamaForCausalLM"], hidden_size=2048, intermediate_size=8192, num_hidden_layers=1,
+              num_attention_heads=32, num_key_value_heads=32, vocab_size=1000, rope_theta=130000.0,
+              rms_norm_eps=1e-5, tie_word_embeddings=True, max_position_embeddings=8192)
+TINY = {"A": TINY_A, "B": TINY_B, "C": TINY_C, "M": MID_M, "W": WIDE_W}
 
 
 class ModelDirs:

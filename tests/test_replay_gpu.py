@@ -118,6 +118,30 @@ def test_layers_of_real_width(engines, model_dirs, dtype):
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_a_layer_of_the_benchmark_widths(engines, model_dirs, dtype):
+    """One layer as wide as SmolLM2-1.7B's, the shapes of the benchmark: a prompt of 2,100 tokens whole (the
+    products with 256 x 256 tiles and operands loaded straight into LDS, their slices of k in the down
+    projection), in portions of many sizes, with its last tokens one by one, and mixed with a shorter request."""
+    folder = model_dirs.get("W")
+    vocab = helpers.TINY["W"]["vocab_size"]
+    requests = {"w0": helpers.random_tokens(vocab, 2100, seed=51), "w1": helpers.random_tokens(vocab, 300, seed=52)}
+    eng = engines("W", dtype, max_tokens=4096)
+    # bfloat16: as in the test above, the tolerance keeps its ratio to the logits' root mean square
+    rms = float(np.sqrt(np.mean(helpers.plain_logits(folder, tuple(requests["w1"])) ** 2)))
+    tol = TOL[dtype] * (max(1.0, rms / 0.25) if dtype == "bfloat16" else 1.0)
+    check = functools.partial(globals()["check"], tol=tol)
+    for mode, make in (("whole", helpers.schedule_whole), ("tail32", helpers.schedule_tail),
+                       ("chunks", lambda r: helpers.schedule_chunks(r, sizes=(1030, 2, 512, 129, 64, 300)))):
+        got = helpers.replay(eng, make(requests))
+        check(folder, requests, got, dtype, mode)
+    steps, peak = helpers.schedule_mixed(requests, seed=5, live=2)
+    got = helpers.replay(eng, steps)
+    check(folder, requests, got, dtype, "mixed")
+    eng.cache.check_invariants()
+    assert eng.cache.used_pages() == 0
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 def test_long_decoding(engines, model_dirs, dtype):
     folder = model_dirs.get("C")
     toks = helpers.random_tokens(helpers.TINY["C"]["vocab_size"], 300, seed=9)
