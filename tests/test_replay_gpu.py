@@ -23,12 +23,14 @@ REQUESTS = {
     "A": {"a0": 5, "a1": 17, "a2": 49, "a3": 128, "a4": 70, "a5": 33},
     "B": {"b0": 1, "b1": 33, "b2": 64, "b3": 94, "b4": 200, "b5": 40},
     "C": {"c0": 3, "c1": 47, "c2": 130, "c3": 65, "c4": 257},
+    "D": {"d0": 2, "d1": 31, "d2": 150, "d3": 64, "d4": 301},
 }
 # more requests than are live at once, so that finished requests' pages are handed out again
 MORE = {
     "A": {"a6": 100, "a7": 60, "a8": 128, "a9": 20, "a10": 81},
     "B": {"b6": 150, "b7": 17, "b8": 256, "b9": 77},
     "C": {"c5": 90, "c6": 33, "c7": 200, "c8": 16, "c9": 129},
+    "D": {"d5": 70, "d6": 129, "d7": 18, "d8": 260},
 }
 
 
@@ -62,7 +64,7 @@ def engines(model_dirs):
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
-@pytest.mark.parametrize("name", ["A", "B", "C"])
+@pytest.mark.parametrize("name", ["A", "B", "C", "D"])
 @pytest.mark.parametrize("mode", ["whole", "tail32", "chunks"])
 def test_single_request_splits(engines, model_dirs, name, dtype, mode):
     folder = model_dirs.get(name)
@@ -77,7 +79,7 @@ def test_single_request_splits(engines, model_dirs, name, dtype, mode):
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
-@pytest.mark.parametrize("name", ["A", "B", "C"])
+@pytest.mark.parametrize("name", ["A", "B", "C", "D"])
 def test_mixed_batches_with_page_reuse(model_dirs, name, dtype):
     from glassbox_amd.engine import Engine
     folder = model_dirs.get(name)
