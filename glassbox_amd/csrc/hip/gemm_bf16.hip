@@ -603,9 +603,62 @@ __global__ void splitk_reduce_kernel(const float* __restrict__ ws, int slices, C
   }
 }
 
+// The same pass for a product that accumulates into the float32 residual, one workgroup a row; with the new row
+// in hand it also does the RMS norm that reads the residual next: h[m, n] = gamma[n] * (r[m, n] * s),
+// s = 1 / sqrt(mean(r[m]^2) + eps), the formula of the norm's own kernel.  Rows of up to SPLIT_NORM_MAX columns.
+constexpr int SPLIT_NORM_MAX = 256 * 4 * 8;
+template <typename G>
+__global__ __launch_bounds__(256) void splitk_reduce_norm_kernel(const float* __restrict__ ws, int slices, float* __restrict__ c,
+                                                                 int ldc, int M, int N, const G* __restrict__ gamma, float eps,
+                                                                 bf16* __restrict__ h, int ldh) {
+  __shared__ float partial[4];
+  const int m = blockIdx.x, tid = threadIdx.x;
+  f32x4 r[8];
+  float ss = 0.f;
+#pragma unroll
+  for (int i = 0; i < 8; ++i) {
+    const int j = (tid + 256 * i) * 4;
+    if (j >= N) break;
+    f32x4 sum = {0.f, 0.f, 0.f, 0.f};  // the slices in their order, then the residual: as the plain second pass does
+    for (int z = 0; z < slices; ++z) sum += *reinterpret_cast<const f32x4*>(ws + ((size_t)z * M + m) * N + j);
+    sum = *reinterpret_cast<const f32x4*>(c + (size_t)m * ldc + j) + sum;
+    *reinterpret_cast<f32x4*>(c + (size_t)m * ldc + j) = sum;
+    r[i] = sum;
+    ss += sum[0] * sum[0] + sum[1] * sum[1] + sum[2] * sum[2] + sum[3] * sum[3];
+  }
+#pragma unroll
+  for (int off = 32; off > 0; off >>= 1) ss += __shfl_xor(ss, off, 64);
+  if (tid % 64 == 0) partial[tid / 64] = ss;
+  __syncthreads();
+  const float total = partial[0] + partial[1] + partial[2] + partial[3];
+  const float scale = 1.0f / sqrtf(total / (float)N + eps);
+#pragma unroll
+  for (int i = 0; i < 8; ++i) {
+    const int j = (tid + 256 * i) * 4;
+    if (j >= N) break;
+    bf16x4 o;
+#pragma unroll
+    for (int e = 0; e < 4; ++e) o[e] = (bf16)((float)gamma[j + e] * (r[i][e] * scale));
+    *reinterpret_cast<bf16x4*>(h + (size_t)m * ldh + j) = o;
+  }
+}
+
+// Folded tiles pay when the product has at most 8 rows and whole tiles of 16 rows of W would leave
+// compute units without a workgroup (measured: with 384 such tiles they no longer do).
+inline bool fold_pays(int M, int N) { return M <= 8 && (N + 15) / 16 < 256; }
+
+// What an accumulating product of these sizes can do for the RMS norm that reads the residual after it:
+// 0 nothing; 1 (the folded kernel, at most 8 rows) the operand bf16(gamma * r) and partial sums, see NormExtras;
+// 2 (a product that divides k, given its workspace) the whole norm, in the pass that adds the slices.
+inline int emit_mode(int M, int N, int K) {
+  if (fold_pays(M, N)) return 1;
+  if (M > 16 && N % 4 == 0 && N <= SPLIT_NORM_MAX && split_plan(M, N, K).slices > 1) return 2;
+  return 0;
+}
+
 template <int EPI, typename CT>
 int launch_split(const bf16* a, int lda, const bf16* w, int ldw, CT* c, int ldc, int M, int N, int K, float* ws,
-                 const SplitPlan& plan, hipStream_t stream) {
+                 const SplitPlan& plan, hipStream_t stream, const NormExtras* norm = nullptr, float eps = 0.f) {
   const dim3 grid((N + 127) / 128, (M + plan.bm - 1) / plan.bm, plan.slices), block(256);
   const bool kfull = K % TBK == 0;
   const bool ring = plan.ring && ring_takes(a, lda, w, ldw, K);
@@ -619,6 +672,17 @@ int launch_split(const bf16* a, int lda, const bf16* w, int ldw, CT* c, int ldc,
   GB_S(1, true) GB_S(1, false) GB_S(2, true) GB_S(2, false)
 #undef GB_S
   if (int rc = launched("gemm_bf16 (split k)")) return rc;
+  if constexpr (EPI == EPI_ACCUMULATE && std::is_same<CT, float>::value) {
+    if (norm && norm->emit_h) {
+      if (norm->emit_gamma_f32)
+        hipLaunchKernelGGL((splitk_reduce_norm_kernel<float>), dim3(M), dim3(256), 0, stream, ws, plan.slices, c, ldc, M, N,
+                           (const float*)norm->emit_gamma, eps, norm->emit_h, norm->emit_ldh);
+      else
+        hipLaunchKernelGGL((splitk_reduce_norm_kernel<bf16>), dim3(M), dim3(256), 0, stream, ws, plan.slices, c, ldc, M, N,
+                           (const bf16*)norm->emit_gamma, eps, norm->emit_h, norm->emit_ldh);
+      return launched("gemm_bf16 (split k, second pass with the norm)");
+    }
+  }
   const int cols = EPI == EPI_SILU_MUL ? N / 2 : N;
   const size_t threads = (size_t)M * (cols / 4);
   hipLaunchKernelGGL((splitk_reduce_kernel<EPI, CT>), dim3((unsigned)((threads + 255) / 256)), dim3(256), 0, stream, ws,
@@ -1000,10 +1064,6 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_fold_kernel(const void* __res
   }
 }
 
-// Folded tiles pay when the product has at most 8 rows and whole tiles of 16 rows of W would leave
-// compute units without a workgroup (measured: with 384 such tiles they no longer do).
-inline bool fold_pays(int M, int N) { return M <= 8 && (N + 15) / 16 < 256; }
-
 template <int EPI, bool RMS, typename CT>
 int launch_fold(const void* a, int lda, const bf16* w, int ldw, CT* c, int ldc, int M, int N, int K, const void* gamma,
                 int gamma_f32, float eps, const NormExtras& extra, hipStream_t stream) {
@@ -1087,6 +1147,9 @@ int launch_skinny(const void* a, int lda, const bf16* w, int ldw, CT* c, int ldc
 // gamma): the rows of a are such an operand and the product is scaled by the norm's factor from n_parts
 // partial sums; eps is that norm's.
 extern "C" int gb_gemm_bf16_emit_parts(int M, int N) { return fold_pays(M, N) ? (N + 7) / 8 : 0; }
+// 0, 1 or 2: see emit_mode.  With 2, gb_gemm_bf16 takes emit_gamma, emit_h and eps (no emit_ss) together with the
+// workspace and writes the normed rows to emit_h.
+extern "C" int gb_gemm_bf16_emit_mode(int M, int N, int K) { return emit_mode(M, N, K); }
 
 // Floats of workspace with which gb_gemm_bf16 would split k for this product (0: it would not).
 extern "C" long long gb_gemm_bf16_split_floats(int M, int N, int K) {
@@ -1110,22 +1173,25 @@ extern "C" int gb_gemm_bf16(const void* a, int lda, const void* w, int ldw, void
   GB_REQUIRE(!gamma || (M <= 64 && c_dtype == kBF16 && epilogue != EPI_ACCUMULATE && ((uintptr_t)gamma % 16 == 0) &&
                         (gamma_dtype == kF32 || gamma_dtype == kBF16)),
              "gemm_bf16: the fused RMS norm serves up to 64 rows with a bfloat16 result");
-  GB_REQUIRE(!emit_h || (epilogue == EPI_ACCUMULATE && fold_pays(M, N) && emit_gamma && emit_ss && emit_ldh >= N &&
-                         (emit_gamma_dtype == kF32 || emit_gamma_dtype == kBF16)),
-             "gemm_bf16: only an accumulating product that gb_gemm_bf16_emit_parts accepts can prepare the next norm");
+  const int emits = emit_h ? emit_mode(M, N, K) : 0;
+  GB_REQUIRE(!emit_h || (epilogue == EPI_ACCUMULATE && emit_gamma && emit_ldh >= N && ((uintptr_t)emit_gamma % 16 == 0) &&
+                         (emit_gamma_dtype == kF32 || emit_gamma_dtype == kBF16) &&
+                         ((emits == 1 && emit_ss) || (emits == 2 && split_ws && emit_ldh % 4 == 0 && ((uintptr_t)emit_h % 8 == 0)))),
+             "gemm_bf16: only an accumulating product that gb_gemm_bf16_emit_mode accepts can prepare the next norm");
   GB_REQUIRE(!parts || (M <= 8 && !gamma && n_parts > 0 && epilogue != EPI_ACCUMULATE),
              "gemm_bf16: partial sums of a norm go with at most 8 rows, no gamma, and a storing epilogue");
   const NormExtras extra{emit_gamma, emit_gamma_dtype == kF32, (bf16*)emit_h, emit_ldh, emit_ss, parts, n_parts};
   if (M == 0) return 0;
   const bf16* W = (const bf16*)w;
-  if (split_ws != nullptr && M > 16 && !gamma && !emit_h && !parts) {  // more than the skinny kernels' best range
+  if (split_ws != nullptr && M > 16 && !gamma && (!emit_h || emits == 2) && !parts) {  // more than the skinny kernels' best range
     const SplitPlan plan = split_plan(M, N, K);
     if (plan.slices > 1 && (epilogue != EPI_SILU_MUL || N % 16 == 0) && (uintptr_t)split_ws % 16 == 0) {
       GB_REQUIRE((long long)plan.floats <= split_ws_floats, "gemm_bf16: the split-k workspace holds %lld floats, %zu are needed",
                  split_ws_floats, plan.floats);
       const bf16* A = (const bf16*)a;
 #define GB_SP(EPI, CT) return launch_split<EPI, CT>(A, lda, W, ldw, (CT*)c, ldc, M, N, K, split_ws, plan, stream)
-      if (epilogue == EPI_ACCUMULATE) GB_SP(EPI_ACCUMULATE, float);
+      if (epilogue == EPI_ACCUMULATE)
+        return launch_split<EPI_ACCUMULATE, float>(A, lda, W, ldw, (float*)c, ldc, M, N, K, split_ws, plan, stream, &extra, eps);
       if (epilogue == EPI_SILU_MUL && c_dtype == kBF16) GB_SP(EPI_SILU_MUL, bf16);
       if (epilogue == EPI_SILU_MUL) GB_SP(EPI_SILU_MUL, float);
       if (c_dtype == kF32) GB_SP(EPI_STORE, float);

@@ -57,6 +57,7 @@ _SIGS = {
                          C.c_longlong, _vp],
         "gb_gemm_bf16_split_floats": [_i, _i, _i],
         "gb_gemm_bf16_emit_parts": [_i, _i],
+        "gb_gemm_bf16_emit_mode": [_i, _i, _i],
         # a, lda, w, ldw, c, ldc, M, N, K, gamma, gamma_dtype, eps, parts, n_parts, cos, sin, slots, k, v,
         # nh, nkv, hd, page, stream
         "gb_gemm_bf16_rope": [_vp, _i, _vp, _i, _vp, _i, _i, _i, _i, _vp, _i, _f, _vp, _i, _vp, _vp, _vp, _vp, _vp,
@@ -269,6 +270,13 @@ def gemm_emit_parts(rows: int, n: int) -> int:
     return int(_lib("gemm_bf16").gb_gemm_bf16_emit_parts(int(rows), int(n)))
 
 
+def gemm_emit_mode(rows: int, n: int, k: int) -> int:
+    """What an accumulating bfloat16 product of these sizes can do for the RMS norm that reads the residual after
+    it: 0 nothing; 1 the operand and partial sums (``gemm(..., emit=(gamma, h, parts))``, see ``gemm_emit_parts``);
+    2 the whole norm (``gemm(..., emit=(gamma, h, eps), workspace=...)``: h receives the normed rows)."""
+    return int(_lib("gemm_bf16").gb_gemm_bf16_emit_mode(int(rows), int(n), int(k)))
+
+
 def gemm_split_floats(rows: int, n: int, k: int) -> int:
     """Floats of workspace with which a bfloat16 product of these sizes would divide k over workgroups
     (``gemm(..., workspace=)``); 0 if it would not: only products with few tiles do."""
@@ -287,9 +295,11 @@ def gemm(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor, accumulate: bool =
     silu(a . gate_j) * (a . up_j), of half as many columns.
     ``rms=(gamma, eps)`` (bfloat16 w and out, at most 64 rows): a is the float32 residual and the
     product is that of its RMS-normed rows, the norm computed inside the product's kernel.
-    ``emit=(gamma, h, parts)`` (accumulating bfloat16 product with ``gemm_emit_parts(M, N) > 0``): besides
+    ``emit=(gamma, h, parts)`` (accumulating bfloat16 product with ``gemm_emit_mode(M, N, K) == 1``): besides
     the new residual r in out, h[m, n] = bf16(gamma[n] r[m, n]) and float32 parts[tile, m] (8 columns a
     tile) of sum(r^2) are written: the work of the RMS norm that reads the residual next.
+    ``emit=(gamma, h, eps)`` with a number as the third entry (``gemm_emit_mode(M, N, K) == 2``, with the
+    workspace): h receives the rows of that norm itself, gamma * r / sqrt(mean(r^2) + eps).
     ``rms_parts=(parts, n_parts, eps)`` (at most 8 rows): a is such an h, and the product is scaled by
     1 / sqrt(sum(parts[:, m]) / K + eps) to that of the normed rows.
     ``workspace`` (float32, at least ``gemm_split_floats(M, N, K)`` elements): lets a bfloat16 product of
@@ -330,7 +340,15 @@ def gemm(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor, accumulate: bool =
         e_gamma = e_h = e_ss = parts = None
         e_ldh = n_parts = 0
         eps = 0.0
-        if emit is not None:
+        if emit is not None and not isinstance(emit[2], torch.Tensor):
+            e_gamma, e_h, eps = emit
+            _dev(e_gamma, e_h)
+            if (not accumulate or workspace is None or gemm_emit_mode(M, N, K) != 2 or e_gamma.numel() != N
+                    or not e_gamma.is_contiguous() or e_h.dtype != torch.bfloat16 or e_h.shape != (M, N)):
+                raise KernelError("gemm: the whole norm can be emitted by an accumulating product that divides k "
+                                  "(gemm_emit_mode 2, with its workspace), given gamma of N entries and a bfloat16 [M, N] buffer")
+            e_ldh = _rows(e_h, "emit h")
+        elif emit is not None:
             e_gamma, e_h, e_ss = emit
             _dev(e_gamma, e_h, e_ss)
             want = gemm_emit_parts(M, N)

@@ -92,7 +92,7 @@ class PagedAttention(Mixer):
             self.position.apply_and_store(ctx, qkv, self.n_heads, n_kv, self.head_dim, *store)
         att = ctx.buffer("att", (n, self.q_dim), ctx.dtype)
         ctx.attention(qkv[:, :self.q_dim], att, cache, self.n_heads, self.scale, self.window)
-        target, handed_on = emit_target(ctx, n, self.width, emit, "mixer")
+        target, handed_on = emit_target(ctx, n, self.width, self.q_dim, emit, "mixer")
         ops.gemm(att, self.wo, residual, accumulate=True, emit=target,
                  workspace=split_workspace(ctx, n, self.width, self.q_dim))
         return handed_on

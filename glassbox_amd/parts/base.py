@@ -25,7 +25,8 @@ Optional, for steps of few rows (each part says by a class attribute whether it 
   ``accepts_fused_norm``: forward(..., norm=) takes the un-normed residual and either the norm's
       ``(gamma, eps)`` or a ``PreNormed`` and lets its first product do the norm's work;
   ``accepts_emit_norm``: forward(..., emit=(gamma, eps)) may let its last product, which adds into the
-      residual, prepare the norm that reads the residual next, and returns a ``PreNormed`` if it did.
+      residual, prepare the norm that reads the residual next, and returns a ``PreNormed`` if it did, or a
+      ``Normed`` if it did all of it (the block then hands those rows on in the norm's place).
 """
 from __future__ import annotations
 
@@ -120,6 +121,11 @@ class Norm(Part):
         (the default) if the norm wants a pass of its own."""
         return None
 
+    def emit_spec(self, ctx, n: int):
+        """What the part before needs to prepare this norm, or to do it, where it makes the residual, or None
+        (the default)."""
+        return None
+
 
 class PositionEncoding(Part):
     def apply_and_store(self, ctx, qkv, n_heads, n_kv_heads, head_dim, slots, k_pages, v_pages) -> None:
@@ -146,20 +152,31 @@ class PreNormed(NamedTuple):
         return (self.parts, self.n_parts, self.eps)
 
 
-def emit_target(ctx, n: int, width: int, emit, tag: str):
-    """Buffers for a product of n rows and ``width`` columns that is asked (``emit=(gamma, eps)``) to prepare
-    the next norm: ``(gemm emit argument, PreNormed to hand on)``, or ``(None, None)`` when nothing is asked
-    or this step's product cannot do it (more than 8 rows, a 32-bit step, too wide a residual)."""
+class Normed(NamedTuple):
+    """The rows of an RMS norm, computed by the product that made the residual (in the pass that adds its slices
+    of k): whoever would have called the norm takes ``rows`` instead."""
+    rows: torch.Tensor
+
+
+def emit_target(ctx, n: int, width: int, in_features: int, emit, tag: str):
+    """Buffers for a product of n rows, ``width`` columns and ``in_features`` of k that is asked
+    (``emit=(gamma, eps)``) to prepare the next norm: ``(gemm emit argument, PreNormed or Normed to hand on)``, or
+    ``(None, None)`` when nothing is asked or this step's product cannot do it (a 32-bit step, sizes that neither
+    the folded kernel nor a product that divides k takes)."""
     from .. import ops
     if emit is None or ctx.dtype != torch.bfloat16 or not ctx.fuse_norms:
         return None, None
-    n_parts = ops.gemm_emit_parts(n, width)
-    if n_parts == 0:
-        return None, None
+    mode = ops.gemm_emit_mode(n, width, in_features)
     gamma, eps = emit
-    rows = ctx.buffer(f"prenorm_rows_{tag}", (n, width), torch.bfloat16)
-    parts = ctx.buffer(f"prenorm_parts_{tag}", (n_parts, 8), torch.float32)
-    return (gamma, rows, parts), PreNormed(rows, parts, n_parts, float(eps))
+    if mode == 1:
+        n_parts = ops.gemm_emit_parts(n, width)
+        rows = ctx.buffer(f"prenorm_rows_{tag}", (n, width), torch.bfloat16)
+        parts = ctx.buffer(f"prenorm_parts_{tag}", (n_parts, 8), torch.float32)
+        return (gamma, rows, parts), PreNormed(rows, parts, n_parts, float(eps))
+    if mode == 2:
+        rows = ctx.buffer(f"normed_rows_{tag}", (n, width), torch.bfloat16)
+        return (gamma, rows, float(eps)), Normed(rows)
+    return None, None
 
 
 def split_workspace(ctx, n: int, out_features: int, in_features: int):

@@ -33,7 +33,7 @@ class SwiGLU(FeedForward):
     def forward(self, ctx, h, residual, norm=None, emit=None):
         """``norm=(gamma, eps)``: h is the un-normed float32 residual and the first product norms it;
         ``norm=PreNormed``: the product before has done most of that.  ``emit=(gamma, eps)``: the down
-        projection may prepare the norm that reads the residual next (returns a PreNormed if it did)."""
+        projection may prepare the norm that reads the residual next (returns a PreNormed or Normed if it did)."""
         n = h.shape[0]
         act = ctx.buffer("act", (n, self.intermediate), ctx.dtype)
         if isinstance(norm, PreNormed):
@@ -50,7 +50,7 @@ class SwiGLU(FeedForward):
             gate_up = ctx.buffer("gate_up", (n, 2 * self.intermediate), ctx.dtype)
             ops.gemm(h, self.w_gate_up, gate_up)
             ops.silu_mul(gate_up, act)
-        target, handed_on = emit_target(ctx, n, self.width, emit, "ffn")
+        target, handed_on = emit_target(ctx, n, self.width, self.intermediate, emit, "ffn")
         ops.gemm(act, self.w_down, residual, accumulate=True, emit=target,
                  workspace=split_workspace(ctx, n, self.width, self.intermediate))
         return handed_on

@@ -30,6 +30,12 @@ class RMSNorm(Norm):
         ops.rmsnorm(x, self.weight, self.eps, out, rows)
         return out
 
+    def emit_spec(self, ctx, n: int) -> Optional[Tuple[torch.Tensor, float]]:
+        """(gamma, eps) if the product that makes the residual may prepare or do this norm (bfloat16 steps)."""
+        if ctx.dtype == torch.bfloat16 and ctx.fuse_norms:
+            return (self.weight, self.eps)
+        return None
+
     def fuse_spec(self, ctx, n: int) -> Optional[Tuple[torch.Tensor, float]]:
         """(gamma, eps) if the next matrix product may compute this norm itself: bfloat16 steps of
         few rows, where a pass of its own costs more than the norm's arithmetic."""

@@ -185,6 +185,36 @@ def test_gemm_bf16_prepares_the_next_norm(M, N, K, N2, silu, gamma_dtype):
     assert ((out.float() - again.float()).abs() <= 2 ** -6 * (1 + again.float().abs())).all()
 
 
+@pytest.mark.parametrize("M,N,K", [(2048, 2048, 8192), (128, 2048, 2048), (40, 1008, 4104), (300, 960, 2560), (64, 2048, 8192)])
+@pytest.mark.parametrize("gamma_dtype", [torch.float32, torch.bfloat16])
+def test_gemm_bf16_that_divides_k_does_the_next_norm(M, N, K, gamma_dtype):
+    """An accumulating product that divides k over workgroups adds its slices row by row, and with a row in hand
+    writes the RMS norm of the new residual too: the rows the norm's own kernel would give."""
+    from glassbox_amd import ops
+    assert ops.gemm_emit_mode(M, N, K) == 2 and ops.gemm_emit_mode(4, N, K) != 2
+    a, w = (rnd(M, K, seed=21) * 0.5).bfloat16(), (rnd(N, K, seed=22) * 0.1).bfloat16()
+    res0, g = rnd(M, N, seed=23).float(), (rnd(N, seed=24) * 0.3 + 1).to(gamma_dtype)
+    eps = 1e-5
+    ws = torch.empty(ops.gemm_split_floats(M, N, K), device=DEV)
+    res, h = to_dev(res0.clone()), torch.full((M, N), 9.0, device=DEV, dtype=torch.bfloat16)
+    ops.gemm(to_dev(a), to_dev(w), res, accumulate=True, emit=(to_dev(g), h, eps), workspace=ws)
+    want_res = res0.double() + a.double() @ w.double().T
+    assert (res.cpu().double() - want_res).abs().max().item() <= 1e-4 * math.sqrt(K)
+    # the residual is the same as without the norm, bit for bit; the rows are those of the norm's kernel but for
+    # the order of its sum (a unit in the last place of bfloat16 at most)
+    plain = to_dev(res0.clone())
+    ops.gemm(to_dev(a), to_dev(w), plain, accumulate=True, workspace=ws)
+    assert torch.equal(res, plain)
+    normed = torch.empty_like(h)
+    ops.rmsnorm(res, to_dev(g), eps, normed)
+    assert ((h.float() - normed.float()).abs() <= 2 ** -7 * normed.float().abs() + 1e-6).all()
+    x = res.cpu().double()
+    want = g.double() * x / torch.sqrt((x * x).mean(-1, keepdim=True) + eps)
+    assert (h.cpu().double() - want).abs().max().item() <= 2 ** -8 * want.abs().max().item() + 1e-6
+    with pytest.raises(ops.KernelError, match="norm"):
+        ops.gemm(to_dev(a), to_dev(w), res, accumulate=True, emit=(to_dev(g), h, eps))       # no workspace
+
+
 @pytest.mark.parametrize("M,N,K", [(17, 96, 4096), (33, 2048, 2048), (64, 2048, 8192), (64, 6144, 2048), (100, 2048, 4160),
                                    (200, 528, 8200), (64, 16384, 2048), (40, 1008, 4104), (512, 2048, 8192),
                                    # a thousand rows and more: slices of k through the 256 x 256 tiles
