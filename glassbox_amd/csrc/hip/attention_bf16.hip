@@ -12,7 +12,7 @@
 //                                             probabilities, taken from the score registers as they
 //                                             are (the k order of both operands is permuted alike)
 // so neither scores nor probabilities pass through LDS, and keys and values go from memory into
-// MFMA operands directly.  Pages: keys [page][kv head][slot][hd], values [page][kv head][hd][slot].
+// MFMA operands directly.  Pages: keys [page][kv head][hd / 8][slot][8], values [page][kv head][hd][slot].
 // A prompt portion's columns are 32 or 64 consecutive tokens of one query head, with the same
 // scheme on the 32x32x16 instruction (described at its kernel).
 //
@@ -73,11 +73,12 @@ __device__ __forceinline__ void attend64(Running<HD>& st, const bf16x8* qf, cons
     const int kc = min(max(kt, tlo), thi);
     const int page = table[kc / P];
     const int slot0 = kc % P;
-    const bf16* kb = kp + (((size_t)page * nkv + kvh) * P + slot0 + j) * HD;
+    // pieces of 8 dimensions, of each the page's slots side by side (key_piece()): the 16 lanes of a group read 256 bytes
+    const bf16* kb = kp + ((size_t)page * nkv + kvh) * P * HD + (slot0 + j) * 8;
 #pragma unroll
     for (int ks = 0; ks < KS; ++ks) {
       const int d0 = ks * 32 + c * 8;
-      kf[t][ks] = d0 < HD ? load8(kb + d0) : zero8();
+      kf[t][ks] = d0 < HD ? load8(kb + (size_t)(ks * 4 + c) * P * 8) : zero8();
     }
     const bf16* vb = vp + ((size_t)page * nkv + kvh) * HD * P + slot0 + 4 * c;
 #pragma unroll
@@ -307,16 +308,18 @@ __device__ __forceinline__ void load_keys(bf16x8 (&kf)[T][HD / 16], const PageSo
   // row r of a group of 16 rows of the score tile takes key 8*((r>>2)&1) + 4*(r>>3) + (r&3) of the group:
   // the probabilities a lane then holds for a value product are those of 8 neighbouring keys
   const int r16 = col & 15, key16 = ((r16 >> 2) & 1) * 8 + (r16 >> 3) * 4 + (r16 & 3);
-  const int mine = key16 * HD + 8 * g;
+  // a key's dimensions lie in pieces of 8, of each piece the page's slots side by side (key_piece()): this lane's
+  // piece of MFMA step ks is number 2 ks + g, and the lanes of a group of 16 keys read 256 bytes in a row
+  const int mine = ((g << src.shift) + key16) * 8;
 #pragma unroll
   for (int t = 0; t < T; ++t) {
     int s0, s1;  // a tile of 32 keys is two groups of 16, each within one page
     const size_t p0 = src.page_of(kbase + 32 * t, &s0), p1 = src.page_of(kbase + 32 * t + 16, &s1);
-    const bf16* b0 = src.kp + ((p0 << src.shift) + s0) * HD;
-    const bf16* b1 = src.kp + ((p1 << src.shift) + s1) * HD;
+    const bf16* b0 = src.kp + (p0 << src.shift) * HD + s0 * 8;
+    const bf16* b1 = src.kp + (p1 << src.shift) * HD + s1 * 8;
     const bf16* kb = ((col & 16) ? b1 : b0) + mine;
 #pragma unroll
-    for (int ks = 0; ks < HD / 16; ++ks) kf[t][ks] = load8(kb + 16 * ks);
+    for (int ks = 0; ks < HD / 16; ++ks) kf[t][ks] = load8(kb + ((size_t)(16 * ks) << src.shift));
   }
 }
 

@@ -34,6 +34,7 @@ __global__ __launch_bounds__(kChunk) void attention_plain_kernel(
   const int32_t* table = tables + (size_t)tok_seq[t] * table_stride;
   const int lo = window > 0 ? max(0, pos - window + 1) : 0;
   const int tid = threadIdx.x;
+  const int piece = key_piece(hd);
 
   for (int d = tid; d < hd; d += kChunk) qs[d] = to_f(q[(size_t)t * q_stride + (size_t)h * hd + d]);
   __syncthreads();
@@ -44,9 +45,12 @@ __global__ __launch_bounds__(kChunk) void attention_plain_kernel(
     float s = -INFINITY;
     if (p <= pos) {
       const int page = table[p / page_size];
-      const T* kr = k_pages + (((size_t)page * nkv + kvh) * page_size + p % page_size) * hd;
+      const T* kb = k_pages + ((size_t)page * nkv + kvh) * page_size * hd;  // pieces of the head size, see key_piece()
       float dot = 0.f;
-      for (int d = 0; d < hd; ++d) dot = fmaf(qs[d], to_f(kr[d]), dot);
+      for (int d0 = 0; d0 < hd; d0 += piece) {
+        const T* kr = kb + key_offset(p % page_size, d0, page_size, piece);
+        for (int e = 0; e < piece; ++e) dot = fmaf(qs[d0 + e], to_f(kr[e]), dot);
+      }
       s = dot * scale;
     }
     const float cm = block_max(s, scratch);

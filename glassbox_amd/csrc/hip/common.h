@@ -25,6 +25,16 @@ constexpr int kWave = 64;
 // dtype codes shared with the Python side
 enum : int { kF32 = 0, kBF16 = 1 };
 
+// Key pages.  The block of one (page, kv head) holds the head's dimensions in pieces of key_piece(hd) elements
+// (8 for every head size that is a multiple of 8), and of each piece the page's slots side by side:
+// [hd / piece][slot in page][piece].  Lanes that take neighbouring keys for an MFMA operand then read
+// neighbouring addresses, which the memory pipeline takes three times as fast as neighbours a whole key apart.
+__host__ __device__ __forceinline__ int key_piece(int hd) { return hd % 8 == 0 ? 8 : hd % 4 == 0 ? 4 : hd % 2 == 0 ? 2 : 1; }
+// offset of dimension d of the key in `slot` inside its (page, kv head) block
+__device__ __forceinline__ int key_offset(int slot, int d, int page_size, int piece) {
+  return ((d / piece) * page_size + slot) * piece + d % piece;
+}
+
 __device__ __forceinline__ float to_f(float v) { return v; }
 __device__ __forceinline__ float to_f(bf16 v) { return (float)v; }
 template <typename T> __device__ __forceinline__ T from_f(float v);

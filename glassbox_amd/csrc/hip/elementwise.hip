@@ -123,9 +123,9 @@ extern "C" int gb_rope_table(const int32_t* pos, const float* inv, float* cosv, 
 // For token t: every query head and key head is rotated in half-split pairs (i, i + hd/2):
 //   x0' = x0 c - x1 s ; x1' = x1 c + x0 s                              (model.rs:110-113)
 // queries are rotated in place inside the stacked qkv row; rotated keys and plain values go to
-// the pages at slot[t] (model.rs:273-275).  Key pages are [page][kv head][slot in page][hd]; value
-// pages are transposed, [page][kv head][hd][slot in page], so that the attention kernels find
-// consecutive keys of one value dimension side by side (the matrix cores' operand layout).
+// the pages at slot[t] (model.rs:273-275).  Key pages are [page][kv head][hd / piece][slot in page][piece]
+// (see key_piece()); value pages are transposed, [page][kv head][hd][slot in page], so that the attention
+// kernels find consecutive keys of one value dimension side by side (the matrix cores' operand layout).
 // With slots == nullptr nothing is stored (a layer that reads another layer's cache).
 // With nkv == 0 the row holds queries only.
 template <typename T>
@@ -140,6 +140,7 @@ __global__ void rope_store_scalar_kernel(T* __restrict__ qkv, int row_stride, co
   const float* s = sinv + (size_t)t * half;
   const int slot = slots ? slots[t] : -1;
   const int page = slot >= 0 ? slot / page_size : 0, off = slot >= 0 ? slot % page_size : 0;
+  const int piece = key_piece(hd);
   // queries, then keys: (nh + nkv) heads of `half` pairs
   const int pairs = (nh + nkv) * half;
   // eight pairs a thread at a time: all loads first, so that they are in flight together (the
@@ -170,9 +171,9 @@ __global__ void rope_store_scalar_kernel(T* __restrict__ qkv, int row_stride, co
         h[i] = y0;  // rotated keys stay in the row too: parts may read them back
         h[i + half] = y1;
         if (head >= nh && slot >= 0) {
-          T* dst = k_pages + (((size_t)page * nkv + (head - nh)) * page_size + off) * hd;
-          dst[i] = y0;
-          dst[i + half] = y1;
+          T* dst = k_pages + ((size_t)page * nkv + (head - nh)) * page_size * hd;
+          dst[key_offset(off, i, page_size, piece)] = y0;
+          dst[key_offset(off, i + half, page_size, piece)] = y1;
         }
       }
     }
@@ -212,6 +213,7 @@ __global__ void rope_store_kernel(T* __restrict__ qkv, int row_stride, const flo
   const bool is_v = unit >= nh + nkv, is_k = unit >= nh && !is_v;
   const int slot = (slots && unit >= nh) ? slots[t] : -1;
   const int page = slot >= 0 ? slot / page_size : 0, off = slot >= 0 ? slot % page_size : 0;
+  const int piece = key_piece(hd);
   for (int j = (lane & 15) * 2; j < half; j += 32) {
     const P x0 = *reinterpret_cast<const P*>(head + j), x1 = *reinterpret_cast<const P*>(head + half + j);
     P y0 = x0, y1 = x1;
@@ -227,9 +229,10 @@ __global__ void rope_store_kernel(T* __restrict__ qkv, int row_stride, const flo
     }
     if (slot < 0) continue;
     if (is_k) {
-      T* dst = k_pages + (((size_t)page * nkv + (unit - nh)) * page_size + off) * hd;
-      *reinterpret_cast<P*>(dst + j) = y0;
-      *reinterpret_cast<P*>(dst + half + j) = y1;
+      // j is even and the pieces hold 4 or 8 elements here: a pair stays inside its piece
+      T* dst = k_pages + ((size_t)page * nkv + (unit - nh)) * page_size * hd;
+      *reinterpret_cast<P*>(dst + key_offset(off, j, page_size, piece)) = y0;
+      *reinterpret_cast<P*>(dst + key_offset(off, half + j, page_size, piece)) = y1;
     } else if (is_v) {
       T* dst = v_pages + ((size_t)page * nkv + (unit - nh - nkv)) * hd * page_size + off;
       dst[(size_t)j * page_size] = x0.a;

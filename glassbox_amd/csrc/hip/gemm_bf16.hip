@@ -57,7 +57,7 @@ struct NormExtras {
 // and nkv value heads of hd rows each.  The product rotates query and key heads by the angles of each
 // row's position (pairs (i, i + hd/2), crates/glassbox-core/src/model.rs:102-115) while the sums are
 // still 32-bit, writes the stacked rows to C as usual, and the key and value heads straight into the
-// cache pages at slots[m] (keys [page][kv head][slot][hd], values [page][kv head][hd][slot]) if slots is
+// cache pages at slots[m] (keys [page][kv head][hd / 8][slot][8], values [page][kv head][hd][slot]) if slots is
 // given: the rotation kernel and its round trip through memory are not needed.
 struct RopeExtras {
   const float* cosv;   // [M][hd/2], nullptr: no rotation
@@ -932,7 +932,8 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_skinny_kernel(const void* __r
         if (rope.slots != nullptr && head >= rope.nh) {
           const int slot = rope.slots[m], page = slot / rope.page_size, off = slot % rope.page_size;
           if (is_key)
-            rope.k_pages[(((size_t)page * rope.nkv + (head - rope.nh)) * rope.page_size + off) * rope.hd + dim] = yb;
+            rope.k_pages[((size_t)page * rope.nkv + (head - rope.nh)) * rope.page_size * rope.hd +
+                         key_offset(off, dim, rope.page_size, 8)] = yb;  // hd is a multiple of 16: pieces of 8
           else
             rope.v_pages[(((size_t)page * rope.nkv + (head - rope.nh - rope.nkv)) * rope.hd + dim) * rope.page_size + off] = yb;
         }

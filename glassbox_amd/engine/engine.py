@@ -72,7 +72,7 @@ class Engine:
                 lc.group = keys.index(spec.group_key)
                 # one page and one state slot more than the manager hands out: filler rows of a replayed step
                 # write there (engine.decode_graphs)
-                shape = (num_pages + 1, spec.num_kv_heads, self.page_size, spec.head_dim)
+                shape = ops.key_pages_shape(num_pages + 1, spec.num_kv_heads, self.page_size, spec.head_dim)
                 lc.k_pages = torch.zeros(shape, dtype=self.dtype, device=self.device)
                 lc.v_pages = torch.zeros((num_pages + 1, spec.num_kv_heads, spec.head_dim, self.page_size),
                                          dtype=self.dtype, device=self.device)   # transposed: see ops._check_pages

@@ -141,17 +141,48 @@ def _i32(t: Optional[torch.Tensor], what: str, n: Optional[int] = None) -> None:
         raise KernelError(f"{what} holds {t.numel()} entries, {n} are needed")
 
 
-def _check_pages(k_pages, v_pages, dtype, what: str) -> None:
-    """Key pages [pages, kv heads, page size, head size]; value pages transposed [pages, kv heads, head size,
-    page size]; both contiguous and of the activations' type."""
-    if k_pages is None or v_pages is None or k_pages.dim() != 4 or v_pages.dim() != 4:
-        raise KernelError(f"{what}: key and value pages must be 4-d tensors")
-    p, h, s, d = k_pages.shape
+def key_piece(head_dim: int) -> int:
+    """Elements of one piece of a key in its page: 8 for head sizes that are a multiple of 8."""
+    return 8 if head_dim % 8 == 0 else 4 if head_dim % 4 == 0 else 2 if head_dim % 2 == 0 else 1
+
+
+def key_pages_shape(pages: int, n_kv_heads: int, page_size: int, head_dim: int) -> tuple:
+    """Key pages hold a head's dimensions in pieces, and of each piece the page's slots side by side:
+    [pages, kv heads, head size / piece, page size, piece].  The lanes that take neighbouring keys for a
+    matrix-core operand then read neighbouring addresses."""
+    piece = key_piece(head_dim)
+    return (pages, n_kv_heads, head_dim // piece, page_size, piece)
+
+
+def pack_keys(keys: torch.Tensor) -> torch.Tensor:
+    """[pages, kv heads, page size, head size] to the layout of key pages."""
+    p, h, s, d = keys.shape
+    piece = key_piece(d)
+    return keys.reshape(p, h, s, d // piece, piece).permute(0, 1, 3, 2, 4).contiguous()
+
+
+def unpack_keys(k_pages: torch.Tensor) -> torch.Tensor:
+    """Key pages to [pages, kv heads, page size, head size]."""
+    p, h, n, s, piece = k_pages.shape
+    return k_pages.permute(0, 1, 3, 2, 4).reshape(p, h, s, n * piece)
+
+
+def _check_pages(k_pages, v_pages, dtype, what: str):
+    """Key pages as ``key_pages_shape`` says; value pages transposed, [pages, kv heads, head size, page size];
+    both contiguous and of the activations' type.  Returns (pages, kv heads, page size, head size)."""
+    if k_pages is None or v_pages is None or k_pages.dim() != 5 or v_pages.dim() != 4:
+        raise KernelError(f"{what}: key pages must be 5-d [pages, kv heads, head size / piece, page size, piece] "
+                          f"and value pages 4-d")
+    p, h, n, s, piece = k_pages.shape
+    d = n * piece
+    if piece != key_piece(d):
+        raise KernelError(f"{what}: key pages of head size {d} are kept in pieces of {key_piece(d)}, not {piece}")
     if tuple(v_pages.shape) != (p, h, d, s):
         raise KernelError(f"{what}: value pages must be [pages, kv heads, head size, page size] = "
                           f"{(p, h, d, s)}, got {tuple(v_pages.shape)}")
     if not k_pages.is_contiguous() or not v_pages.is_contiguous() or k_pages.dtype != dtype or v_pages.dtype != dtype:
         raise KernelError(f"{what}: pages must be contiguous and of the activations' type")
+    return p, h, s, d
 
 
 # ------------------------------------------------------------------ elementwise
@@ -211,10 +242,9 @@ def rope_store(qkv: torch.Tensor, cos: Optional[torch.Tensor], sin: Optional[tor
     page_size = 0
     if slots is not None:
         _i32(slots, "slots", n)
-        _check_pages(k_pages, v_pages, qkv.dtype, "rope_store")
-        if (k_pages.shape[1], k_pages.shape[3]) != (n_kv_heads, head_dim):
+        _, p_heads, page_size, p_hd = _check_pages(k_pages, v_pages, qkv.dtype, "rope_store")
+        if (p_heads, p_hd) != (n_kv_heads, head_dim):
             raise KernelError("rope_store: pages do not have this layer's kv heads and head size")
-        page_size = k_pages.shape[2]
     if rotate:
         if cos is None or sin is None or cos.shape != (n, head_dim // 2) and cos.shape[0] < n:
             raise KernelError("rope_store: rotation needs cos/sin tables of [n, head_dim/2]")
@@ -394,10 +424,9 @@ def gemm_rope(a: torch.Tensor, w: torch.Tensor, qkv: torch.Tensor, n_heads: int,
     page_size = 0
     if slots is not None:
         _i32(slots, "slots", M)
-        _check_pages(k_pages, v_pages, torch.bfloat16, "gemm_rope")
-        if (k_pages.shape[1], k_pages.shape[3]) != (n_kv_heads, head_dim):
+        _, p_heads, page_size, p_hd = _check_pages(k_pages, v_pages, torch.bfloat16, "gemm_rope")
+        if (p_heads, p_hd) != (n_kv_heads, head_dim):
             raise KernelError("gemm_rope: pages do not have this layer's kv heads and head size")
-        page_size = k_pages.shape[2]
     if cos is not None:
         if sin is None or cos.shape[1] != head_dim // 2 or cos.shape[0] < M or cos.dtype != torch.float32 \
                 or not cos.is_contiguous() or not sin.is_contiguous() or sin.shape != cos.shape:
@@ -427,12 +456,11 @@ def attention_plain(q: torch.Tensor, out: torch.Tensor, positions: torch.Tensor,
     """Paged attention, one block per (token, head); q may be a view into the stacked qkv rows."""
     _dev(q, out, positions, tok_seq, tables, k_pages, v_pages)
     n = q.shape[0]
-    _, nkv, page_size, hd = k_pages.shape
-    if q.shape[1] != n_heads * hd or out.shape != (n, n_heads * hd):
-        raise KernelError("attention: q and out must be [n, heads * head size]")
     if q.dtype != out.dtype:
         raise KernelError("attention: q and out must share one element type")
-    _check_pages(k_pages, v_pages, q.dtype, "attention")
+    _, nkv, page_size, hd = _check_pages(k_pages, v_pages, q.dtype, "attention")
+    if q.shape[1] != n_heads * hd or out.shape != (n, n_heads * hd):
+        raise KernelError("attention: q and out must be [n, heads * head size]")
     _i32(positions, "positions", n)
     _i32(tok_seq, "tok_seq", n)
     if tables.dtype != torch.int32 or tables.dim() != 2 or tables.stride(1) != 1:
@@ -446,7 +474,8 @@ def attention_plain(q: torch.Tensor, out: torch.Tensor, positions: torch.Tensor,
 def tuned_attention_supports(k_pages: torch.Tensor, n_heads: int, window: int) -> bool:
     """Whether the matrix-core attention kernels take this layer: bfloat16 pages, a head size that is
     a multiple of 16 up to 128, at most 16 query heads per kv head, pages of 16, 32, 64 ... keys."""
-    _, nkv, page, hd = k_pages.shape
+    _, nkv, n_pieces, page, piece = k_pages.shape
+    hd = n_pieces * piece
     return (k_pages.dtype == torch.bfloat16 and hd % 16 == 0 and 16 <= hd <= 128 and n_heads % nkv == 0
             and n_heads // nkv <= 16 and page >= 16 and page & (page - 1) == 0)
 
@@ -466,8 +495,7 @@ def attention_decode(q: torch.Tensor, out: torch.Tensor, ctx, cache, n_heads: in
     n_dec = ctx.host["n_decode"]
     k_pages, v_pages = cache.k_pages, cache.v_pages
     _dev(q, out, k_pages, v_pages)
-    _check_pages(k_pages, v_pages, torch.bfloat16, "attention_decode")
-    _, nkv, page, hd = k_pages.shape
+    _, nkv, page, hd = _check_pages(k_pages, v_pages, torch.bfloat16, "attention_decode")
     if q.dtype != torch.bfloat16 or out.dtype != torch.bfloat16 or q.shape[1] != n_heads * hd:
         raise KernelError("attention_decode: q and out must be bfloat16 [n, heads * head size]")
     tables = ctx.tables[cache.group]
@@ -488,8 +516,7 @@ def attention_prefill(q: torch.Tensor, out: torch.Tensor, ctx, cache, n_heads: i
     n_dec, S = ctx.host["n_decode"], ctx.num_seqs
     k_pages, v_pages = cache.k_pages, cache.v_pages
     _dev(q, out, k_pages, v_pages)
-    _check_pages(k_pages, v_pages, torch.bfloat16, "attention_prefill")
-    _, nkv, page, hd = k_pages.shape
+    _, nkv, page, hd = _check_pages(k_pages, v_pages, torch.bfloat16, "attention_prefill")
     if q.dtype != torch.bfloat16 or out.dtype != torch.bfloat16 or q.shape[1] != n_heads * hd:
         raise KernelError("attention_prefill: q and out must be bfloat16 [n, heads * head size]")
     tables = ctx.tables[cache.group]

@@ -72,7 +72,7 @@ class StateSpec:
 @dataclass
 class LayerCache:
     """What the engine hands a mixer: its layer's pages, the index of their page group, its state."""
-    k_pages: Optional[torch.Tensor] = None   # [pages, kv heads, page size, head size]
+    k_pages: Optional[torch.Tensor] = None   # [pages, kv heads, head size / piece, page size, piece] (ops.key_pages_shape)
     v_pages: Optional[torch.Tensor] = None   # [pages, kv heads, head size, page size] (transposed)
     group: int = 0
     state: Optional[torch.Tensor] = None     # [slots, *state shape]

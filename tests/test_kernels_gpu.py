@@ -343,7 +343,7 @@ def test_rope_table_and_rotation(hd, theta):
     assert np.abs(cos.cpu().numpy() - c_want).max() < 1e-7 and np.abs(sin.cpu().numpy() - s_want).max() < 1e-7
     qkv = rnd(n, (nh + 2 * nkv) * hd, seed=3)
     page = 16
-    k_pages = torch.zeros(4, nkv, page, hd, device=DEV)
+    k_pages = torch.zeros(ops.key_pages_shape(4, nkv, page, hd), device=DEV)
     v_pages = torch.zeros(4, nkv, hd, page, device=DEV)
     slots = torch.tensor([3, 16 + 15, 32, 0, 63], dtype=torch.int32, device=DEV)
     buf = to_dev(qkv.clone())
@@ -354,7 +354,7 @@ def test_rope_table_and_rotation(hd, theta):
     assert (got_q - q_want).abs().max().item() < 1e-5
     assert torch.equal(got_q[0], qkv[0, :nh * hd].double().reshape(nh, hd)), "position 0 must leave the vector as it is"
     for i, s in enumerate(slots.tolist()):
-        got_k = k_pages[s // page, :, s % page, :].cpu().double()
+        got_k = ops.unpack_keys(k_pages)[s // page, :, s % page, :].cpu().double()
         got_v = v_pages[s // page, :, :, s % page].cpu()
         assert (got_k - k_want[i]).abs().max().item() < 1e-5
         assert torch.equal(got_v, qkv[i, (nh + nkv) * hd:].reshape(nkv, hd))
@@ -393,7 +393,7 @@ def test_gemm_bf16_rotates_and_writes_the_cache(M, nh, nkv, hd, K, normed):
     prod = h64 @ w.double().T
     q_want = llama.rope(prod[:, :nh * hd].reshape(M, nh, hd), pos, theta).reshape(M, nh * hd)
     store = nkv > 0
-    k_pages = torch.zeros(4, max(nkv, 1), page, hd, device=DEV, dtype=torch.bfloat16)
+    k_pages = torch.zeros(ops.key_pages_shape(4, max(nkv, 1), page, hd), device=DEV, dtype=torch.bfloat16)
     v_pages = torch.zeros(4, max(nkv, 1), hd, page, device=DEV, dtype=torch.bfloat16)
     qkv = torch.full((M, N), 9.0, device=DEV, dtype=torch.bfloat16)
     ops.gemm_rope(a_dev, to_dev(w), qkv, nh, nkv, hd, cos, sin, to_dev(slots) if store else None,
@@ -404,10 +404,11 @@ def test_gemm_bf16_rotates_and_writes_the_cache(M, nh, nkv, hd, K, normed):
         k_want = llama.rope(prod[:, nh * hd:(nh + nkv) * hd].reshape(M, nkv, hd), pos, theta)
         v_want = prod[:, (nh + nkv) * hd:].reshape(M, nkv, hd)
         for i, sl in enumerate(slots.tolist()):
-            assert (k_pages[sl // page, :, sl % page, :].cpu().double() - k_want[i]).abs().max().item() <= tol
+            assert (ops.unpack_keys(k_pages)[sl // page, :, sl % page, :].cpu().double() - k_want[i]).abs().max().item() <= tol
             assert (v_pages[sl // page, :, :, sl % page].cpu().double() - v_want[i]).abs().max().item() <= tol
         # the rows hold what the pages hold
-        assert torch.equal(qkv[0, nh * hd:(nh + nkv) * hd].reshape(nkv, hd), k_pages[slots[0] // page, :, slots[0] % page, :])
+        assert torch.equal(qkv[0, nh * hd:(nh + nkv) * hd].reshape(nkv, hd),
+                           ops.unpack_keys(k_pages)[slots[0] // page, :, slots[0] % page, :])
         # the two kernels it replaces round once more (the product to bfloat16 before the rotation)
         two = torch.empty_like(qkv)
         ops.gemm(a_dev, to_dev(w), two, rms=rms)
@@ -442,7 +443,7 @@ def test_rope_store_writes_values_of_portions_in_tiles(dtype, hd, page):
     cos, sin = torch.rand(n, hd // 2, device=DEV), torch.rand(n, hd // 2, device=DEV)
     results = []
     for portions in (None, (n_dec, i32(q_start), i32(q_lens), i32(pos0), n_dec, len(q_lens) - n_dec, max(q_lens))):
-        k_pages = torch.zeros(next_page, nkv, page, hd, device=DEV, dtype=dtype)
+        k_pages = torch.zeros(ops.key_pages_shape(next_page, nkv, page, hd), device=DEV, dtype=dtype)
         v_pages = torch.zeros(next_page, nkv, hd, page, device=DEV, dtype=dtype)
         buf = to_dev(qkv.clone())
         ops.rope_store(buf, cos, sin, i32(slots), k_pages, v_pages, nh, nkv, hd, portions=portions)
@@ -508,7 +509,7 @@ def test_attention_plain_kernel(dtype, nh, nkv, hd, window):
     scale = 1 / math.sqrt(hd)
     out = torch.empty(n, nh * hd, device=DEV, dtype=dtype)
     ops.attention_plain(to_dev(q), out, torch.tensor(positions, dtype=torch.int32, device=DEV),
-                        torch.tensor(tok_seq, dtype=torch.int32, device=DEV), to_dev(tables), to_dev(k_pages),
+                        torch.tensor(tok_seq, dtype=torch.int32, device=DEV), to_dev(tables), to_dev(ops.pack_keys(k_pages)),
                         to_dev(v_pages), nh, scale, window)
     want = plain_attention_rows(q, ks, vs, tok_seq, positions, nh, scale, window)
     tol = 2e-5 if dtype == torch.float32 else 2 ** -7
@@ -537,7 +538,7 @@ def test_attention_finds_one_far_key(dtype):
         qq = qq.reshape(1, nh * hd).to(dtype)
         out = torch.empty(1, nh * hd, device=DEV, dtype=dtype)
         ops.attention_plain(to_dev(qq), out, torch.tensor([ctx - 1], dtype=torch.int32, device=DEV),
-                            torch.tensor([0], dtype=torch.int32, device=DEV), to_dev(tables), to_dev(kp),
+                            torch.tensor([0], dtype=torch.int32, device=DEV), to_dev(tables), to_dev(ops.pack_keys(kp)),
                             to_dev(v_pages), nh, 1 / math.sqrt(hd), 0)
         want = vs[0][target].float().repeat_interleave(2, 0).reshape(-1)
         assert (out.cpu().float()[0] - want).abs().max().item() < 2e-2, f"key at {target} was not found"
@@ -582,7 +583,7 @@ def test_tuned_attention_against_the_plain_kernel(nh, nkv, hd, window, page):
     n = sum(q_lens)
     q = (rnd(n, nh * hd, seed=11) * 0.7).bfloat16()
     scale = 1 / math.sqrt(hd)
-    cache = SimpleNamespace(k_pages=to_dev(k_pages), v_pages=to_dev(v_pages), group=0)
+    cache = SimpleNamespace(k_pages=to_dev(ops.pack_keys(k_pages)), v_pages=to_dev(v_pages), group=0)
     assert ops.tuned_attention_supports(cache.k_pages, nh, window)
     out = torch.zeros(n, nh * hd, device=DEV, dtype=torch.bfloat16)
     qd = to_dev(q)
@@ -613,7 +614,7 @@ def test_tuned_prefill_long_portions(nh, nkv, hd, window):
     n = sum(q_lens)
     q = (rnd(n, nh * hd, seed=12) * 0.7).bfloat16()
     scale = 1 / math.sqrt(hd)
-    cache = SimpleNamespace(k_pages=to_dev(k_pages), v_pages=to_dev(v_pages), group=0)
+    cache = SimpleNamespace(k_pages=to_dev(ops.pack_keys(k_pages)), v_pages=to_dev(v_pages), group=0)
     out = torch.zeros(n, nh * hd, device=DEV, dtype=torch.bfloat16)
     qd = to_dev(q)
     ops.attention_prefill(qd, out, ctx, cache, nh, scale, window)
@@ -645,7 +646,7 @@ def test_tuned_decode_with_a_workgroup_per_request_and_kv_head(nh, nkv, hd, wind
     n = len(ctx_lens)
     q = (rnd(n, nh * hd, seed=13) * 0.7).bfloat16()
     scale = 1 / math.sqrt(hd)
-    cache = SimpleNamespace(k_pages=to_dev(k_pages), v_pages=to_dev(v_pages), group=0)
+    cache = SimpleNamespace(k_pages=to_dev(ops.pack_keys(k_pages)), v_pages=to_dev(v_pages), group=0)
     out = torch.zeros(n, nh * hd, device=DEV, dtype=torch.bfloat16)
     ops.attention_decode(to_dev(q), out, ctx, cache, nh, scale, window)
     want = plain_attention_rows(q, ks, vs, ctx.tok_seq, ctx.pos_list, nh, scale, window)
@@ -670,7 +671,7 @@ def test_tuned_decode_finds_one_far_key_in_every_chunk_position():
         for max_context in (1500, 4096):                       # one and several chunks per workgroup
             ctx = BareContext([1], [ctxlen], tables, max_context=max_context)
             out = torch.zeros(1, nh * hd, device=DEV, dtype=torch.bfloat16)
-            cache = SimpleNamespace(k_pages=to_dev(kp), v_pages=to_dev(v_pages), group=0)
+            cache = SimpleNamespace(k_pages=to_dev(ops.pack_keys(kp)), v_pages=to_dev(v_pages), group=0)
             ops.attention_decode(to_dev(q), out, ctx, cache, nh, 1 / math.sqrt(hd), 0)
             want = vs[0][target].float().repeat_interleave(2, 0).reshape(-1)
             assert (out.cpu().float()[0] - want).abs().max().item() < 2e-2, f"key at {target} was not found"
@@ -690,7 +691,7 @@ def test_tuned_prefill_short_portions_over_long_contexts(nh, nkv, hd, window):
     n = sum(q_lens)
     q = (rnd(n, nh * hd, seed=14) * 0.7).bfloat16()
     scale = 1 / math.sqrt(hd)
-    cache = SimpleNamespace(k_pages=to_dev(k_pages), v_pages=to_dev(v_pages), group=0)
+    cache = SimpleNamespace(k_pages=to_dev(ops.pack_keys(k_pages)), v_pages=to_dev(v_pages), group=0)
     out = torch.zeros(n, nh * hd, device=DEV, dtype=torch.bfloat16)
     qd = to_dev(q)
     ops.attention_decode(qd, out, ctx, cache, nh, scale, window)
@@ -728,7 +729,7 @@ def test_tuned_prefill_sees_exactly_the_causal_keys(nh, ctxlen, qlen):
         kp[tables[0, p // page], :, p % page, :] = (axis * lengths[p].float()).bfloat16()
     q = (axis * 768).repeat(qlen, nh).bfloat16()             # neighbours differ by 12 and more in score
     out = torch.zeros(qlen, nh * hd, device=DEV, dtype=torch.bfloat16)
-    cache = SimpleNamespace(k_pages=to_dev(kp), v_pages=to_dev(v_pages), group=0)
+    cache = SimpleNamespace(k_pages=to_dev(ops.pack_keys(kp)), v_pages=to_dev(v_pages), group=0)
     ops.attention_prefill(to_dev(q), out, ctx, cache, nh, 1 / math.sqrt(hd), 0)
     got = out.cpu().float().reshape(qlen, nkv, nh // nkv, hd)
     want = vs[0][110:110 + qlen].float()[:, :, None, :]      # not the value of the position after it

@@ -77,7 +77,7 @@ def test_swiglu_part(model_dirs):
 @pytest.mark.parametrize("window", [0, 5])
 def test_attention_part_with_rotary(model_dirs, window):
     """The mixer alone: two requests of different length in one step, against the plain formulas."""
-    from glassbox_amd import Engine
+    from glassbox_amd import Engine, ops
     from glassbox_amd.parts.attention import PagedAttention
     from glassbox_amd.parts.base import LayerCache
     from glassbox_amd.parts.rotary import Rotary
@@ -90,7 +90,8 @@ def test_attention_part_with_rotary(model_dirs, window):
     lengths = [19, 7]
     ctx, _ = context_for(eng, lengths)
     pages = 512 // 16
-    cache = LayerCache(torch.zeros(pages, nkv, 16, hd, device=DEV), torch.zeros(pages, nkv, hd, 16, device=DEV), 0)
+    cache = LayerCache(torch.zeros(ops.key_pages_shape(pages, nkv, 16, hd), device=DEV),
+                       torch.zeros(pages, nkv, hd, 16, device=DEV), 0)
     h = rnd(sum(lengths), d, seed=5).float()
     x = torch.zeros(sum(lengths), d, device=DEV)
     part.forward(ctx, h.to(DEV), x, cache)
