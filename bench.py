@@ -45,7 +45,12 @@ def main() -> int:
     ap.add_argument("--only", choices=["decode", "prefill"], default=None,
                     help="for profiling: run only the decode steps (after their prefill) or only the 2,048-token prefill")
     ap.add_argument("--no-graph", action="store_true", help="run decode steps without HIP graph replay")
+    ap.add_argument("--prefill-tokens", type=int, default=PREFILL_TOKENS,
+                    help="with --only prefill, for profiling: a prompt of another length than the 2,048 tokens of the record")
     a = ap.parse_args()
+    if a.prefill_tokens != PREFILL_TOKENS and a.only != "prefill":
+        print("bench.py: --prefill-tokens goes with --only prefill; the record's prefill is of 2,048 tokens")
+        return 2
     if a.gpus != 1:
         print(f"bench.py: this engine runs on one GPU; --gpus {a.gpus} is not supported")
         return 2
@@ -61,7 +66,7 @@ def main() -> int:
     model = build_model(cfg)
     init_random(model, seed=0, dtype=a.dtype, device="cuda:0")
     batches = [a.batch] + ([] if a.no_points else [b for b in (1, 64) if b != a.batch])
-    max_tokens = max(batches) * (a.context + 64)
+    max_tokens = max(max(batches) * (a.context + 64), a.prefill_tokens + 64)
     eng = Engine(model, dtype=a.dtype, max_tokens=max_tokens, max_seqs=max(batches), page_size=16)
     vocab = cfg.vocab_size
     g = torch.Generator().manual_seed(1)
@@ -74,10 +79,10 @@ def main() -> int:
 
     # ---- prefill: one step of 2,048 tokens, logits for the last one
     def prefill_once(name):
-        toks = torch.randint(0, vocab, (PREFILL_TOKENS,), generator=g).tolist()
+        toks = torch.randint(0, vocab, (a.prefill_tokens,), generator=g).tolist()
         torch.cuda.synchronize()
         t0 = time.perf_counter()
-        eng.step([(name, toks, [PREFILL_TOKENS - 1])])
+        eng.step([(name, toks, [a.prefill_tokens - 1])])
         torch.cuda.synchronize()
         dt = time.perf_counter() - t0
         eng.end_request(name)
@@ -88,7 +93,7 @@ def main() -> int:
         prefill_once("warm")
         pf = min(prefill_once(f"pf{i}") for i in range(3))
     if a.only == "prefill":
-        print(json.dumps({"prefill_ms": round(pf * 1e3, 3), "tokens": PREFILL_TOKENS}))
+        print(json.dumps({"prefill_ms": round(pf * 1e3, 3), "tokens": a.prefill_tokens}))
         return 0
     T = PREFILL_TOKENS
     pf_flops = 2 * T * layer_params * L + L * 4 * qd * (T * (T + 1) // 2) + 2 * d * vocab
