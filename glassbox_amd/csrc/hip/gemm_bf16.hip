@@ -252,6 +252,24 @@ __global__ __launch_bounds__(256, WN == 2 ? 2 : 1) void gemm_tiled_kernel(const 
       }
     return;
   }
+  if constexpr (EPI == EPI_ACCUMULATE) {
+    // a wave whose tiles lie wholly inside C reads all old values of a tile before it adds: behind the checks
+    // below every read would wait for the one before it
+    if (m0 + (wm + 1) * 32 * WM <= M && blockIdx.x * BN + (wn + 1) * 32 * WN <= N) {
+#pragma unroll
+      for (int i = 0; i < WM; ++i)
+#pragma unroll
+        for (int j = 0; j < WN; ++j) {
+          CT* base = c + (size_t)(m0 + wm * 32 * WM + i * 32 + 4 * (lane / 32)) * ldc + blockIdx.x * BN + wn * 32 * WN + j * 32 + lane % 32;
+          float old[16];
+#pragma unroll
+          for (int r = 0; r < 16; ++r) old[r] = (float)base[(size_t)(8 * (r / 4) + r % 4) * ldc];
+#pragma unroll
+          for (int r = 0; r < 16; ++r) base[(size_t)(8 * (r / 4) + r % 4) * ldc] = (CT)(old[r] + acc[i][j][r]);
+        }
+      return;
+    }
+  }
 #pragma unroll
   for (int i = 0; i < WM; ++i)
 #pragma unroll
@@ -491,6 +509,25 @@ __global__ __launch_bounds__(512, 1) void gemm_ring_kernel(const bf16* __restric
         if (gm < M) c[(size_t)gm * ldc + gn] = (CT)(g / (1.0f + __expf(-g)) * u);
       }
     return;
+  }
+  if constexpr (EPI == EPI_ACCUMULATE) {
+    // as in the tiled kernel: inside C, all old values of a tile are read before any is added to
+    if (m0 + (wm + 1) * RTM * 32 <= M && blockIdx.x * RBN + (wn + 1) * RTN * 32 <= N) {
+#pragma unroll
+      for (int i = 0; i < RTM; ++i) {
+        CT* base = c + (size_t)(m0 + wm * RTM * 32 + i * 32 + 4 * (lane / 32)) * ldc + blockIdx.x * RBN + wn * RTN * 32 + lane % 32;
+        float old[RTN][16];
+#pragma unroll
+        for (int j = 0; j < RTN; ++j)
+#pragma unroll
+          for (int r = 0; r < 16; ++r) old[j][r] = (float)base[(size_t)(8 * (r / 4) + r % 4) * ldc + j * 32];
+#pragma unroll
+        for (int j = 0; j < RTN; ++j)
+#pragma unroll
+          for (int r = 0; r < 16; ++r) base[(size_t)(8 * (r / 4) + r % 4) * ldc + j * 32] = (CT)(old[j][r] + acc[i][j][r]);
+      }
+      return;
+    }
   }
 #pragma unroll
   for (int i = 0; i < RTM; ++i)
