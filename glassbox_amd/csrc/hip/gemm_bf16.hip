@@ -626,10 +626,25 @@ __global__ void splitk_reduce_kernel(const float* __restrict__ ws, int slices, C
   if (idx >= (size_t)M * groups) return;
   const int m = (int)(idx / groups), j = (int)(idx % groups) * 4;
   f32x4 sum = {0.f, 0.f, 0.f, 0.f}, up = {0.f, 0.f, 0.f, 0.f};
-  for (int z = 0; z < slices; ++z) {
-    const float* row = ws + ((size_t)z * M + m) * N;
-    sum += *reinterpret_cast<const f32x4*>(row + j);
-    if (EPI == EPI_SILU_MUL) up += *reinterpret_cast<const f32x4*>(row + N / 2 + j);
+  const size_t copy = (size_t)M * N;  // floats between one slice's copy of C and the next
+  const float* row = ws + (size_t)m * N;
+  int z = 0;
+  for (; z + 4 <= slices; z += 4) {  // four slices' loads are on their way together; the sums keep the order of z
+    f32x4 v[4], u[4];
+#pragma unroll
+    for (int t = 0; t < 4; ++t) {
+      v[t] = *reinterpret_cast<const f32x4*>(row + (z + t) * copy + j);
+      if (EPI == EPI_SILU_MUL) u[t] = *reinterpret_cast<const f32x4*>(row + (z + t) * copy + N / 2 + j);
+    }
+#pragma unroll
+    for (int t = 0; t < 4; ++t) {
+      sum += v[t];
+      if (EPI == EPI_SILU_MUL) up += u[t];
+    }
+  }
+  for (; z < slices; ++z) {
+    sum += *reinterpret_cast<const f32x4*>(row + z * copy + j);
+    if (EPI == EPI_SILU_MUL) up += *reinterpret_cast<const f32x4*>(row + z * copy + N / 2 + j);
   }
   CT* out = c + (size_t)m * ldc + j;
 #pragma unroll
@@ -657,8 +672,19 @@ __global__ __launch_bounds__(256) void splitk_reduce_norm_kernel(const float* __
     const int j = (tid + 256 * i) * 4;
     if (j >= N) break;
     f32x4 sum = {0.f, 0.f, 0.f, 0.f};  // the slices in their order, then the residual: as the plain second pass does
-    for (int z = 0; z < slices; ++z) sum += *reinterpret_cast<const f32x4*>(ws + ((size_t)z * M + m) * N + j);
-    sum = *reinterpret_cast<const f32x4*>(c + (size_t)m * ldc + j) + sum;
+    const size_t copy = (size_t)M * N;
+    const float* row = ws + (size_t)m * N + j;
+    const f32x4 old = *reinterpret_cast<const f32x4*>(c + (size_t)m * ldc + j);
+    int z = 0;
+    for (; z + 4 <= slices; z += 4) {  // four slices' loads on their way together
+      f32x4 v[4];
+#pragma unroll
+      for (int t = 0; t < 4; ++t) v[t] = *reinterpret_cast<const f32x4*>(row + (z + t) * copy);
+#pragma unroll
+      for (int t = 0; t < 4; ++t) sum += v[t];
+    }
+    for (; z < slices; ++z) sum += *reinterpret_cast<const f32x4*>(row + z * copy);
+    sum = old + sum;
     *reinterpret_cast<f32x4*>(c + (size_t)m * ldc + j) = sum;
     r[i] = sum;
     ss += sum[0] * sum[0] + sum[1] * sum[1] + sum[2] * sum[2] + sum[3] * sum[3];
