@@ -243,6 +243,55 @@ __global__ void rope_store_kernel(T* __restrict__ qkv, int row_stride, const flo
   }
 }
 
+// The same for head sizes that are a multiple of 16, bfloat16, with 16-byte aligned rows: a lane takes a whole
+// piece of 8 dimensions and its partner piece hd/2 further on as 16-byte words, so that a key's pieces go to
+// their places in the page (key_piece()) in one store each.  hd / 16 lanes a head.
+__global__ void rope_store_pieces_kernel(bf16* __restrict__ qkv, int row_stride, const float* __restrict__ cosv,
+                                         const float* __restrict__ sinv, const int32_t* __restrict__ slots,
+                                         bf16* __restrict__ k_pages, bf16* __restrict__ v_pages, int nh, int nkv, int hd,
+                                         int page_size, int rotate, int v_rows) {
+  const int t = blockIdx.x;
+  const int half = hd / 2, lanes = half / 8;  // lanes a head
+  const int idx = blockIdx.y * blockDim.x + threadIdx.x;
+  const int unit = idx / lanes, j = (idx % lanes) * 8;
+  const int units = nh + nkv + ((slots && t < v_rows) ? nkv : 0);  // rows from v_rows on: values are stored by tiles
+  if (unit >= units) return;
+  bf16* head = qkv + (size_t)t * row_stride + (size_t)unit * hd;
+  const bool is_v = unit >= nh + nkv, is_k = unit >= nh && !is_v;
+  const int slot = (slots && unit >= nh) ? slots[t] : -1;
+  const int page = slot >= 0 ? slot / page_size : 0, off = slot >= 0 ? slot % page_size : 0;
+  const bf16x8 x0 = *reinterpret_cast<const bf16x8*>(head + j), x1 = *reinterpret_cast<const bf16x8*>(head + half + j);
+  bf16x8 y0 = x0, y1 = x1;
+  if (!is_v && rotate) {
+    const float* cr = cosv + (size_t)t * half + j;
+    const float* sr = sinv + (size_t)t * half + j;
+    const f32x4 c0 = *reinterpret_cast<const f32x4*>(cr), c1 = *reinterpret_cast<const f32x4*>(cr + 4);
+    const f32x4 s0 = *reinterpret_cast<const f32x4*>(sr), s1 = *reinterpret_cast<const f32x4*>(sr + 4);
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+      const float c = e < 4 ? c0[e] : c1[e - 4], sn = e < 4 ? s0[e] : s1[e - 4];
+      const float a = (float)x0[e], b = (float)x1[e];
+      y0[e] = (bf16)(a * c - b * sn);
+      y1[e] = (bf16)(b * c + a * sn);
+    }
+    *reinterpret_cast<bf16x8*>(head + j) = y0;  // rotated keys stay in the row too: parts may read them back
+    *reinterpret_cast<bf16x8*>(head + half + j) = y1;
+  }
+  if (slot < 0) return;
+  if (is_k) {
+    bf16* dst = k_pages + ((size_t)page * nkv + (unit - nh)) * page_size * hd;
+    *reinterpret_cast<bf16x8*>(dst + key_offset(off, j, page_size, 8)) = y0;
+    *reinterpret_cast<bf16x8*>(dst + key_offset(off, half + j, page_size, 8)) = y1;
+  } else if (is_v) {
+    bf16* dst = v_pages + ((size_t)page * nkv + (unit - nh - nkv)) * hd * page_size + off;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+      dst[(size_t)(j + e) * page_size] = x0[e];
+      dst[(size_t)(half + j + e) * page_size] = x1[e];
+    }
+  }
+}
+
 // Values of prompt portions, sixteen positions at a time: the transposed page holds the sixteen slots
 // of one dimension side by side, so a tile of 16 tokens x hd is turned in LDS and written as whole
 // 16-byte words instead of two bytes at a time.  grid (groups of 16 positions, kv heads, requests
@@ -337,6 +386,17 @@ extern "C" int gb_rope_store(void* qkv, int dtype, int row_stride, const float* 
   }
   const bool pairs_of_two = hd % 4 == 0 && row_stride % 2 == 0 && (uintptr_t)qkv % 8 == 0 && (uintptr_t)k_pages % 8 == 0 &&
                             (!rotate || ((uintptr_t)cosv % 8 == 0 && (uintptr_t)sinv % 8 == 0));
+  const bool pieces = dtype == kBF16 && hd % 16 == 0 && row_stride % 8 == 0 && (uintptr_t)qkv % 16 == 0 &&
+                      (uintptr_t)k_pages % 16 == 0 && (!rotate || ((uintptr_t)cosv % 16 == 0 && (uintptr_t)sinv % 16 == 0));
+  if (pieces) {
+    const int units = nh + nkv + (slots ? nkv : 0), lanes = units * (hd / 16);
+    const int threads = lanes >= 256 ? 256 : 64;
+    const dim3 grid(n, (lanes + threads - 1) / threads);
+    GB_REQUIRE(grid.y <= 65535, "rope_store: %d heads are too many for one launch", units);
+    hipLaunchKernelGGL(rope_store_pieces_kernel, grid, dim3(threads), 0, stream, (bf16*)qkv, row_stride, cosv, sinv, slots,
+                       (bf16*)k_pages, (bf16*)v_pages, nh, nkv, hd, page_size, rotate, v_rows);
+    return launched("rope_store");
+  }
   if (pairs_of_two) {
     const int units = nh + nkv + (slots ? nkv : 0);
     const int threads = n <= 64 ? 64 : 256;  // few tokens: more, smaller workgroups

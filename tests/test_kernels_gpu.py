@@ -364,6 +364,42 @@ ROPE_PRODUCTS = [(1, 4, 2, 16, 64), (8, 3, 1, 32, 96), (5, 6, 2, 48, 80), (8, 32
                  (64, 15, 5, 64, 960), (7, 4, 0, 32, 64)]
 
 
+@pytest.mark.parametrize("nh,nkv,hd,page", [(4, 2, 16, 16), (32, 32, 64, 16), (5, 1, 48, 32), (8, 2, 128, 16), (3, 3, 80, 64)])
+def test_rope_store_in_bfloat16_moves_whole_pieces(nh, nkv, hd, page):
+    """bfloat16 rows of head sizes in steps of 16 (a lane takes 8 dimensions and their partners): rotated queries
+    in the row, rotated keys in the row and in their pages, values in theirs, against float64
+    (crates/glassbox-core/src/model.rs:102-115, 273-275)."""
+    from glassbox_amd import ops
+    from plain import llama
+    n, theta = 37, 130000.0
+    g = torch.Generator().manual_seed(hd)
+    pos = torch.randint(0, 6000, (n,), generator=g).tolist()
+    s64, c64 = llama.rope_angles(pos, hd, theta)
+    cos, sin = to_dev(torch.from_numpy(c64).float()), to_dev(torch.from_numpy(s64).float())
+    qkv = rnd(n, (nh + 2 * nkv) * hd, seed=7).bfloat16()
+    pages = 4
+    slots = torch.randperm(pages * page, generator=g)[:n].to(torch.int32)
+    k_pages = torch.zeros(ops.key_pages_shape(pages, nkv, page, hd), device=DEV, dtype=torch.bfloat16)
+    v_pages = torch.zeros(pages, nkv, hd, page, device=DEV, dtype=torch.bfloat16)
+    buf = to_dev(qkv.clone())
+    ops.rope_store(buf, cos, sin, to_dev(slots), k_pages, v_pages, nh, nkv, hd)
+    q_want = llama.rope(qkv[:, :nh * hd].double().reshape(n, nh, hd), pos, theta)
+    k_want = llama.rope(qkv[:, nh * hd:(nh + nkv) * hd].double().reshape(n, nkv, hd), pos, theta)
+    got = buf.cpu()
+    tol = 2 ** -8 * 1.5 * qkv.abs().max().item()   # one rounding to bfloat16 of a value up to sqrt(2) times the largest input
+    assert (got[:, :nh * hd].double().reshape(n, nh, hd) - q_want).abs().max().item() <= tol
+    assert (got[:, nh * hd:(nh + nkv) * hd].double().reshape(n, nkv, hd) - k_want).abs().max().item() <= tol
+    assert torch.equal(got[:, (nh + nkv) * hd:], qkv[:, (nh + nkv) * hd:]), "values stay as they are"
+    idx = slots.long()
+    assert torch.equal(ops.unpack_keys(k_pages).cpu()[idx // page, :, idx % page, :], got[:, nh * hd:(nh + nkv) * hd].reshape(n, nkv, hd))
+    assert torch.equal(v_pages.cpu()[idx // page, :, :, idx % page], qkv[:, (nh + nkv) * hd:].reshape(n, nkv, hd))
+    free = torch.ones(pages * page, dtype=torch.bool)
+    free[idx] = False
+    fi = torch.nonzero(free).flatten()
+    assert ops.unpack_keys(k_pages).cpu()[fi // page, :, fi % page, :].abs().sum().item() == 0
+    assert v_pages.cpu()[fi // page, :, :, fi % page].abs().sum().item() == 0
+
+
 @pytest.mark.parametrize("M,nh,nkv,hd,K,normed", [p + (False,) for p in ROPE_PRODUCTS] +
                          [p + (True,) for p in ROPE_PRODUCTS if p[0] <= 16])   # the norm on the way in serves 16 rows
 def test_gemm_bf16_rotates_and_writes_the_cache(M, nh, nkv, hd, K, normed):
