@@ -1,6 +1,8 @@
 // Memory-bound parts of a decoder step, in 32-bit and bfloat16 storage: embedding
 // gather, RMS norm, rotary table, rotation fused with the cache write, SiLU-multiply,
 // and page copies.  All arithmetic is 32-bit; only loads and stores differ by type.
+#include <type_traits>
+
 #include "common.h"
 
 using namespace gb;
@@ -75,15 +77,80 @@ __global__ void rmsnorm_kernel(const float* __restrict__ x, const G* __restrict_
   for (int c = tid + VPT * nt; c < d; c += nt) orow[c] = from_f<O>(to_f(gamma[c]) * (xr[c] * s));
 }
 
+// The same with four neighbouring columns a thread as one word (rows of a multiple of 4 columns, up to
+// 4 * V4 * threads of them): a quarter of the loads and stores.
+template <typename G, typename O, int V4>
+__global__ void rmsnorm_words_kernel(const float* __restrict__ x, const G* __restrict__ gamma, const int32_t* __restrict__ rows,
+                                     O* __restrict__ out, int d, float eps) {
+  __shared__ float partial[16];
+  const int r = blockIdx.x, tid = threadIdx.x, nt = blockDim.x;
+  const float* xr = x + (size_t)(rows ? rows[r] : r) * d;
+  f32x4 v[V4], g[V4];
+  float ss = 0.f;
+#pragma unroll
+  for (int j = 0; j < V4; ++j) {
+    const int c = (tid + j * nt) * 4;
+    v[j] = f32x4{0.f, 0.f, 0.f, 0.f};
+    g[j] = v[j];
+    if (c < d) {
+      v[j] = *reinterpret_cast<const f32x4*>(xr + c);
+      if constexpr (std::is_same<G, float>::value) {
+        g[j] = *reinterpret_cast<const f32x4*>(gamma + c);
+      } else {
+        const bf16x4 gb = *reinterpret_cast<const bf16x4*>(gamma + c);
+#pragma unroll
+        for (int e = 0; e < 4; ++e) g[j][e] = (float)gb[e];
+      }
+    }
+  }
+#pragma unroll
+  for (int j = 0; j < V4; ++j)
+#pragma unroll
+    for (int e = 0; e < 4; ++e) ss += v[j][e] * v[j][e];
+  ss = wave_sum(ss);
+  if (tid % kWave == 0) partial[tid / kWave] = ss;
+  __syncthreads();
+  float total = 0.f;
+  for (int w = 0; w < (nt + kWave - 1) / kWave; ++w) total += partial[w];
+  const float s = 1.0f / sqrtf(total / (float)d + eps);
+  O* orow = out + (size_t)r * d;
+#pragma unroll
+  for (int j = 0; j < V4; ++j) {
+    const int c = (tid + j * nt) * 4;
+    if (c >= d) continue;
+    if constexpr (std::is_same<O, float>::value) {
+      f32x4 o;
+#pragma unroll
+      for (int e = 0; e < 4; ++e) o[e] = g[j][e] * (v[j][e] * s);
+      *reinterpret_cast<f32x4*>(orow + c) = o;
+    } else {
+      bf16x4 o;
+#pragma unroll
+      for (int e = 0; e < 4; ++e) o[e] = (bf16)(g[j][e] * (v[j][e] * s));
+      *reinterpret_cast<bf16x4*>(orow + c) = o;
+    }
+  }
+}
+
 extern "C" int gb_rmsnorm(const float* x, const void* gamma, int gamma_dtype, const int32_t* rows, void* out,
                           int out_dtype, int m, int d, float eps, hipStream_t stream) {
   GB_REQUIRE(m >= 0 && d > 0, "rmsnorm: bad sizes m=%d d=%d", m, d);
   if (m == 0) return 0;
   const int threads = d >= 1024 ? 256 : (d >= 256 ? 128 : 64);
   const int per_thread = (d + threads - 1) / threads;
+  // whole words where the rows allow it (every row then starts at a multiple of 16 bytes)
+  const bool words = d % 4 == 0 && d <= 4 * 8 * threads && (uintptr_t)x % 16 == 0 && (uintptr_t)gamma % 16 == 0 &&
+                     (uintptr_t)out % 16 == 0;
+  const int words_per_thread = (d / 4 + threads - 1) / threads;
 #define GB_LAUNCH(G, O)                                                                                                     \
   do {                                                                                                                      \
-    if (per_thread <= 4)                                                                                                    \
+    if (words && words_per_thread <= 2)                                                                                     \
+      hipLaunchKernelGGL((rmsnorm_words_kernel<G, O, 2>), dim3(m), dim3(threads), 0, stream, x, (const G*)gamma, rows, (O*)out, d, eps); \
+    else if (words && words_per_thread <= 4)                                                                                \
+      hipLaunchKernelGGL((rmsnorm_words_kernel<G, O, 4>), dim3(m), dim3(threads), 0, stream, x, (const G*)gamma, rows, (O*)out, d, eps); \
+    else if (words)                                                                                                         \
+      hipLaunchKernelGGL((rmsnorm_words_kernel<G, O, 8>), dim3(m), dim3(threads), 0, stream, x, (const G*)gamma, rows, (O*)out, d, eps); \
+    else if (per_thread <= 4)                                                                                               \
       hipLaunchKernelGGL((rmsnorm_kernel<G, O, 4>), dim3(m), dim3(threads), 0, stream, x, (const G*)gamma, rows, (O*)out, d, eps); \
     else                                                                                                                    \
       hipLaunchKernelGGL((rmsnorm_kernel<G, O, 16>), dim3(m), dim3(threads), 0, stream, x, (const G*)gamma, rows, (O*)out, d, eps); \
