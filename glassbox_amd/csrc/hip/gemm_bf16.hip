@@ -1003,13 +1003,27 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_skinny_kernel(const void* __r
       }
     }
   } else {
+    // accumulating: all of a thread's old values are asked for before any is added to (behind the checks one
+    // by one, every read would wait for the one before it)
+    float old[RT][MT];
+    if (EPI == EPI_ACCUMULATE) {
+#pragma unroll
+      for (int rt = 0; rt < RT; ++rt) {
+        const int n = (blockIdx.x * RT + rt) * 16 + nrow;
+#pragma unroll
+        for (int t = 0; t < MT; ++t) {
+          const int m = t * 16 + l % 16;
+          old[rt][t] = (m < M && n < N) ? (float)c[(size_t)m * ldc + n] : 0.f;
+        }
+      }
+    }
 #pragma unroll
     for (int rt = 0; rt < RT; ++rt) {
       const int n = (blockIdx.x * RT + rt) * 16 + nrow;
 #pragma unroll
       for (int t = 0; t < MT; ++t) {
         const int m = t * 16 + l % 16;
-        if (m < M && n < N) store_c<CT>(c + (size_t)m * ldc + n, v[rt][t], EPI == EPI_ACCUMULATE);
+        if (m < M && n < N) c[(size_t)m * ldc + n] = (CT)(EPI == EPI_ACCUMULATE ? old[rt][t] + v[rt][t] : v[rt][t]);
       }
     }
   }
