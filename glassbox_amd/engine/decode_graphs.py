@@ -19,6 +19,8 @@ every part must declare ``replayable`` (parts.base.Part).
 """
 from __future__ import annotations
 
+import contextlib
+import gc
 from collections import OrderedDict
 from typing import List, Sequence, Tuple
 
@@ -28,6 +30,22 @@ from .context import StepContext, Workspace
 
 BUCKET = 1024
 MAX_SHAPES = 64   # shapes kept (buffers and a graph each); the least recently used one goes first
+
+
+@contextlib.contextmanager
+def capture(graph: "torch.cuda.CUDAGraph"):
+    """``torch.cuda.graph(graph)`` with the garbage collector held off.  A graph that dies synchronises the
+    device (torch's destructor does, on this platform), which no call may do while a stream captures: an
+    engine dropped earlier, which the collector frees when it pleases because engine and graphs refer to each
+    other, must not be freed in here.  Nothing in here drops a graph by itself."""
+    was_on = gc.isenabled()
+    gc.disable()
+    try:
+        with torch.cuda.graph(graph):
+            yield
+    finally:
+        if was_on:
+            gc.enable()
 
 
 def padded_rows(n: int) -> int:
@@ -131,7 +149,7 @@ class DecodeGraphs:
         else:
             torch.cuda.synchronize()
             graph = torch.cuda.CUDAGraph()
-            with torch.cuda.graph(graph):
+            with capture(graph):
                 shape.ctx.memo.clear()
                 shape.logits = eng.model.forward(shape.ctx, eng.layers)
             if self.workspace.epoch != self.epoch:

@@ -15,6 +15,7 @@ import torch
 
 from .. import ops
 from .context import StepContext
+from .decode_graphs import capture
 from .engine import Engine, EngineError
 
 
@@ -120,7 +121,7 @@ class DecodeLoop:
         else:
             torch.cuda.synchronize()
             graph = torch.cuda.CUDAGraph()
-            with torch.cuda.graph(graph):
+            with capture(graph):
                 self._run()
             self.graphs[bucket] = graph
             graph.replay()                   # capture does not execute

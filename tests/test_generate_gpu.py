@@ -332,3 +332,40 @@ def test_decode_graph_shapes_are_kept_up_to_a_limit(model_dirs, monkeypatch):
                 nxt[r] = int(row.argmax())
         assert len(engs[0].decode_graphs.shapes) <= 2
     assert engs[0].decode_graphs.replays >= 6
+
+
+def test_nothing_is_collected_while_a_step_is_captured(model_dirs):
+    """Graphs of an engine that was dropped are freed by the garbage collector (engine and graphs refer to each
+    other), and a graph that dies synchronises the device, which is not allowed while a stream captures: the
+    collector is held off for the length of a capture, and is back on after it."""
+    import gc
+    import torch
+    from glassbox_amd.engine import Engine
+    folder = model_dirs.get("A")
+    toks = helpers.random_tokens(helpers.TINY["A"]["vocab_size"], 12, seed=5)
+
+    def decode(eng, steps, seen=None):
+        eng.step([("r", toks, [])])
+        if seen is not None:
+            plain = eng.model.forward
+            def spy(ctx, layers):
+                if torch.cuda.is_current_stream_capturing():
+                    seen.append(gc.isenabled())
+                return plain(ctx, layers)
+            eng.model.forward = spy
+        nxt = 7
+        for _ in range(steps):
+            nxt = int(eng.step([("r", [nxt], [0])])[0].argmax())
+        eng.end_request("r")
+        return nxt
+
+    first = Engine(folder, dtype="bfloat16", max_tokens=256, max_seqs=2)
+    want = decode(first, 5)
+    assert first.decode_graphs.replays >= 3
+    del first                                   # garbage with graphs in it, for the collector to find some time
+    seen = []
+    assert gc.isenabled()
+    second = Engine(folder, dtype="bfloat16", max_tokens=256, max_seqs=2)
+    assert decode(second, 5, seen) == want
+    assert seen and not any(seen), "the collector was on during a capture"
+    assert gc.isenabled()
