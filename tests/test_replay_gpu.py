@@ -189,3 +189,43 @@ def test_trace_run_program(model_dirs, tmp_path, dtype):
         assert row == data.shape[0]
     got = {r: np.concatenate(p, 0) for r, p in got.items()}
     check(folder, requests, got, dtype, "trace_run")
+
+
+@pytest.mark.parametrize("seed", range(8))
+def test_random_configurations(tmp_path, seed):
+    """Configurations drawn at random (head sizes that the matrix-core kernels take and others, heads in groups of
+    one to four, widths, feed-forward sizes and vocabularies that are no power of two, one to three layers, tied
+    or not): mixed steps over a pool that is used again, in 32-bit and in bfloat16, against the plain
+    implementation."""
+    import random
+    from plain import llama as plain_llama
+    from glassbox_amd.config import config_from_dict
+    from glassbox_amd.engine import Engine
+    from glassbox_amd.weights import write_random_model
+    rng = random.Random(4000 + seed)
+    hd = rng.choice([16, 32, 48, 64, 80, 96, 112, 128, 24, 40, 8])
+    nkv = rng.choice([1, 2, 3, 5])
+    nh = nkv * rng.choice([1, 2, 3, 4])
+    vocab = rng.randrange(90, 700)
+    cfg_d = dict(architectures=["LlamaForCausalLM"], hidden_size=rng.choice([8, 16, 24]) * rng.randrange(3, 12),
+                 intermediate_size=16 * rng.randrange(4, 20), num_hidden_layers=rng.choice([1, 2, 3]),
+                 num_attention_heads=nh, num_key_value_heads=nkv, head_dim=hd, vocab_size=vocab,
+                 rope_theta=float(rng.choice([10000, 130000, 500000])), rms_norm_eps=rng.choice([1e-5, 1e-6, 3e-5]),
+                 tie_word_embeddings=rng.random() < 0.5, max_position_embeddings=1024)
+    folder = str(tmp_path / "model")
+    write_random_model(config_from_dict(cfg_d), folder, seed, norm_init="uniform", dtype=torch.float32)
+    requests = {f"r{i}": helpers.random_tokens(vocab, rng.randrange(1, 260), seed=seed * 10 + i) for i in range(4)}
+    cfg, w = plain_llama.load_folder(folder)
+    want = {r: plain_llama.forward(w, cfg, list(t), torch.float64).numpy() for r, t in requests.items()}
+    steps, peak = helpers.schedule_mixed(requests, seed=seed, live=rng.choice([2, 3, 4]))
+    rms = max(float(np.sqrt(np.mean(x ** 2))) for x in want.values())
+    for dtype in ("float32", "bfloat16"):
+        eng = Engine(folder, dtype=dtype, max_tokens=peak, max_seqs=4)
+        got = helpers.replay(eng, steps)
+        tol = TOL[dtype] * (max(1.0, rms / 0.25) if dtype == "bfloat16" else 1.0)   # as in the tests above
+        for r, toks in requests.items():
+            bad = helpers.first_bad(got[r], want[r], tol)
+            assert bad is None, (f"{cfg_d}, request {r} ({len(toks)} tokens), {dtype}: first wrong position {bad[0]}, "
+                                 f"max abs error {bad[1]:.3e}")
+        eng.cache.check_invariants()
+        assert eng.cache.used_pages() == 0
