@@ -364,8 +364,20 @@ template <int LEFT> __device__ __forceinline__ void vm_wait() { __builtin_amdgcn
 template <int EPI, typename CT>
 __global__ __launch_bounds__(512, 1) void gemm_ring_kernel(const bf16* __restrict__ a, int lda, const bf16* __restrict__ w, int ldw,
                                                            CT* __restrict__ c, int ldc, int M, int N, int K, int k_slice) {
+  int bx = blockIdx.x, by = blockIdx.y;
   if (k_slice > 0) {  // split k: workgroup z of a tile sums its own slice of k into its own copy of C
-    const int z = blockIdx.z;
+    int z = blockIdx.z;
+    // The chip deals workgroups round its 8 dies by their number, and each die has a second-level cache of its
+    // own.  With the grid as it stands a die would hold one column tile over all row tiles and all slices (8 + 32
+    // different operand pieces a k-step among its 32 workgroups); numbered anew, it holds an eighth of the grid in
+    // a row: one slice, some row tiles, all column tiles (4 + 8 pieces), which its cache then serves.
+    const int gx = gridDim.x, gy = gridDim.y, total = gx * gy * gridDim.z;
+    if (total % 8 == 0) {
+      const int id = bx + gx * (by + gy * z), anew = (id % 8) * (total / 8) + id / 8;
+      bx = anew % gx;
+      by = (anew / gx) % gy;
+      z = anew / (gx * gy);
+    }
     a += (size_t)z * k_slice;
     w += (size_t)z * k_slice;
     c += (size_t)z * M * ldc;
@@ -375,16 +387,16 @@ __global__ __launch_bounds__(512, 1) void gemm_ring_kernel(const bf16* __restric
   __shared__ __attribute__((aligned(16))) bf16 Ws[RING_STAGES][RBN * RBK];
   const int tid = threadIdx.x, lane = tid % 64, wave = tid / 64;
   const int wm = wave / RGN, wn = wave % RGN;
-  const int m0 = blockIdx.y * RBM;
+  const int m0 = by * RBM;
   const int half = N / 2;  // EPI_SILU_MUL: number of gate rows
   // row of W behind row r of the workgroup's W tile (r = wn * 64 + j * 32 + column); with EPI_SILU_MUL a wave's
   // first column tile holds gate rows and its second the up rows that belong to them
   auto w_row = [&](int r) -> int {
     if (EPI == EPI_SILU_MUL) {
-      const int n = blockIdx.x * (RBN / 2) + (r / 64) * 32 + r % 32;
+      const int n = bx * (RBN / 2) + (r / 64) * 32 + r % 32;
       return n < half ? ((r % 64) / 32 ? half + n : n) : 0;
     }
-    return min(blockIdx.x * RBN + r, N - 1);
+    return min(bx * RBN + r, N - 1);
   };
   // a wave's load instruction moves 16 rows x 4 pieces; rows beyond M or N are read from a row that exists
   const bf16* asrc[RLA];
@@ -498,7 +510,7 @@ __global__ __launch_bounds__(512, 1) void gemm_ring_kernel(const bf16* __restric
 
   // accumulator layout of a 32x32 tile: lane holds column lane%32, rows 8*(r/4) + 4*(lane/32) + r%4
   if (EPI == EPI_SILU_MUL) {
-    const int gn = blockIdx.x * (RBN / 2) + wn * 32 + lane % 32;
+    const int gn = bx * (RBN / 2) + wn * 32 + lane % 32;
     if (gn >= half) return;
 #pragma unroll
     for (int i = 0; i < RTM; ++i)
@@ -512,10 +524,10 @@ __global__ __launch_bounds__(512, 1) void gemm_ring_kernel(const bf16* __restric
   }
   if constexpr (EPI == EPI_ACCUMULATE) {
     // as in the tiled kernel: inside C, all old values of a tile are read before any is added to
-    if (m0 + (wm + 1) * RTM * 32 <= M && blockIdx.x * RBN + (wn + 1) * RTN * 32 <= N) {
+    if (m0 + (wm + 1) * RTM * 32 <= M && bx * RBN + (wn + 1) * RTN * 32 <= N) {
 #pragma unroll
       for (int i = 0; i < RTM; ++i) {
-        CT* base = c + (size_t)(m0 + wm * RTM * 32 + i * 32 + 4 * (lane / 32)) * ldc + blockIdx.x * RBN + wn * RTN * 32 + lane % 32;
+        CT* base = c + (size_t)(m0 + wm * RTM * 32 + i * 32 + 4 * (lane / 32)) * ldc + bx * RBN + wn * RTN * 32 + lane % 32;
         float old[RTN][16];
 #pragma unroll
         for (int j = 0; j < RTN; ++j)
@@ -533,7 +545,7 @@ __global__ __launch_bounds__(512, 1) void gemm_ring_kernel(const bf16* __restric
   for (int i = 0; i < RTM; ++i)
 #pragma unroll
     for (int j = 0; j < RTN; ++j) {
-      const int gn = blockIdx.x * RBN + wn * RTN * 32 + j * 32 + lane % 32;
+      const int gn = bx * RBN + wn * RTN * 32 + j * 32 + lane % 32;
       if (gn >= N) continue;
 #pragma unroll
       for (int r = 0; r < 16; ++r) {
