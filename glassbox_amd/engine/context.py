@@ -22,10 +22,16 @@ class Workspace:
     def __init__(self, device):
         self.device = device
         self._flat: Dict[Tuple[str, torch.dtype], torch.Tensor] = {}
+        #: the views handed out, by (name, dtype, shape): a step asks for the same few hundred again and again
+        self._views: Dict[tuple, torch.Tensor] = {}
         #: counts the times a buffer was replaced by a larger one: a captured graph holds the old addresses
         self.epoch = 0
 
     def buffer(self, name: str, shape: Sequence[int], dtype: torch.dtype) -> torch.Tensor:
+        vkey = (name, dtype, tuple(shape))
+        view = self._views.get(vkey)
+        if view is not None:
+            return view
         count = 1
         for s in shape:
             count *= int(s)
@@ -39,7 +45,11 @@ class Workspace:
                 self.epoch += 1
             flat = torch.empty(grow, dtype=dtype, device=self.device)
             self._flat[key] = flat
-        return flat[:count].view(*shape)
+            self._views = {k: v for k, v in self._views.items() if (k[0], k[1]) != key}   # they point into the old buffer
+        view = flat[:count].view(*shape)
+        if len(self._views) < 4096:
+            self._views[vkey] = view
+        return view
 
     def bytes(self) -> int:
         return sum(t.numel() * t.element_size() for t in self._flat.values())

@@ -106,12 +106,13 @@ def _check(lib, rc: int) -> None:
 
 
 _raw_stream = getattr(torch._C, "_cuda_getCurrentRawStream", None)
+_get_device = getattr(torch._C, "_cuda_getDevice", torch.cuda.current_device)   # CUDA is up by the time a kernel is launched
 
 
 def _stream():
     # every kernel launch asks for the stream: the raw handle costs a fraction of a Stream object
     if _raw_stream is not None:
-        return _raw_stream(torch.cuda.current_device())
+        return _raw_stream(_get_device())
     return torch.cuda.current_stream().cuda_stream
 
 
