@@ -9,6 +9,7 @@ and stream owner; no torch operator computes anything here.
 from __future__ import annotations
 
 import ctypes as C
+import functools
 from typing import Optional
 
 import torch
@@ -295,12 +296,14 @@ def copy_rows(base: torch.Tensor, src: torch.Tensor, dst: torch.Tensor) -> None:
 FUSED_NORM_MAX_ROWS = 16   # measured: beyond one 16-row block the re-reading of float32 rows costs more than a norm pass
 
 
+@functools.lru_cache(maxsize=4096)   # a pure function of the sizes, asked for at every product
 def gemm_emit_parts(rows: int, n: int) -> int:
     """How many partial sums an accumulating bfloat16 product of ``rows`` rows and ``n`` columns writes when
     asked to prepare the norm that follows (``gemm(..., emit=...)``); 0 if that product cannot."""
     return int(_lib("gemm_bf16").gb_gemm_bf16_emit_parts(int(rows), int(n)))
 
 
+@functools.lru_cache(maxsize=4096)   # a pure function of the sizes, asked for at every product
 def gemm_emit_mode(rows: int, n: int, k: int) -> int:
     """What an accumulating bfloat16 product of these sizes can do for the RMS norm that reads the residual after
     it: 0 nothing; 1 the operand and partial sums (``gemm(..., emit=(gamma, h, parts))``, see ``gemm_emit_parts``);
@@ -308,6 +311,7 @@ def gemm_emit_mode(rows: int, n: int, k: int) -> int:
     return int(_lib("gemm_bf16").gb_gemm_bf16_emit_mode(int(rows), int(n), int(k)))
 
 
+@functools.lru_cache(maxsize=4096)   # a pure function of the sizes, asked for at every product
 def gemm_split_floats(rows: int, n: int, k: int) -> int:
     """Floats of workspace with which a bfloat16 product of these sizes would divide k over workgroups
     (``gemm(..., workspace=)``); 0 if it would not: only products with few tiles do."""
@@ -481,6 +485,7 @@ def tuned_attention_supports(k_pages: torch.Tensor, n_heads: int, window: int) -
             and n_heads // nkv <= 16 and page >= 16 and page & (page - 1) == 0)
 
 
+@functools.lru_cache(maxsize=4096)   # a pure function of the sizes, asked for at every product
 def decode_chunk(n_decode: int, n_kv_heads: int, max_context: int) -> int:
     """Keys per workgroup of the decode kernel: a multiple of 256.  With a workgroup for every compute
     unit from requests and kv heads alone, each takes a whole context (and sixteen waves: nothing is
@@ -512,6 +517,11 @@ def attention_decode(q: torch.Tensor, out: torch.Tensor, ctx, cache, n_heads: in
                                              max_context, _stream()))
 
 
+@functools.lru_cache(maxsize=4096)
+def _prefill_parts(max_q: int, max_ctx: int, n_heads: int, n_seqs: int, hd: int) -> int:
+    return int(_lib("attention_bf16").gb_attention_prefill_parts(max_q, max_ctx, n_heads, n_seqs, hd))
+
+
 def attention_prefill(q: torch.Tensor, out: torch.Tensor, ctx, cache, n_heads: int, scale: float, window: int) -> None:
     """The requests of the step that bring more than one token (they follow the single-token ones)."""
     n_dec, S = ctx.host["n_decode"], ctx.num_seqs
@@ -526,7 +536,7 @@ def attention_prefill(q: torch.Tensor, out: torch.Tensor, ctx, cache, n_heads: i
     # the portions' rows follow the single-token requests' rows; few and short portions over long contexts share
     # their keys among workgroups, which need room for their sums
     first_row, n_rows = n_dec, q.shape[0] - n_dec
-    parts = lib.gb_attention_prefill_parts(max_q, max_ctx, n_heads, S - n_dec, hd)
+    parts = _prefill_parts(max_q, max_ctx, n_heads, S - n_dec, hd)
     ws = ctx.buffer("attn_parts", (parts * n_rows * n_heads * (hd + 2),), torch.float32) if parts > 1 else None
     _check(lib, lib.gb_attention_prefill_bf16(_p(q), _rows(q, "q"), _p(out), _rows(out, "out"), _p(ctx.q_start),
                                               _p(ctx.q_len), _p(ctx.pos0), n_dec, S - n_dec, max_q, max_ctx, _p(tables),
