@@ -15,7 +15,7 @@ import sys
 import time
 from typing import List
 
-USAGE = """usage:
+USAGE = """
   glassbox generate --model DIR --prompt IDS [-n 128] [--dtype bfloat16|float32]
                     [--temp 0] [--top-p 1] [--top-k 0] [--min-p 0] [--repeat-penalty 1] [--seed 0]
                     [--blocks 2048] [--budget 256] [--max-seqs 32] [--no-prefix-cache]
