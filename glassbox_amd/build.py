@@ -43,7 +43,7 @@ LIBRARIES: Dict[str, tuple] = {
     "gemm_f32": ("hip", ["hip/gemm_f32.hip"], ["hip/common.h"]),
     "gemm_bf16": ("hip", ["hip/gemm_bf16.hip"], ["hip/common.h"]),
     "attention_plain": ("hip", ["hip/attention_plain.hip"], ["hip/common.h"]),
-    "attention_bf16": ("hip", ["hip/attention_bf16.hip"], ["hip/common.h"]),
+    "attention_bf16": ("hip", ["hip/attention_bf16.hip"], ["hip/common.h", "hip/attention_bf16.h"]),
     "sampling": ("hip", ["hip/sampling.hip"], ["hip/common.h"]),
 }
 

@@ -20,7 +20,10 @@
 // (chunk, kv head, request), four waves taking 64 keys each in turn; partial results are merged
 // in a fixed order (waves in LDS, chunks by a second kernel), so the result is the same on every
 // run.  crates/glassbox-core/src/model.rs:285-312 is the formula.
+#include "attention_bf16.h"
 #include "common.h"
+
+#include <mutex>
 
 using namespace gb;
 
@@ -756,6 +759,57 @@ extern "C" int gb_attention_decode_bf16(const void* q, int q_stride, void* out, 
     return launched("attention_decode_reduce");
   }
   return 0;
+}
+
+// ------------------------------------------------------- decoding without a workspace from the caller
+// The chunks' partial results of gb_attention_decode_bf16 in memory that the library itself holds: a file-scope
+// array on every GPU, instead of the caller's ws_acc / ws_ml.  For callers that cannot allocate.  Declared and
+// described in attention_bf16.h.
+namespace {
+static __device__ __align__(256) float scratch[GB_DECODE_STATIC_FLOATS];
+// In host code the array's name is only a handle for hipGetSymbolAddress; the address kernels may use is asked
+// for once per device, with that device current, and kept here.
+constexpr int kMaxDevices = 64;
+float* scratch_of_device[kMaxDevices];
+std::mutex scratch_lock;
+
+int static_scratch(float** ptr) {
+  int device = -1;
+  hipError_t e = hipGetDevice(&device);
+  if (e != hipSuccess) return fail("attention_decode_static: hipGetDevice: %s", hipGetErrorString(e));
+  if (device < 0 || device >= kMaxDevices) return fail("attention_decode_static: device %d is beyond the %d this library keeps scratch for", device, kMaxDevices);
+  std::lock_guard<std::mutex> hold(scratch_lock);
+  if (!scratch_of_device[device]) {
+    void* p = nullptr;
+    e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+    if (e != hipSuccess || !p) return fail("attention_decode_static: hipGetSymbolAddress on device %d: %s", device, hipGetErrorString(e));
+    scratch_of_device[device] = static_cast<float*>(p);
+  }
+  *ptr = scratch_of_device[device];
+  return 0;
+}
+}  // namespace
+
+extern "C" int gb_attention_decode_bf16_static(const void* q, int q_stride, void* out, int out_stride, const int32_t* positions,
+                                               const int32_t* tables, int table_stride, const void* k_pages,
+                                               const void* v_pages, int n_decode, int nh, int nkv, int hd, int page_size,
+                                               float scale, int window, int chunk, int max_context, hipStream_t stream) {
+  GB_REQUIRE(n_decode >= 0 && nh > 0 && hd > 0 && chunk > 0 && max_context > 0, "attention_decode_static: bad sizes");
+  const long long splits = ((long long)max_context + chunk - 1) / chunk;
+  const long long cells = (long long)n_decode * nh * splits;
+  float *ws_acc = nullptr, *ws_ml = nullptr;
+  if (splits > 1) {  // one chunk a request writes its result directly: nothing is kept between the kernels
+    GB_REQUIRE(cells * (hd + 2) <= (long long)GB_DECODE_STATIC_FLOATS,
+               "attention_decode_static: %d requests x %d heads x %lld chunks x (%d + 2) floats = %lld exceed the %lld floats "
+               "the library holds: use fewer chunks (a larger chunk), or gb_attention_decode_bf16 with a workspace",
+               n_decode, nh, splits, hd, cells * (hd + 2), (long long)GB_DECODE_STATIC_FLOATS);
+    float* base = nullptr;
+    if (int rc = static_scratch(&base)) return rc;
+    ws_acc = base;
+    ws_ml = base + cells * hd;  // cells * hd floats: a multiple of 16 floats, so still 64-byte aligned
+  }
+  return gb_attention_decode_bf16(q, q_stride, out, out_stride, ws_acc, ws_ml, positions, tables, table_stride, k_pages, v_pages,
+                                  n_decode, nh, nkv, hd, page_size, scale, window, chunk, max_context, stream);
 }
 
 // How the prompt portions of a step are spread over the chip.  A pair of blocks of 32 tokens is the unit of work.
