@@ -60,7 +60,16 @@ void CacheManager::release(Group& g, int32_t page) {
   if (--g.refs[page] == 0) {
     if (g.has_hash[page]) g.cached.push_back(page);
     else g.free.push_back(page);
+    // a copy into this page that the engine has not made yet is void: the page may be handed out again, as
+    // another copy's destination too, and two copies into one page would land in an undefined order
+    drop_copies_into((int)(&g - groups_.data()), page);
   }
+}
+
+void CacheManager::drop_copies_into(int group, int32_t dst) {
+  copies_.erase(std::remove_if(copies_.begin(), copies_.end(),
+                               [&](const CopyOp& c) { return c.group == group && c.dst == dst; }),
+                copies_.end());
 }
 
 void CacheManager::retain(Group& g, int32_t page) {
@@ -253,7 +262,10 @@ int CacheManager::remove_seq(int64_t id) {
   for (size_t gi = 0; gi < groups_.size(); ++gi)
     for (int32_t page : s.tables[gi])
       if (page >= 0) release(groups_[gi], page);
-  if (s.state_slot >= 0) free_slots_.push_back(s.state_slot);
+  if (s.state_slot >= 0) {
+    free_slots_.push_back(s.state_slot);
+    drop_copies_into(-1, s.state_slot);
+  }
   seqs_.erase(it);
   return 0;
 }

@@ -24,7 +24,7 @@ struct GroupSpec {
   int num_pages = 0;
 };
 
-struct CopyOp {        // device work the engine must do before the next step
+struct CopyOp {        // device work the engine must do before the next step; dropped if dst is given back first
   int group;           // >= 0: copy page src -> dst in every layer of the group
   int src;             //  -1 : copy state slot src -> dst
   int dst;
@@ -91,6 +91,7 @@ class CacheManager {
   int alloc(Group& g);
   void release(Group& g, int32_t page);
   void retain(Group& g, int32_t page);
+  void drop_copies_into(int group, int32_t dst);  // group -1: a state slot
   int need_in_group(const Seq& s, int gi, int n) const;
 
   int page_size_;

@@ -136,20 +136,33 @@ class Engine:
     def reserve(self, entries: Sequence[Entry]) -> None:
         """Makes room for every entry's tokens; raises OutOfPages when the pool is too small
         (entries reserved before the failing one keep their pages; nothing is written)."""
-        for request, tokens, _ in entries:
-            if request not in self._ids:
-                self.add_request(request)
-            self.cache.reserve(self._ids[request], len(tokens))
-        self._apply_copies()
+        added = []
+        try:
+            for request, tokens, _ in entries:
+                if request not in self._ids:
+                    self.add_request(request)
+                    added.append(request)
+                self.cache.reserve(self._ids[request], len(tokens))
+        except Exception:
+            for request in added:   # a step that did not happen leaves no request behind
+                self.end_request(request)
+            raise
+        finally:
+            self._apply_copies()    # also when a later entry found no room: what was asked for is not left pending
 
     def _apply_copies(self) -> None:
         copies = self.cache.take_copies()
         if not copies:
             return
-        by_group: Dict[int, List[Tuple[int, int]]] = {}
+        # one launch copies many pages at once, in no order: pairs go into one launch only while no page is both
+        # read and written in it (a source that was given back may come again as a later copy's destination)
+        batches: List[Tuple[int, List[Tuple[int, int]]]] = []
         for g, src, dst in copies:
-            by_group.setdefault(g, []).append((src, dst))
-        for g, pairs in by_group.items():
+            last = batches[-1] if batches else None
+            if (last is None or last[0] != g or any(dst == s or dst == d or src == d for s, d in last[1])):
+                batches.append((g, []))
+            batches[-1][1].append((src, dst))
+        for g, pairs in batches:
             src = torch.tensor([p[0] for p in pairs], dtype=torch.int32, device=self.device)
             dst = torch.tensor([p[1] for p in pairs], dtype=torch.int32, device=self.device)
             for lc in self.layers:

@@ -61,6 +61,54 @@ def test_fork_copies_on_write():
     kv.check_invariants()
 
 
+def test_a_copy_into_a_page_that_is_given_back_is_dropped():
+    """A copy that the engine has not made yet must not outlive its destination: the freed page is handed out
+    again (last in, first out), also as another copy's destination, and two copies into one page in one launch
+    would land in an undefined order."""
+    kv = full(3, share=False)
+    kv.add_seq(0, [])
+    kv.reserve(0, 3)
+    kv.commit(0, [1, 2, 3])
+    kv.fork(0, 1)
+    kv.fork(0, 2)
+    kv.reserve(1, 1)                      # copy-on-write: page of request 0 -> a fresh page
+    fresh = kv.table(1)[0]
+    kv.remove_seq(1)                      # ended between two steps, before the engine made the copy
+    kv.reserve(2, 1)                      # takes the same page again (the free list is last in, first out)
+    assert kv.table(2)[0] == fresh
+    assert kv.take_copies() == [(0, kv.table(0)[0], fresh)], "the dropped request's copy must be gone, this one kept"
+    kv.check_invariants()
+    # truncating to a page boundary gives the copied page back too
+    kv.fork(0, 3)
+    kv.reserve(3, 1)
+    kv.truncate(3, 0)
+    assert kv.take_copies() == []
+    # a state slot that is given back takes its pending copy with it
+    st = full(4, share=False, slots=2)
+    st.add_seq(0, [])
+    st.fork(0, 1)
+    st.remove_seq(1)
+    assert st.take_copies() == []
+    st.check_invariants()
+
+
+def test_reserve_that_fails_after_a_copy_on_write_elsewhere_leaves_that_copy_pending():
+    """Pool of exactly the pages needed: the second request of a step finds no room after the first one's
+    copy-on-write took the last page.  The first one's copy stays valid (its page stays reserved)."""
+    kv = full(2, share=False)
+    kv.add_seq(0, [])
+    kv.reserve(0, 3)
+    kv.commit(0, [1, 2, 3])
+    kv.fork(0, 1)
+    kv.fork(0, 2)
+    kv.reserve(1, 1)                      # the last free page
+    with pytest.raises(OutOfPages):
+        kv.reserve(2, 1)
+    assert kv.table(2) == kv.table(0), "a failed reserve changes nothing"
+    assert kv.take_copies() == [(0, kv.table(0)[0], kv.table(1)[0])]
+    kv.check_invariants()
+
+
 def test_the_whole_prompt_is_never_reused():
     # kv.rs:143: the last token always runs
     kv = full(8)
