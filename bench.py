@@ -2,15 +2,23 @@
 """Decode and prefill throughput of the engine on SmolLM2-1.7B shapes with random weights.
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--batch 8] [--context 4096] [--layers 24]
-                    [--shapes smollm2-1.7b|smollm2-360m|llama-3-8b]
+                    [--shapes smollm2-1.7b|smollm2-360m|llama-3-8b] [--reps 3]
 
-A step is one decode step of the whole batch through Engine.step and the device sampler, the
-sampled tokens fed back as the next step's input.  The batch is first prefilled (through the same
-step function, in portions of 2,048 tokens) so that the last timed step reaches the context length.
-Prints one JSON line.  One GPU only: for --gpus > 1 it says so and exits with 2.
+A step is one decode step of the whole batch through the path that generation uses: ``Engine.step`` (which
+replays steps of single tokens from HIP graphs) and the device sampler (``sampling.sample_rows``), the sampled
+tokens fed back as the next step's input.  The batch is first prefilled (through the same step function, in
+portions of 2,048 tokens) so that the last timed step reaches the context length.  K steps are timed ``--reps``
+times in a row, each time between synchronisations; ``ms_per_step`` and ``value`` are the mean over the
+repetitions and ``reps`` holds their spread.  ``points.decode_b<batch>_scheduler`` is the same workload as
+requests under ``Scheduler.step`` (plan, step, sample, finish).  Prints one JSON line.  One GPU only: for
+--gpus > 1 it says so and exits with 2.
 """
 import argparse
+import datetime
 import json
+import os
+import statistics
+import subprocess
 import sys
 import time
 
@@ -45,6 +53,8 @@ def main() -> int:
     ap.add_argument("--only", choices=["decode", "prefill"], default=None,
                     help="for profiling: run only the decode steps (after their prefill) or only the 2,048-token prefill")
     ap.add_argument("--no-graph", action="store_true", help="run decode steps without HIP graph replay")
+    ap.add_argument("--reps", type=int, default=3, help="times the K timed steps are repeated (mean and spread are reported)")
+    ap.add_argument("--no-scheduler", action="store_true", help="skip the figure through Scheduler.step")
     ap.add_argument("--prefill-tokens", type=int, default=PREFILL_TOKENS,
                     help="with --only prefill, for profiling: a prompt of another length than the 2,048 tokens of the record")
     a = ap.parse_args()
@@ -58,7 +68,8 @@ def main() -> int:
     import torch
     from glassbox_amd.config import config_from_dict
     from glassbox_amd.engine import Engine
-    from glassbox_amd.engine.decode_loop import DecodeLoop
+    from glassbox_amd.engine import Scheduler, SchedulerConfig
+    from glassbox_amd.sampling import SamplerConfig, sample_rows
     from glassbox_amd.weights import build_model, init_random
 
     MODEL = SHAPES[a.shapes]
@@ -67,7 +78,8 @@ def main() -> int:
     init_random(model, seed=0, dtype=a.dtype, device="cuda:0")
     batches = [a.batch] + ([] if a.no_points else [b for b in (1, 64) if b != a.batch])
     max_tokens = max(max(batches) * (a.context + 64), a.prefill_tokens + 64)
-    eng = Engine(model, dtype=a.dtype, max_tokens=max_tokens, max_seqs=max(batches), page_size=16)
+    eng = Engine(model, dtype=a.dtype, max_tokens=max_tokens, max_seqs=max(batches), page_size=16,
+                 graph_decode=False if a.no_graph else None)
     vocab = cfg.vocab_size
     g = torch.Generator().manual_seed(1)
 
@@ -104,44 +116,87 @@ def main() -> int:
         prefill = {"value": round(T / pf, 1), "tokens": T, "ms": round(pf * 1e3, 3),
                    "frac": round(pf_flops / pf / (peak * 1e12), 4)}
 
-    # ---- decode
-    def decode_run(batch, steps, warmup):
-        start = a.context - steps - warmup
+    # ---- decode: Engine.step and the device sampler, tokens fed back
+    def decode_run(batch, steps, warmup, reps):
+        start = a.context - reps * steps - warmup
         names = [f"d{batch}_{i}" for i in range(batch)]
         prompts = [torch.randint(0, vocab, (start,), generator=g).tolist() for _ in names]
         for at in range(0, start - 1, PREFILL_TOKENS):        # leave the last prompt token for the first decode step
             n = min(PREFILL_TOKENS, start - 1 - at)
             for name, p in zip(names, prompts):
                 eng.step([(name, p[at:at + n], [])])
-        loop = DecodeLoop(eng, names, [p[-1] for p in prompts], use_graph=not a.no_graph)
+        greedy_rows, uniforms = [SamplerConfig()] * batch, [0.0] * batch
+        tokens = [p[-1] for p in prompts]
+
+        def one_step():
+            nonlocal tokens
+            logits = eng.step([(name, [t], [0]) for name, t in zip(names, tokens)])
+            tokens, _ = sample_rows(logits, greedy_rows, uniforms)     # reads the tokens back: the step has ended
+
         for _ in range(warmup):
-            loop.step()
+            one_step()
+        times = []
+        for _ in range(reps):
+            torch.cuda.synchronize()
+            t0 = time.perf_counter()
+            for _ in range(steps):
+                one_step()
+            torch.cuda.synchronize()
+            times.append(time.perf_counter() - t0)
+        for name in names:
+            eng.end_request(name)
+        mean_ctx = a.context - (reps * steps + 1) / 2
+        return times, mean_ctx
+
+    # ---- the same workload as requests under the scheduler: plan, step, sample, finish
+    def scheduler_run(batch, steps, warmup):
+        slack = 4 * batch + 8          # tokens that the first requests decode while the last ones are still prompts
+        budget = warmup + steps + slack
+        start = a.context - budget
+        sched = Scheduler(eng, SchedulerConfig(token_budget=PREFILL_TOKENS, max_seqs=batch))
+        ids = [sched.submit(torch.randint(0, vocab, (start,), generator=g).tolist(), budget) for _ in range(batch)]
+        while not all(sched.outputs[i].tokens for i in ids):
+            sched.step()                                       # prompts, in portions under the token budget
+        for _ in range(warmup):
+            sched.step()
         torch.cuda.synchronize()
         t0 = time.perf_counter()
         for _ in range(steps):
-            loop.step()
+            sched.step()
         torch.cuda.synchronize()
         dt = time.perf_counter() - t0
-        loop.close()
-        for name in names:
-            eng.end_request(name)
-        mean_ctx = a.context - (steps + 1) / 2
-        return dt, mean_ctx
+        if sched.running() != batch:
+            raise RuntimeError("a request ended inside the timed steps of the scheduler figure")
+        for i in ids:
+            sched.abort(i)
+        return dt
 
-    dt, mean_ctx = decode_run(a.batch, a.steps, a.warmup)
-    step_s = dt / a.steps
+    times, mean_ctx = decode_run(a.batch, a.steps, a.warmup, a.reps)
+    step_s = statistics.mean(times) / a.steps
     value = a.batch / step_s
     bytes_step = weight_bytes + a.batch * mean_ctx * kv_bytes_per_token
     achieved = bytes_step / step_s / 1e9
     points = {}
+    if not a.no_scheduler:
+        sdt = scheduler_run(a.batch, a.steps, a.warmup)
+        points[f"decode_b{a.batch}_scheduler"] = round(a.batch * a.steps / sdt, 1)
     if not a.no_points:
         for b in (1, 64):
             if b == a.batch:
                 points[f"decode_b{b}"] = round(value, 1)
                 continue
             k = max(8, min(a.steps, 32))
-            pdt, _ = decode_run(b, k, min(a.warmup, 4))
-            points[f"decode_b{b}"] = round(b * k / pdt, 1)
+            pts, _ = decode_run(b, k, min(a.warmup, 4), 1)
+            points[f"decode_b{b}"] = round(b * k / pts[0], 1)
+
+    def commit():
+        here = os.path.dirname(os.path.abspath(__file__))
+        try:
+            r = subprocess.run(["git", "-C", here, "rev-parse", "--short", "HEAD"], capture_output=True, text=True, timeout=10)
+            return r.stdout.strip() or None
+        except (OSError, subprocess.SubprocessError):
+            return None
+    ms = [t / a.steps * 1e3 for t in times]
 
     out = {
         "metric": f"decode tok/s at batch {a.batch}, {NAMES[a.shapes]}, context {a.context} "
@@ -155,6 +210,11 @@ def main() -> int:
                    "rms_norm_eps": cfg.rms_norm_eps, "tied": cfg.tie_word_embeddings, "global_batch": a.batch,
                    "seq_len": a.context, "page_size": eng.page_size, "parallelism": "single GPU",
                    "graph": not a.no_graph},
+        "reps": {"n": a.reps, "ms_per_step": [round(m, 4) for m in ms], "mean_ms": round(statistics.mean(ms), 4),
+                 "sd_ms": round(statistics.stdev(ms), 4) if len(ms) > 1 else 0.0},
+        "meta": {"gpu": torch.cuda.get_device_name(0), "commit": commit(),
+                 "date": datetime.datetime.now(datetime.timezone.utc).strftime("%Y-%m-%dT%H:%M:%SZ"),
+                 "torch": torch.__version__, "path": "Engine.step + sampling.sample_rows"},
         "prefill": prefill,
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": PEAK["hbm_gbs"], "unit": "GB/s",
                      "frac": round(achieved / PEAK["hbm_gbs"], 4)},

@@ -29,7 +29,8 @@ _ARCH = "gfx950"
 
 HIP_FLAGS = [
     f"--offload-arch={_ARCH}", "-O3", "-std=c++17", "-fPIC", "-shared", "-fno-gpu-rdc",
-    # packed fp32 instructions off: some of their forms have given wrong results on these machines
+    # the compiler may not form packed fp32 instructions (v_pk_*_f32) from float code: some of their forms have
+    # given wrong results on gfx950 hardware, silently
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
     "-Wno-unused-result", "-Wno-unknown-warning-option",
 ]

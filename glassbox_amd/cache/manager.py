@@ -1,7 +1,7 @@
 """Python face of the host cache manager (csrc/host/cache_manager.cpp).
 
 The manager decides which pages of which pool belong to which request; it owns
-no device memory (``cache/pools.py`` does).  Requests are named by integers.
+no device memory (the engine holds the pages, ``engine/engine.py``).  Requests are named by integers.
 """
 from __future__ import annotations
 

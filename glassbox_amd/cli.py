@@ -24,6 +24,8 @@ USAGE = """
   glassbox bench single --model DIR [--dtype ...] [--label L] [--out FILE]      (pp512 / tg128, as glassbox-bench)
   glassbox bench serve  --model DIR [--dtype ...] [--workload chat|system|long] [--requests N] [--rates R,R,...]
                         [--blocks N] [--budget 512] [--max-seqs 32] [--out FILE]    (requests against the clock)
+  glassbox bench kernels [--shapes smollm2-1.7b|smollm2-360m|llama-3-8b] [--rows 1,8,64,...] [--dtype ...] [--out FILE]
+                        (each matrix product of a layer alone, as glassbox-bench kernels)
   glassbox replay   --model DIR --dtype D --out DIR --max-tokens N              (same as bin/trace_run)"""
 
 
@@ -274,6 +276,69 @@ def cmd_bench_serve(a) -> int:
     return 0
 
 
+KERNEL_SHAPES = {   # hidden, intermediate, query heads, kv heads, head size, vocabulary
+    "smollm2-1.7b": (2048, 8192, 32, 32, 64, 49152),
+    "smollm2-360m": (960, 2560, 15, 5, 64, 49152),
+    "llama-3-8b": (4096, 14336, 32, 8, 128, 128256),
+}
+
+
+def cmd_bench_kernels(a) -> int:
+    """The matrix products of one layer and of the head, each alone, at several numbers of rows: time, bytes of
+    weights a second and floating-point operations a second, as ``glassbox-bench kernels`` prints for the
+    reference's matmul (crates/glassbox-bench/src/main.rs:509-536).  Every product runs as the engine runs it
+    (bfloat16: with the workspace that lets it divide k; the feed-forward's first product with its SiLU-multiply
+    epilogue, the projections that end a part adding into the 32-bit residual).  The weights are rotated through
+    copies of more than 512 MB in all, so that no launch finds them in a cache."""
+    import torch
+    from . import ops
+    from .weights import compute_dtype
+    dt = compute_dtype(a.dtype)
+    d, inter, nh, nkv, hd, vocab = KERNEL_SHAPES[a.shapes]
+    rows_list = [int(r) for r in a.rows.replace(",", " ").split()]
+    products = [("qkv", (nh + 2 * nkv) * hd, d, "store"), ("o", d, nh * hd, "add"), ("gate_up", 2 * inter, d, "silu"),
+                ("down", d, inter, "add"), ("head", vocab, d, "f32")]
+    dev = torch.device("cuda:0")
+    results = []
+    print(f"{'product':8} {'N':>6} {'K':>6} {'rows':>5} {'us':>9} {'GB/s':>8} {'TFLOP/s':>8}")
+    for name, n_out, k, mode in products:
+        w_bytes = n_out * k * (2 if dt == torch.bfloat16 else 4)
+        copies = max(2, -(-(512 << 20) // w_bytes))
+        ws = [(torch.randn(n_out, k, device=dev) * 0.02).to(dt) for _ in range(copies)]
+        for m in rows_list:
+            x = (torch.randn(m, k, device=dev) * 0.5).to(dt)
+            silu = mode == "silu" and dt == torch.bfloat16
+            out_cols = n_out // 2 if silu else n_out
+            out = torch.zeros(m, out_cols, device=dev, dtype=torch.float32 if mode in ("add", "f32") else dt)
+            floats = ops.gemm_split_floats(m, n_out, k) if dt == torch.bfloat16 and m > 16 else 0
+            work = torch.empty(floats, device=dev, dtype=torch.float32) if floats else None
+
+            def run(i):
+                ops.gemm(x, ws[i % copies], out, accumulate=mode == "add", silu_mul=silu, workspace=work)
+            for i in range(3):
+                run(i)
+            iters = int(min(200, max(5, 2e11 / (2.0 * n_out * k * max(m, 64)))))
+            start, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            torch.cuda.synchronize()
+            start.record()
+            for i in range(iters):
+                run(i)
+            end.record()
+            torch.cuda.synchronize()
+            us = start.elapsed_time(end) * 1e3 / iters
+            res = {"product": name, "n": n_out, "k": k, "rows": m, "us": us, "weight_gb_s": w_bytes / us / 1e3,
+                   "tflop_s": 2.0 * n_out * k * m / us / 1e6}
+            results.append(res)
+            print(f"{name:8} {n_out:6} {k:6} {m:5} {us:9.1f} {res['weight_gb_s']:8.0f} {res['tflop_s']:8.1f}", flush=True)
+        del ws
+    if a.out:
+        with open(a.out, "w") as fh:
+            json.dump({"engine": "glassbox_amd", "shapes": a.shapes, "dtype": a.dtype, "results": results,
+                       "meta": {"gpu": torch.cuda.get_device_name(0),
+                                "date": time.strftime("%Y-%m-%dT%H:%M:%SZ", time.gmtime())}}, fh, indent=2)
+    return 0
+
+
 def main(argv=None) -> int:
     ap = argparse.ArgumentParser(prog="glassbox", usage=USAGE)
     sub = ap.add_subparsers(dest="cmd")
@@ -295,6 +360,11 @@ def main(argv=None) -> int:
     bv.add_argument("--rates", default="inf", help="requests a second, several separated by commas; inf = all at once")
     bv.add_argument("--blocks", type=int, default=4096); bv.add_argument("--budget", type=int, default=512)
     bv.add_argument("--max-seqs", type=int, default=32); bv.add_argument("--out", default=None)
+    bk = bsub.add_parser("kernels")
+    bk.add_argument("--shapes", default="smollm2-1.7b", choices=sorted(KERNEL_SHAPES))
+    bk.add_argument("--dtype", default="bfloat16", choices=["bfloat16", "bf16", "float32", "f32", "fp32"])
+    bk.add_argument("--rows", default="1,8,64,128,512,2048", help="numbers of rows, separated by commas")
+    bk.add_argument("--out", default=None)
     rp = sub.add_parser("replay"); _add_model(rp)
     rp.add_argument("--out", required=True); rp.add_argument("--max-tokens", type=int, required=True)
     a = ap.parse_args(argv)
@@ -308,6 +378,8 @@ def main(argv=None) -> int:
         return cmd_bench_single(a)
     if a.cmd == "bench" and a.bench_cmd == "serve":
         return cmd_bench_serve(a)
+    if a.cmd == "bench" and a.bench_cmd == "kernels":
+        return cmd_bench_kernels(a)
     if a.cmd == "replay":
         import os
         import subprocess

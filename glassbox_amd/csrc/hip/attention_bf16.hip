@@ -821,19 +821,15 @@ struct PrefillPlan {
   int per_group, split, parts;
 };
 inline PrefillPlan prefill_plan(int max_q_len, int max_context, int nh, int n_seqs, int hd) {
-  static const int forced = [] { const char* e = getenv("GB_PREFILL_SPLIT"); return e ? atoi(e) : 0; }();
-  static const int forced_parts = [] { const char* e = getenv("GB_PREFILL_PARTS"); return e ? atoi(e) : 0; }();
-  static const int forced_four = [] { const char* e = getenv("GB_PREFILL_FOUR"); return e ? atoi(e) : 0; }();
   const long long pairs = (long long)((max_q_len + 63) / 64) * nh * n_seqs;
   // measured (32 heads of 64: 2,048 tokens 47.9 -> 40.7 us, 3,072 tokens 88.6 -> 79.4 with two pairs of two waves
   // each in place of four pairs; from 4,096 tokens on no gain): four pairs a workgroup once each compute unit
   // has two such workgroups
-  const long long four = forced_four > 0 ? forced_four : hd <= 64 ? 2048 : 1024;
+  const long long four = hd <= 64 ? 2048 : 1024;
   PrefillPlan p{pairs >= four ? 4 : pairs >= 512 ? 2 : 1, 1, 1};
   if (hd <= 64) {
     p.split = 4 / p.per_group;
     if (p.per_group == 1 && pairs <= 128) p.split = 8;
-    if (forced == 1 || forced == 2 || forced == 4 || forced == 8) p.split = forced, p.per_group = forced == 8 ? 1 : 4 / forced;
   } else if (p.per_group < 4) {  // one block at a time: waves share keys only in a workgroup of one pair
     p.per_group = 1;
     p.split = pairs <= 128 ? 8 : 4;
@@ -844,7 +840,6 @@ inline PrefillPlan prefill_plan(int max_q_len, int max_context, int nh, int n_se
     int parts = (int)(256 / (pairs > 0 ? pairs : 1));
     parts = parts > 8 ? 8 : parts;
     while (parts > 1 && parts * 4 * 4 > tiles) --parts;
-    if (forced_parts >= 1 && forced_parts <= 8) parts = forced_parts;
     if (parts > 1) p.parts = parts, p.split = 4;
   }
   return p;

@@ -287,15 +287,10 @@ __global__ __launch_bounds__(256, WN == 2 ? 2 : 1) void gemm_tiled_kernel(const 
 // Tile of the workgroup, 128 x (64 WN), and the depth of the register prefetch.  128 x 128 re-reads
 // the operands least; 128 x 64 when that would leave compute units idle.  The wide tile's registers
 // allow two workgroups a compute unit only with one k-step of prefetch, the narrow tile's with two.
-// GB_TILED="wn,depth" overrides (for measurements).
 inline void tiled_plan(int M, int N, int* wn, int* depth) {
   const int blocks = ((M + 127) / 128) * ((N + 127) / 128);
   *wn = blocks < 384 ? 1 : 2;
   *depth = *wn == 1 ? 2 : 1;
-  if (const char* env = getenv("GB_TILED")) {
-    int b = 0, d = 0;
-    if (sscanf(env, "%d,%d", &b, &d) == 2 && (b == 1 || b == 2) && (d == 1 || d == 2)) *wn = b, *depth = d;
-  }
 }
 
 template <int EPI, typename CT>
@@ -556,13 +551,9 @@ __global__ __launch_bounds__(512, 1) void gemm_ring_kernel(const bf16* __restric
 }
 
 // The ring kernel pays where its tiles occupy at least three quarters of the compute units and the loads are whole
-// 16-byte pieces.  GB_RING=0 switches it off (for measurements).
-inline bool ring_on() {
-  static const bool on = [] { const char* e = getenv("GB_RING"); return !(e && e[0] == '0'); }();
-  return on;
-}
+// 16-byte pieces.
 inline bool ring_takes(const void* a, int lda, const void* w, int ldw, int K) {
-  return ring_on() && K % RBK == 0 && K >= RBK * RING_STAGES && lda % 8 == 0 && ldw % 8 == 0 && (uintptr_t)a % 16 == 0 &&
+  return K % RBK == 0 && K >= RBK * RING_STAGES && lda % 8 == 0 && ldw % 8 == 0 && (uintptr_t)a % 16 == 0 &&
          (uintptr_t)w % 16 == 0;
 }
 inline bool ring_pays(int epi, const void* a, int lda, const void* w, int ldw, int M, int N, int K) {
@@ -597,7 +588,7 @@ inline SplitPlan split_plan(int M, int N, int K) {
   SplitPlan p{M <= 64 ? 64 : 128, 1, 0, 0, false};
   // many rows, a long k and few 256 x 256 tiles (the down projection of a prompt portion): slices of k fill the
   // chip with the ring kernel's tiles once; a slice keeps 1,024 of k or more
-  if (ring_on() && M >= 1024 && K >= 4096 && K % TBK == 0 && N % 8 == 0) {
+  if (M >= 1024 && K >= 4096 && K % TBK == 0 && N % 8 == 0) {
     const int tiles = ((M + RBM - 1) / RBM) * ((N + RBN - 1) / RBN);
     int want = tiles < 192 ? 256 / tiles : 1;
     if (want > K / 1024) want = K / 1024;
@@ -1172,7 +1163,6 @@ int launch_fold(const void* a, int lda, const bf16* w, int ldw, CT* c, int ldc, 
 }
 
 // Waves per workgroup, loads in flight per wave and row tiles per workgroup.
-// GB_SKINNY="waves,iters,rowtiles" overrides (for measurements).
 inline void skinny_plan(int tiles, int K, int mt, int* waves, int* iters, int* rt) {
   // measured on SmolLM2-1.7B and Llama-3-8B shapes: sixteen waves a workgroup keep the most loads in
   // flight; two row tiles a workgroup halve the re-reading of A once that still leaves workgroups for
@@ -1182,15 +1172,6 @@ inline void skinny_plan(int tiles, int K, int mt, int* waves, int* iters, int* r
   *rt = tiles >= 384 ? 2 : 1;
   const int per_wave = (blocks + *waves - 1) / *waves;
   *iters = (mt == 1 && per_wave >= 2) ? 2 : 1;
-  if (const char* env = getenv("GB_SKINNY")) {
-    int wv = 0, it = 0, r = 0;
-    if (sscanf(env, "%d,%d,%d", &wv, &it, &r) == 3 && (wv == 4 || wv == 16) && (it == 1 || (it == 2 && mt == 1)) &&
-        (r == 1 || r == 2)) {
-      *waves = wv;
-      *iters = it;
-      *rt = r;
-    }
-  }
 }
 
 template <int MT, int EPI, bool RMS, typename CT>

@@ -12,7 +12,6 @@ from typing import Dict, List, Optional, Sequence, Tuple
 
 import torch
 
-from .. import ops
 
 
 class Workspace:
@@ -58,7 +57,7 @@ class Workspace:
 class StepContext:
     def __init__(self, *, device, dtype, page_size: int, workspace: Workspace, n: int, num_seqs: int,
                  token_ids, positions, tok_seq, slots: List[torch.Tensor], tables: List[torch.Tensor],
-                 q_start, q_len, pos0, state_slots, want, host: dict, attention_impl: str = "auto"):
+                 q_start, q_len, pos0, state_slots, want, host: dict, kernels: str = "auto"):
         self.device, self.dtype, self.page_size, self.workspace = device, dtype, page_size, workspace
         self.n, self.num_seqs = n, num_seqs
         self.token_ids, self.positions, self.tok_seq = token_ids, positions, tok_seq
@@ -68,10 +67,12 @@ class StepContext:
         #: per request, as Python lists: first row, rows, first position, state slot; and the step's shape
         #: (n_decode, max_q_len, max_context): for kernel selection and for parts written in Python
         self.host = host
-        self.attention_impl = attention_impl
-        #: whether norms may be computed inside the next matrix product (steps of few rows); "plain" turns
-        #: every fusion off, so that tests can compare the fused kernels with their separate twins
-        self.fuse_norms = attention_impl != "plain"
+        #: "auto": parts take their tuned and fused kernels where these apply; "plain": every part takes its plain
+        #: kernels, one per operation (the engine's ``kernels`` argument: tests compare the two)
+        self.kernels = kernels
+        self.tuned = kernels != "plain"
+        #: whether norms may be computed inside the matrix products around them
+        self.fuse_norms = self.tuned
         self.memo: dict = {}
 
     def buffer(self, name: str, shape, dtype) -> torch.Tensor:
@@ -85,22 +86,3 @@ class StepContext:
         if n_dec >= self.num_seqs:
             return None
         return (n_dec, self.q_start, self.q_len, self.pos0, n_dec, self.num_seqs - n_dec, int(self.host["max_q_len"]))
-
-    # -------------------------------------------------------------------------------
-    def attention(self, q: torch.Tensor, out: torch.Tensor, cache, n_heads: int, scale: float, window: int) -> None:
-        """Paged attention of every row of the step over its request's cache.
-
-        float32 always takes the plain kernel.  bfloat16 takes the tuned kernels where they apply:
-        requests with one row go to the split-context decode kernel, longer portions to the
-        matrix-core prefill kernel; ``attention_impl='plain'`` forces the plain kernel."""
-        tables = self.tables[cache.group]
-        impl = self.attention_impl
-        if self.dtype == torch.float32 or impl == "plain" or not ops.tuned_attention_supports(cache.k_pages, n_heads, window):
-            ops.attention_plain(q, out, self.positions, self.tok_seq, tables, cache.k_pages, cache.v_pages,
-                                n_heads, scale, window)
-            return
-        h = self.host
-        if h["n_decode"] > 0:
-            ops.attention_decode(q, out, self, cache, n_heads, scale, window)
-        if h["n_decode"] < self.num_seqs:
-            ops.attention_prefill(q, out, self, cache, n_heads, scale, window)

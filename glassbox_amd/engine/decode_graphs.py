@@ -21,6 +21,7 @@ from __future__ import annotations
 
 import contextlib
 import gc
+import weakref
 from collections import OrderedDict
 from typing import List, Sequence, Tuple
 
@@ -35,9 +36,9 @@ MAX_SHAPES = 64   # shapes kept (buffers and a graph each); the least recently u
 @contextlib.contextmanager
 def capture(graph: "torch.cuda.CUDAGraph"):
     """``torch.cuda.graph(graph)`` with the garbage collector held off.  A graph that dies synchronises the
-    device (torch's destructor does, on this platform), which no call may do while a stream captures: an
-    engine dropped earlier, which the collector frees when it pleases because engine and graphs refer to each
-    other, must not be freed in here.  Nothing in here drops a graph by itself."""
+    device (torch's destructor does, on this platform), which no call may do while a stream captures.  The
+    graphs of an engine die with it by reference count (they hold the engine weakly); the collector is held off
+    all the same, for graphs that a caller of torch keeps in a cycle of its own.  Nothing in here drops a graph."""
     was_on = gc.isenabled()
     gc.disable()
     try:
@@ -88,12 +89,14 @@ class _Shape:
         d_slots = [self.dev[off + g * rows:off + (g + 1) * rows] for g in range(G)]
         t0 = off + G * rows
         d_tables = [self.dev[t0 + g * rows * stride:t0 + (g + 1) * rows * stride].view(rows, stride) for g in range(G)]
+        # what never changes between the steps of this shape.  First positions and state slots do change: they are
+        # ``ctx.pos0`` and ``ctx.state_slots`` on the device, which is where a replayable part reads them
         host = {"q_start": list(range(rows)), "q_len": [1] * rows, "n_decode": rows, "max_q_len": 1,
-                "max_context": bucket, "graph": True}
+                "max_context": bucket, "graph": True, "pos0": None, "state_slots": None}
         self.ctx = StepContext(device=engine.device, dtype=engine.dtype, page_size=P, workspace=workspace, n=rows,
                                num_seqs=rows, token_ids=d[0], positions=d[1], tok_seq=d[2], slots=d_slots,
                                tables=d_tables, q_start=d[3], q_len=d[4], pos0=d[1], state_slots=d[5], want=d[6],
-                               host=host, attention_impl=engine.attention_impl)
+                               host=host, kernels=engine.kernels)
         self.copied = torch.cuda.Event()
         self.runs = 0
         self.graph = None
@@ -102,7 +105,9 @@ class _Shape:
 
 class DecodeGraphs:
     def __init__(self, engine):
-        self.engine = engine
+        # the engine owns this object; a weak reference back, so that the two are no cycle and the graphs die by
+        # reference count when the engine does (never at a moment of the garbage collector's choosing)
+        self._engine = weakref.ref(engine)
         #: buffers of its own: steps of other shapes make the engine's buffers grow, and a graph holds addresses
         self.workspace = Workspace(engine.device)
         self.shapes: "OrderedDict[Tuple[int, int], _Shape]" = OrderedDict()
@@ -113,8 +118,16 @@ class DecodeGraphs:
         """Whether the step is one token per request with the logits wanted after each."""
         return all(len(t) == 1 and list(w) == [0] for _, t, w in entries)
 
+    @property
+    def engine(self):
+        eng = self._engine()
+        if eng is None:
+            raise RuntimeError("the engine of these graphs is gone")
+        return eng
+
     def run(self, entries: Sequence[Tuple[int, List[int], List[int]]]) -> torch.Tensor:
-        eng, cache = self.engine, self.engine.cache
+        eng = self.engine
+        cache = eng.cache
         n = len(entries)
         sids = [e[0] for e in entries]
         longest = cache.max_len(sids) + 1

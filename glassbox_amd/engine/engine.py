@@ -14,7 +14,8 @@ import torch
 from .. import ops
 from ..cache.manager import FULL, CacheManager, GroupSpec, OutOfPages
 from ..parts.base import LayerCache
-from ..weights.loader import compute_dtype, load_model
+from ..config import config_from_dir
+from ..weights.loader import build_model, compute_dtype, load_weights
 from .context import StepContext, Workspace
 from .decode_graphs import DecodeGraphs
 
@@ -25,6 +26,22 @@ class EngineError(RuntimeError):
     pass
 
 
+def check_supported(model, dtype: torch.dtype, page_size: int) -> None:
+    """Raises EngineError, naming the sizes at fault, if the kernels would refuse this model at these settings
+    (``DecoderModel.refusals``: every part is asked).  Needs no GPU: an engine asks before it loads weights."""
+    lines = []
+    if page_size <= 0 or page_size % 16:
+        lines.append(f"page_size: {page_size} is not a positive multiple of 16")
+    if model.vocab_size > ops.MAX_VOCAB:
+        key = getattr(model, "arg_keys", {}).get("vocab")
+        lines.append("vocab" + (f" (config.json: {key})" if key else "") +
+                     f": {model.vocab_size} is above {ops.MAX_VOCAB}, the largest vocabulary the sampler takes")
+    lines += model.refusals(dtype, page_size)
+    if lines:
+        name = {torch.bfloat16: "bfloat16", torch.float32: "float32"}.get(dtype, str(dtype))
+        raise EngineError(f"this model cannot run in {name} with pages of {page_size}:\n  " + "\n  ".join(lines))
+
+
 class Engine:
     """model: a folder (config.json + model.safetensors) or a built and loaded model.
 
@@ -33,23 +50,30 @@ class Engine:
     reference, crates/glassbox-core/src/kv.rs:11).
     graph_decode: replay steps of one token per request from HIP graphs (engine.decode_graphs); by
     default where the arithmetic is bfloat16 and every part of the model allows it.
+    kernels: "auto", or "plain": every part takes its plain kernels, one per operation and nothing fused, which
+    is what the tuned kernels are compared with.
     """
 
     def __init__(self, model, dtype="bfloat16", max_tokens: int = 4096, max_seqs: int = 32, page_size: int = 16,
-                 prefix_caching: bool = False, device: str = "cuda:0", attention_impl: str = "auto",
+                 prefix_caching: bool = False, device: str = "cuda:0", kernels: str = "auto",
                  graph_decode: Optional[bool] = None):
         ops.require_gpu()
         self.dtype = compute_dtype(dtype)
         self.device = torch.device(device)
         torch.cuda.set_device(self.device)
-        if isinstance(model, (str, os.PathLike)):
-            model = load_model(str(model), self.dtype, self.device)
-        self.model = model
         self.page_size = int(page_size)
-        if self.page_size <= 0 or self.page_size % 16:
-            raise EngineError(f"page size {page_size} must be a positive multiple of 16")
+        if isinstance(model, (str, os.PathLike)):
+            folder = str(model)
+            model = build_model(config_from_dir(folder))
+            check_supported(model, self.dtype, self.page_size)      # before the weights are read
+            load_weights(model, os.path.join(folder, "model.safetensors"), self.dtype, self.device)
+        else:
+            check_supported(model, self.dtype, self.page_size)
+        self.model = model
         self.max_seqs = int(max_seqs)
-        self.attention_impl = attention_impl
+        if kernels not in ("auto", "plain"):
+            raise EngineError(f"kernels={kernels!r}: 'auto' (tuned and fused kernels where they apply) or 'plain'")
+        self.kernels = kernels
         num_pages = max(1, -(-int(max_tokens) // self.page_size))
 
         # page groups: cache layers whose mixers keep the same span of positions share page numbers
@@ -77,7 +101,9 @@ class Engine:
                 lc.v_pages = torch.zeros((num_pages + 1, spec.num_kv_heads, spec.head_dim, self.page_size),
                                          dtype=self.dtype, device=self.device)   # transposed: see ops._check_pages
             if state is not None:
-                lc.state = torch.zeros((self.max_seqs + 1,) + tuple(state.shape), dtype=state.dtype, device=self.device)
+                lc.state = torch.full((self.max_seqs + 1,) + tuple(state.shape), state.initial, dtype=state.dtype,
+                                      device=self.device)
+                lc.state_initial = state.initial
             self.layers.append(lc)
         self.spare_page, self.spare_state_slot = num_pages, self.max_seqs
 
@@ -105,10 +131,7 @@ class Engine:
         self._next_id += 1
         reused = self.cache.add_seq(sid, list(prompt))
         self._ids[request] = sid
-        slot = self.cache.state_slot(sid)
-        for lc in self.layers:
-            if lc.state is not None:
-                lc.state[slot].zero_()   # a fresh request starts from empty state
+        self.reset_state(sid)   # a fresh request starts from the state's initial value
         return reused
 
     def end_request(self, request: Hashable) -> None:
@@ -188,7 +211,7 @@ class Engine:
         self._validate(entries)
         self.reserve(entries)
         by_id = [(self._ids[r], t, w) for r, t, w in entries]
-        logits = self.run_reserved(by_id)
+        logits = self.run_reserved(by_id, validated=True)
         for sid, tokens, _ in by_id:
             self.cache.commit(sid, tokens)
         return logits
@@ -203,12 +226,13 @@ class Engine:
             if any(w < 0 or w >= len(tokens) for w in want):
                 raise EngineError(f"request {request!r}: wanted places must lie among its {len(tokens)} tokens")
 
-    def run_reserved(self, entries: Sequence[Tuple[int, List[int], List[int]]]) -> torch.Tensor:
+    def run_reserved(self, entries: Sequence[Tuple[int, List[int], List[int]]], validated: bool = False) -> torch.Tensor:
         """The step itself, on the cache manager's own request numbers: pages for the tokens are
         reserved already and nothing is committed (the scheduler does both around this call)."""
         if not entries:
             return torch.empty((0, self.model.vocab_size), dtype=torch.float32, device=self.device)
-        self._validate(entries)
+        if not validated:
+            self._validate(entries)
         self._apply_copies()
         self.steps += 1
         graphs = self.decode_graphs
@@ -218,11 +242,13 @@ class Engine:
         return self.model.forward(ctx, self.layers)
 
     def reset_state(self, sid: int) -> None:
-        """Empties the state slot of a request that starts (again) from its first token."""
+        """Sets the state slot of a request that starts (again) from its first token to its initial value."""
+        if not self.has_state:
+            return
         slot = self.cache.state_slot(sid)
         for lc in self.layers:
             if lc.state is not None and slot >= 0:
-                lc.state[slot].zero_()
+                lc.state[slot].fill_(lc.state_initial)
 
     # ---------------------------------------------------------------- metadata
     def _build_context(self, entries) -> StepContext:
@@ -277,4 +303,4 @@ class Engine:
                            num_seqs=S, token_ids=cut(0, n), positions=cut(n, n), tok_seq=cut(2 * n, n), slots=slots,
                            tables=tables, q_start=cut(3 * n, S), q_len=cut(3 * n + S, S), pos0=cut(3 * n + 2 * S, S),
                            state_slots=cut(3 * n + 3 * S, S), want=cut(3 * n + 4 * S, W), host=host,
-                           attention_impl=self.attention_impl)
+                           kernels=self.kernels)

@@ -34,7 +34,9 @@ def build_llama(cfg: LlamaConfig) -> DecoderModel:
     head = LMHead(cfg.vocab_size, d, tied_to=embedding if cfg.tie_word_embeddings else None)
     return DecoderModel(cfg, embedding, blocks, schedule, RMSNorm(d, cfg.rms_norm_eps), head,
                         # a tied checkpoint may still carry the head; the reference ignores it (load.rs:70-75)
-                        ignorable=("lm_head.weight",) if cfg.tie_word_embeddings else ())
+                        ignorable=("lm_head.weight",) if cfg.tie_word_embeddings else (),
+                        arg_keys={"width": "hidden_size", "intermediate": "intermediate_size", "head_dim": "head_dim",
+                                  "n_heads * head_dim": "num_attention_heads, head_dim", "vocab": "vocab_size"})
 
 
 register_architecture("LlamaForCausalLM", LlamaConfig, build_llama, model_type="llama")

@@ -455,6 +455,10 @@ def gemm_rope(a: torch.Tensor, w: torch.Tensor, qkv: torch.Tensor, n_heads: int,
 
 
 # ----------------------------------------------------------------------- attention
+MAX_HEAD_DIM = 256        # attention_plain.hip: a head's dimensions are held by one block of threads
+MAX_VOCAB = 1 << 20       # sampling.hip: a token id takes 20 bits of the (logit, token) key the sampler searches
+
+
 def attention_plain(q: torch.Tensor, out: torch.Tensor, positions: torch.Tensor, tok_seq: torch.Tensor,
                     tables: torch.Tensor, k_pages: torch.Tensor, v_pages: torch.Tensor, n_heads: int,
                     scale: float, window: int = 0) -> None:

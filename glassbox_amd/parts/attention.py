@@ -15,7 +15,26 @@ from typing import Dict, Optional
 import torch
 
 from .. import ops
-from .base import FULL, WINDOW, CacheSpec, LayerCache, Mixer, PositionEncoding, PreNormed, TensorSpec, emit_target, split_workspace
+from .base import (FULL, WINDOW, CacheSpec, LayerCache, Mixer, PositionEncoding, PreNormed, TensorSpec, emit_target,
+                   needs_multiple_of_8, split_workspace)
+
+
+def paged_attention(ctx, q: torch.Tensor, out: torch.Tensor, cache: LayerCache, n_heads: int, scale: float,
+                    window: int) -> None:
+    """Attention of every row of the step over its request's pages.
+
+    float32 always takes the plain kernel.  bfloat16 takes the tuned kernels where they apply: requests with
+    one row go to the split-context decode kernel, longer portions to the matrix-core prefill kernel; a step
+    with ``ctx.tuned`` off takes the plain kernel throughout."""
+    if ctx.dtype == torch.float32 or not ctx.tuned or not ops.tuned_attention_supports(cache.k_pages, n_heads, window):
+        ops.attention_plain(q, out, ctx.positions, ctx.tok_seq, ctx.tables[cache.group], cache.k_pages, cache.v_pages,
+                            n_heads, scale, window)
+        return
+    n_decode = ctx.host["n_decode"]
+    if n_decode > 0:
+        ops.attention_decode(q, out, ctx, cache, n_heads, scale, window)
+    if n_decode < ctx.num_seqs:
+        ops.attention_prefill(q, out, ctx, cache, n_heads, scale, window)
 
 
 class PagedAttention(Mixer):
@@ -59,6 +78,15 @@ class PagedAttention(Mixer):
             self.wqkv = torch.cat([tensors["q_proj.weight"], tensors["k_proj.weight"], tensors["v_proj.weight"]], 0)
         self.wo = tensors["o_proj.weight"].contiguous()
 
+    def streamed_matrices(self):
+        return [self.wqkv, self.wo]
+
+    def problems(self, dtype, page_size):
+        out = needs_multiple_of_8(dtype, "width", self.width) + needs_multiple_of_8(dtype, "n_heads * head_dim", self.q_dim)
+        if self.head_dim > ops.MAX_HEAD_DIM:
+            out.append(("head_dim", f"{self.head_dim} is above {ops.MAX_HEAD_DIM}, the largest head the attention kernels take"))
+        return out + self.position.problems(dtype, page_size)
+
     accepts_fused_norm = True
     accepts_emit_norm = True
 
@@ -91,7 +119,7 @@ class PagedAttention(Mixer):
                          workspace=None if norm is not None else split_workspace(ctx, n, rows, self.width))
             self.position.apply_and_store(ctx, qkv, self.n_heads, n_kv, self.head_dim, *store)
         att = ctx.buffer("att", (n, self.q_dim), ctx.dtype)
-        ctx.attention(qkv[:, :self.q_dim], att, cache, self.n_heads, self.scale, self.window)
+        paged_attention(ctx, qkv[:, :self.q_dim], att, cache, self.n_heads, self.scale, self.window)
         target, handed_on = emit_target(ctx, n, self.width, self.q_dim, emit, "mixer")
         ops.gemm(att, self.wo, residual, accumulate=True, emit=target,
                  workspace=split_workspace(ctx, n, self.width, self.q_dim))

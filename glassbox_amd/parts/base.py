@@ -18,6 +18,9 @@ Interfaces (all activations are [tokens, width] tensors on the device;
       .state_spec  -> StateSpec | None              fixed-size per-request state it needs
   FeedForward.forward(ctx, h, residual)             adds its output into ``residual`` (float32)
   Block.forward(ctx, x, cache)                      one layer: arrangement of the four above
+      .cache_spec() / .state_spec()                 what the cache layer it writes holds (from its mixer)
+  Part.streamed_matrices()                          tensors a step reads whole (the bytes of a decode step)
+  Part.problems(dtype, page_size)                   what the kernels would refuse, asked when the engine is built
   Part.replayable                                   class attribute: the part's launches may be replayed
                                                     from a HIP graph (see Part)
 
@@ -31,7 +34,7 @@ Optional, for steps of few rows (each part says by a class attribute whether it 
 from __future__ import annotations
 
 from dataclasses import dataclass
-from typing import Dict, Iterator, NamedTuple, Optional, Tuple
+from typing import Dict, Iterator, List, NamedTuple, Optional, Tuple
 
 import torch
 
@@ -64,9 +67,11 @@ class CacheSpec:
 
 @dataclass(frozen=True)
 class StateSpec:
-    """Fixed-size state of one layer for each live request (one slot per request)."""
+    """Fixed-size state of one layer for each live request (one slot per request).  A request that starts
+    from its first token finds every element of its slot at ``initial``."""
     shape: Tuple[int, ...]
     dtype: torch.dtype = torch.float32
+    initial: float = 0.0
 
 
 @dataclass
@@ -76,6 +81,7 @@ class LayerCache:
     v_pages: Optional[torch.Tensor] = None   # [pages, kv heads, head size, page size] (transposed)
     group: int = 0
     state: Optional[torch.Tensor] = None     # [slots, *state shape]
+    state_initial: float = 0.0               # what a slot holds when its request starts
     writable: bool = True                    # False: the layer reads another layer's cache
 
 
@@ -110,6 +116,33 @@ class Part:
         self.load(own)
         for cname, child in self.children().items():
             child.load_tree(tensors, f"{prefix}{cname}." if cname else prefix)
+
+    def streamed_matrices(self) -> List[torch.Tensor]:
+        """The tensors on the device that a step reads whole, whatever its tokens: what a decode step has to
+        stream from memory once (a table that is only gathered from is not among them).  By default those of the
+        children; a part with matrices of its own adds them."""
+        out: List[torch.Tensor] = []
+        for child in self.children().values():
+            out.extend(child.streamed_matrices())
+        return out
+
+    def problems(self, dtype: torch.dtype, page_size: int) -> List[Tuple[str, str]]:
+        """Why the kernels would refuse this part at these settings: pairs (name of the constructor argument,
+        what is wrong with it), empty if nothing is.  The engine asks once, before the first step, so that a
+        configuration the kernels do not take is refused when the engine is built and not after the weights
+        are loaded.  By default what the children say."""
+        out: List[Tuple[str, str]] = []
+        for child in self.children().values():
+            out.extend(child.problems(dtype, page_size))
+        return out
+
+
+def needs_multiple_of_8(dtype: torch.dtype, what: str, size: int) -> List[Tuple[str, str]]:
+    """The bfloat16 products load operands 16 bytes at a time: their inner size must be a multiple of 8."""
+    if dtype == torch.bfloat16 and size % 8:
+        return [(what, f"{size} is not a multiple of 8, which the bfloat16 matrix products need of their inner size "
+                       f"(the float32 path takes it)")]
+    return []
 
 
 class Norm(Part):
@@ -200,3 +233,19 @@ class Mixer(Part):
 class FeedForward(Part):
     def forward(self, ctx, h: torch.Tensor, residual: torch.Tensor) -> None:
         raise NotImplementedError
+
+
+class Block(Part):
+    """One layer: an arrangement of norms, a mixer and a feed-forward (or whatever else it is made of).  The
+    model asks the block, not its parts, what the cache layer it writes must hold."""
+
+    def forward(self, ctx, x: torch.Tensor, cache: Optional[LayerCache]) -> None:
+        raise NotImplementedError
+
+    def cache_spec(self) -> Optional[CacheSpec]:
+        """Paged keys and values this block writes, or None."""
+        return None
+
+    def state_spec(self) -> Optional[StateSpec]:
+        """Fixed-size state per request this block keeps, or None."""
+        return None

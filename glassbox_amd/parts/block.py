@@ -13,10 +13,10 @@ from __future__ import annotations
 
 from typing import Dict, Optional
 
-from .base import FeedForward, LayerCache, Mixer, Norm, Normed, Part
+from .base import Block, CacheSpec, FeedForward, LayerCache, Mixer, Norm, Normed, Part, StateSpec
 
 
-class PreNormBlock(Part):
+class PreNormBlock(Block):
     replayable = True
 
     def __init__(self, mixer_norm: Norm, mixer: Mixer, ffn_norm: Norm, ffn: FeedForward,
@@ -26,6 +26,12 @@ class PreNormBlock(Part):
 
     def children(self) -> Dict[str, Part]:
         return dict(zip(self.names, (self.mixer_norm, self.mixer, self.ffn_norm, self.ffn)))
+
+    def cache_spec(self) -> Optional[CacheSpec]:
+        return self.mixer.cache_spec
+
+    def state_spec(self) -> Optional[StateSpec]:
+        return self.mixer.state_spec
 
     def entry_norm(self, ctx, n: int):
         """``(gamma, eps)`` of the norm this block begins with, if the product that made the residual before

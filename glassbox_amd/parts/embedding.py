@@ -8,7 +8,7 @@ from typing import Dict, Optional
 import torch
 
 from .. import ops
-from .base import Part, TensorSpec
+from .base import Part, TensorSpec, needs_multiple_of_8
 
 
 class Embedding(Part):
@@ -45,6 +45,12 @@ class LMHead(Part):
 
     def matrix(self) -> torch.Tensor:
         return self.tied_to.table if self.tied_to is not None else self.weight
+
+    def streamed_matrices(self):
+        return [self.matrix()]
+
+    def problems(self, dtype, page_size):
+        return needs_multiple_of_8(dtype, "width", self.width)
 
     def forward(self, ctx, rows):
         logits = ctx.buffer("logits", (rows.shape[0], self.vocab), torch.float32)

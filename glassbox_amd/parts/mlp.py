@@ -7,7 +7,7 @@ from typing import Dict, Optional
 import torch
 
 from .. import ops
-from .base import FeedForward, PreNormed, TensorSpec, emit_target, split_workspace
+from .base import FeedForward, PreNormed, TensorSpec, emit_target, needs_multiple_of_8, split_workspace
 
 
 class SwiGLU(FeedForward):
@@ -26,6 +26,12 @@ class SwiGLU(FeedForward):
     def load(self, tensors):
         self.w_gate_up = torch.cat([tensors["gate_proj.weight"], tensors["up_proj.weight"]], 0)
         self.w_down = tensors["down_proj.weight"].contiguous()
+
+    def streamed_matrices(self):
+        return [self.w_gate_up, self.w_down]
+
+    def problems(self, dtype, page_size):
+        return needs_multiple_of_8(dtype, "width", self.width) + needs_multiple_of_8(dtype, "intermediate", self.intermediate)
 
     accepts_fused_norm = True
     accepts_emit_norm = True

@@ -31,8 +31,10 @@ class DecoderModel(Part):
 
     def __init__(self, config, embedding: Embedding, blocks: Sequence[Part], schedule: Sequence[LayerCall],
                  final_norm: Norm, head: LMHead, names=("model.embed_tokens", "model.layers.{}", "model.norm", "lm_head"),
-                 ignorable: Sequence[str] = ()):
+                 ignorable: Sequence[str] = (), arg_keys: Optional[Dict[str, str]] = None):
         self.config = config
+        #: constructor argument of a part -> the key of config.json that set it, for messages
+        self.arg_keys = dict(arg_keys or {})
         self.embedding, self.blocks, self.schedule = embedding, list(blocks), list(schedule)
         self.final_norm, self.head = final_norm, head
         self.names = tuple(names)
@@ -70,13 +72,11 @@ class DecoderModel(Part):
         self._owners = owners
 
     def cache_specs(self) -> List[Optional[CacheSpec]]:
-        """What each cache layer holds, from the mixer of the block that writes it."""
-        return [getattr(self.blocks[self.schedule[self._owners[c]].block].mixer, "cache_spec", None)
-                for c in range(self.num_cache_layers)]
+        """What each cache layer holds: the block that writes it says."""
+        return [self.blocks[self.schedule[self._owners[c]].block].cache_spec() for c in range(self.num_cache_layers)]
 
     def state_specs(self) -> List[Optional[StateSpec]]:
-        return [getattr(self.blocks[self.schedule[self._owners[c]].block].mixer, "state_spec", None)
-                for c in range(self.num_cache_layers)]
+        return [self.blocks[self.schedule[self._owners[c]].block].state_spec() for c in range(self.num_cache_layers)]
 
     # the step ---------------------------------------------------------------------
     def forward(self, ctx, caches: Sequence[LayerCache]) -> torch.Tensor:
@@ -105,16 +105,32 @@ class DecoderModel(Part):
         rows = self.final_norm.forward(ctx, x, rows=ctx.want, out_name="h_out")
         return self.head.forward(ctx, rows)
 
+    def streamed_matrices(self) -> List[torch.Tensor]:
+        """Every tensor a step reads whole, once each: those of the scheduled blocks (a block named twice, or a
+        table that two parts share, counts once) and of the head; each part says which are its own."""
+        seen, out = set(), []
+        parts = [self.blocks[call.block] for call in self.schedule] + [self.final_norm, self.head]
+        for part in parts:
+            for t in part.streamed_matrices():
+                if t.data_ptr() not in seen:
+                    seen.add(t.data_ptr())
+                    out.append(t)
+        return out
+
     def weight_bytes(self) -> int:
         """Bytes of the matrices a decode step reads once (model.rs:175-184: norm vectors excluded)."""
-        seen, total = set(), 0
-        for call in self.schedule:
-            blk = self.blocks[call.block]
-            for part in (getattr(blk, "mixer", None), getattr(blk, "ffn", None)):
-                for t in vars(part).values() if part is not None else ():
-                    if isinstance(t, torch.Tensor) and t.dim() == 2 and t.data_ptr() not in seen:
-                        seen.add(t.data_ptr())
-                        total += t.numel() * t.element_size()
-        head = self.head.matrix()
-        total += head.numel() * head.element_size()
-        return total
+        return sum(t.numel() * t.element_size() for t in self.streamed_matrices())
+
+    def refusals(self, dtype, page_size: int) -> List[str]:
+        """One line for each thing the kernels would refuse at these settings, every part asked
+        (``Part.problems``); a complaint that many layers share is given once, with the first layer that has it.
+        ``arg_keys`` (from the builder) says which key of config.json set a part's argument."""
+        seen, lines = set(), []
+        for name, part in self.children().items():
+            for arg, why in part.problems(dtype, page_size):
+                if (arg, why) in seen:
+                    continue
+                seen.add((arg, why))
+                key = self.arg_keys.get(arg)
+                lines.append(f"{name}: {arg}" + (f" (config.json: {key})" if key else "") + f": {why}")
+        return lines

@@ -29,3 +29,10 @@ def model_dirs(tmp_path_factory):
     import helpers
     base = tmp_path_factory.mktemp("models")
     return helpers.ModelDirs(str(base))
+
+
+@pytest.fixture(scope="session")
+def bf16_bound():
+    """The tolerance of bfloat16 engines with tuned kernels: see helpers.Bf16Bound."""
+    import helpers
+    return helpers.Bf16Bound()

@@ -61,10 +61,70 @@ def _load(folder: str):
 
 
 @functools.lru_cache(maxsize=None)
-def plain_logits(folder: str, tokens: Tuple[int, ...]) -> np.ndarray:
-    """Logits at every position by the plain implementation in float64."""
+def _load_rounded(folder: str):
+    """The folder's weights as a bfloat16 engine holds them: matrices rounded to bfloat16, vectors (stored in
+    32-bit) as they are."""
     cfg, w = _load(folder)
+    return cfg, {k: (v.bfloat16().float() if v.dim() == 2 else v) for k, v in w.items()}
+
+
+@functools.lru_cache(maxsize=None)
+def plain_logits(folder: str, tokens: Tuple[int, ...], rounded: bool = False) -> np.ndarray:
+    """Logits at every position by the plain implementation in float64.  ``rounded``: with the matrices rounded
+    to bfloat16 first, which is what a bfloat16 engine is given: what then differs is the engine's arithmetic."""
+    cfg, w = _load_rounded(folder) if rounded else _load(folder)
     return plain_llama.forward(w, cfg, list(tokens), torch.float64).numpy()
+
+
+def oracle(folder: str, tokens: Sequence[int], dtype: str) -> np.ndarray:
+    """What an engine of ``dtype`` is compared with: the plain implementation on the weights that engine holds."""
+    return plain_logits(folder, tuple(tokens), dtype == "bfloat16")
+
+
+#: float32: the engine's stated target, absolute.
+TOL_F32 = 1e-4
+#: bfloat16, the plain kernels (one per operation, nothing fused) against the plain implementation on the same
+#: rounded weights, relative to the request's largest logit: measured 1.4e-3 (two tiny layers) to 7.7e-3 (a layer
+#: 2,048 wide).  The tuned kernels are then held to twice the plain kernels' own error (``Bf16Bound``).
+TOL_BF16_PLAIN_REL = 1.5e-2
+
+
+def max_error(got: Dict[str, np.ndarray], folder: str, requests: Dict[str, List[int]], dtype: str) -> float:
+    return max(float(np.abs(got[r] - oracle(folder, t, dtype)).max()) for r, t in requests.items())
+
+
+class Bf16Bound:
+    """How far a bfloat16 engine may be from the plain implementation (float64, on the rounded weights): twice as
+    far as the engine with plain kernels is on the same requests run whole.  That engine computes every operation
+    by a kernel of its own, in bfloat16 with 32-bit sums like the tuned ones; what the tuned kernels add is the order
+    of their sums and their fusions, which must not cost more than the rounding itself.  The plain engine's own error
+    is bounded by ``TOL_BF16_PLAIN_REL``."""
+
+    def __init__(self):
+        self._made: Dict[Tuple, float] = {}
+
+    def get(self, folder: str, requests: Dict[str, List[int]], page_size: int = 16) -> float:
+        from glassbox_amd.engine import Engine
+        key = (folder, page_size, tuple(sorted((r, tuple(t)) for r, t in requests.items())))
+        if key not in self._made:
+            eng = Engine(folder, dtype="bfloat16", max_tokens=sum(len(t) + 64 for t in requests.values()), max_seqs=2,
+                         kernels="plain", page_size=page_size)
+            self._made[key] = self.measure(eng, requests, lambda r: oracle(folder, requests[r], "bfloat16"))
+        return self._made[key]
+
+    @staticmethod
+    def measure(plain_engine, requests: Dict[str, List[int]], want_of) -> float:
+        """Twice the largest error of ``plain_engine`` (bfloat16, plain kernels) over the requests run whole;
+        ``want_of(request)`` gives the plain implementation's logits."""
+        got = replay(plain_engine, schedule_whole(requests))
+        worst = 0.0
+        for r in requests:
+            want = want_of(r)
+            err = float(np.abs(got[r] - want).max())
+            limit = TOL_BF16_PLAIN_REL * max(1.0, float(np.abs(want).max()))
+            assert err <= limit, f"plain kernels in bfloat16, request {r}: {err:.3e} from the plain implementation (limit {limit:.3e})"
+            worst = max(worst, err)
+        return 2.0 * worst
 
 
 def random_tokens(vocab: int, n: int, seed: int) -> List[int]:

@@ -185,3 +185,57 @@ def test_bad_files(tmp_path):
     p.write_bytes(b"abc")
     with pytest.raises(WeightError, match="too short"):
         load_weights(build_model(cfg), str(p), torch.float32, "cpu")
+
+
+# ------------------------------------------------- what the kernels do not take is refused before weights are read
+@pytest.mark.parametrize("patch,dtype,words", [
+    (dict(hidden_size=60, head_dim=16), "bfloat16", ["hidden_size", "60", "multiple of 8"]),
+    (dict(intermediate_size=100), "bfloat16", ["intermediate_size", "100", "multiple of 8"]),
+    (dict(num_attention_heads=3, num_key_value_heads=1, head_dim=20), "bfloat16", ["num_attention_heads, head_dim", "60"]),
+    (dict(head_dim=264), "bfloat16", ["head_dim", "264", "256"]),
+    (dict(head_dim=264), "float32", ["head_dim", "264", "256"]),
+    (dict(vocab_size=(1 << 20) + 8), "bfloat16", ["vocab_size", "1048584"]),
+    (dict(vocab_size=(1 << 20) + 8), "float32", ["vocab_size", "1048584"]),
+])
+def test_sizes_the_kernels_refuse_are_refused_when_the_engine_is_built(patch, dtype, words):
+    """A configuration that LlamaConfig accepts but a kernel would refuse at the first step (an inner size of a
+    bfloat16 product that is no multiple of 8, a head above 256, a vocabulary above 2^20) is named when the engine
+    is built, with the key of config.json that set it.  No GPU and no weights are needed to find out."""
+    from glassbox_amd.engine.engine import EngineError, check_supported
+    from glassbox_amd.weights import compute_dtype
+    model = build_model(config_from_dict(dict(helpers.TINY_A, **patch)))
+    with pytest.raises(EngineError) as e:
+        check_supported(model, compute_dtype(dtype), 16)
+    for w in words:
+        assert w in str(e.value), str(e.value)
+    assert str(e.value).count("\n") == 1, "a complaint that every layer shares is given once"
+
+
+def test_what_only_bfloat16_refuses_runs_in_float32_and_page_sizes_are_checked():
+    from glassbox_amd.engine.engine import EngineError, check_supported
+    model = build_model(config_from_dict(dict(helpers.TINY_A, hidden_size=60, head_dim=16, intermediate_size=100)))
+    check_supported(model, torch.float32, 16)
+    with pytest.raises(EngineError) as e:
+        check_supported(model, torch.bfloat16, 16)
+    assert "hidden_size" in str(e.value) and "intermediate_size" in str(e.value)     # every complaint in one error
+    for name in ("A", "B", "C", "D", "M", "W"):
+        for dtype in (torch.float32, torch.bfloat16):
+            check_supported(build_model(config_from_dict(helpers.TINY[name])), dtype, 16)
+    with pytest.raises(EngineError, match="page_size"):
+        check_supported(build_model(config_from_dict(helpers.TINY_A)), torch.float32, 24)
+
+
+def test_the_bytes_of_a_decode_step_are_the_matrices_each_part_names():
+    """weight_bytes: every matrix a step reads whole, once (crates/glassbox-core/src/model.rs:175-184: norm vectors
+    are not counted): the parts say which, the model adds them up; a tied head is the embedding table, counted once,
+    an untied model's table is only gathered from and not counted."""
+    from glassbox_amd.weights import random_tensors
+    for name in ("A", "B"):
+        raw = helpers.TINY[name]
+        cfg = config_from_dict(raw)
+        model = build_model(cfg)
+        model.load_tree(random_tensors(model, 0))
+        d, I, L, V = cfg.hidden_size, cfg.intermediate_size, cfg.num_hidden_layers, cfg.vocab_size
+        per_layer = d * (cfg.q_dim + 2 * cfg.kv_dim) + cfg.q_dim * d + 3 * I * d
+        assert model.weight_bytes() == 4 * (L * per_layer + V * d)
+        assert len(model.streamed_matrices()) == 4 * L + 1

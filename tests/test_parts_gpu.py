@@ -130,9 +130,13 @@ def register_toy():
         """state <- decay * state + (1 - decay) * h_t ; out_t = state_t . W^T.  The state lives in the
         request's slot between steps.  Written with tensor operations: a toy, not a kernel."""
 
+        #: steps of one token per request read slots and rows from the context's device tensors only (below),
+        #: so the engine may replay them from a graph
+        replayable = True
+
         def __init__(self, width, decay):
             self.width, self.decay = width, decay
-            self.state_spec = StateSpec((width,), torch.float32)
+            self.state_spec = StateSpec((width,), torch.float32, initial=0.25)   # a request starts from 0.25, not 0
             self.w = None
 
         def tensor_specs(self) -> Dict[str, TensorSpec]:
@@ -141,8 +145,19 @@ def register_toy():
         def load(self, tensors):
             self.w = tensors["mix.weight"].float()
 
+        def streamed_matrices(self):
+            return [self.w]
+
         def forward(self, ctx, h, residual, cache):
             host = ctx.host
+            if host["max_q_len"] == 1:
+                # one row a request: all of them at once, slots taken from the device (a replayed step has no host
+                # lists; its filler rows share the engine's spare slot, whose contents nobody reads)
+                slots = ctx.state_slots.long()
+                st = self.decay * cache.state.index_select(0, slots) + (1 - self.decay) * h.float()
+                cache.state.index_copy_(0, slots, st)
+                residual += st @ self.w.T
+                return
             for s in range(ctx.num_seqs):
                 slot, a, n = host["state_slots"][s], host["q_start"][s], host["q_len"][s]
                 st = cache.state[slot]
@@ -201,7 +216,7 @@ def toy_plain(w, cfg, tokens):
     x = attn_block(x, 0, keep=True)
     p = "model.layers.1."
     h = plain.rms_norm(x, W[p + "input_layernorm.weight"], eps)
-    st, outs = torch.zeros(d, dtype=torch.float64), []
+    st, outs = torch.full((d,), 0.25, dtype=torch.float64), []
     for t in range(T):
         st = cfg["decay"] * st + (1 - cfg["decay"]) * h[t]
         outs.append(st @ W[p + "self_attn.mix.weight"].T)
@@ -237,12 +252,23 @@ def test_toy_architecture_registers_builds_and_steps(tmp_path, dtype):
                         (steps_mixed, peak)):
         eng = Engine(folder, dtype=dtype, max_tokens=pool, max_seqs=3)
         assert len(eng.group_keys) == 2 and eng.has_state      # all keys; a window of 6; and state slots
+        # every part of the toy says it can be replayed, the mixer with state included: bfloat16 steps of single
+        # tokens come from graphs
+        assert (eng.decode_graphs is not None) == (dtype == "bfloat16")
         got = helpers.replay(eng, steps)
         for r in requests:
             bad = helpers.first_bad(got[r], want[r], tol)
             assert bad is None, f"{r}: first wrong position {bad}"
         eng.cache.check_invariants()
         assert eng.cache.used_pages(0) == 0 and eng.cache.used_pages(1) == 0 and eng.cache.free_state_slots() == 3
+        if eng.decode_graphs is not None and steps is steps_mixed:
+            assert eng.decode_graphs.replays > 0, "the mixed schedule's single-token steps were not replayed"
+    # the bytes of a decode step: every matrix once, the block that runs twice and the tied table included once
+    model = eng.model
+    mats = model.streamed_matrices()
+    assert len({t.data_ptr() for t in mats}) == len(mats)
+    assert model.embedding.table.data_ptr() in {t.data_ptr() for t in mats}            # the tied head
+    assert model.weight_bytes() == sum(t.numel() * t.element_size() for t in mats)
     # pages of the windowed group went back while requests were still running
     eng = Engine(folder, dtype=dtype, max_tokens=512, max_seqs=3)
     eng.step([("w", requests["t2"], [])])

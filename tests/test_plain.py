@@ -154,6 +154,61 @@ def test_norm_weights_sit_where_they_should(tiny):
     assert torch.allclose(llama.forward(w2, cfg, toks), base * 3, rtol=1e-9)     # the final norm scales the logits
 
 
+def library_model(w, cfg, tokens):
+    """The whole model from library routines only (torch.nn.functional's rms_norm, linear,
+    scaled_dot_product_attention with a causal mask, silu, embedding), wired as the reference wires its layers
+    (crates/glassbox-core/src/model.rs:251-361).  The rotation has no library routine: it is the plain one, which
+    the known-vector tests above pin.  Shares nothing else with tests/plain."""
+    W = {k: v.double() for k, v in w.items()}
+    d, nh, nkv, hd, eps = cfg["hidden_size"], cfg["num_attention_heads"], cfg["num_key_value_heads"], cfg["head_dim"], cfg["rms_norm_eps"]
+    T = len(tokens)
+    x = F.embedding(torch.tensor(tokens), W["model.embed_tokens.weight"])
+    for i in range(cfg["num_hidden_layers"]):
+        p = f"model.layers.{i}."
+        h = F.rms_norm(x, (d,), W[p + "input_layernorm.weight"], eps)
+        q = F.linear(h, W[p + "self_attn.q_proj.weight"]).view(T, nh, hd)
+        k = F.linear(h, W[p + "self_attn.k_proj.weight"]).view(T, nkv, hd)
+        v = F.linear(h, W[p + "self_attn.v_proj.weight"]).view(T, nkv, hd)
+        q, k = llama.rope(q, range(T), cfg["rope_theta"]), llama.rope(k, range(T), cfg["rope_theta"])
+        k, v = k.repeat_interleave(nh // nkv, dim=1), v.repeat_interleave(nh // nkv, dim=1)   # query head h reads kv head h // group
+        att = F.scaled_dot_product_attention(q.transpose(0, 1), k.transpose(0, 1), v.transpose(0, 1), is_causal=True)
+        x = x + F.linear(att.transpose(0, 1).reshape(T, nh * hd), W[p + "self_attn.o_proj.weight"])
+        h = F.rms_norm(x, (d,), W[p + "post_attention_layernorm.weight"], eps)
+        x = x + F.linear(F.silu(F.linear(h, W[p + "mlp.gate_proj.weight"])) * F.linear(h, W[p + "mlp.up_proj.weight"]),
+                         W[p + "mlp.down_proj.weight"])
+    head = W["model.embed_tokens.weight"] if cfg["tie_word_embeddings"] else W["lm_head.weight"]
+    return F.linear(F.rms_norm(x, (d,), W["model.norm.weight"], eps), head)
+
+
+def test_the_whole_model_is_the_library_routines_wired_as_the_reference_wires_them(tiny):
+    """What pins the arrangement of a layer (which norm feeds what, where the residual is taken and added, how heads
+    are cut out of the stacked rows and grouped): the same model built from library routines.  A norm after the
+    mixer instead of before it, a residual taken from the normed rows, heads cut in another order, or keys shared
+    by the wrong query heads would each show."""
+    for name in ("A", "B"):
+        cfg, w = tiny[name]
+        toks = helpers.random_tokens(cfg["vocab_size"], 33, seed=4)
+        assert torch.allclose(llama.forward(w, cfg, toks), library_model(w, cfg, toks), atol=1e-10, rtol=0), name
+
+
+def test_dead_layers_leave_the_residual_alone(tiny):
+    """With the output projections at zero every layer adds nothing: the logits are the head of the normed
+    embeddings.  A layer that passed its normed rows on, or wrote its output over the residual, would change them."""
+    cfg, w = tiny["B"]
+    toks = helpers.random_tokens(cfg["vocab_size"], 9, seed=5)
+    dead = {k: (torch.zeros_like(v) if k.endswith(("o_proj.weight", "down_proj.weight")) else v) for k, v in w.items()}
+    x = w["model.embed_tokens.weight"].double()[torch.tensor(toks)]
+    want = F.linear(F.rms_norm(x, (cfg["hidden_size"],), w["model.norm.weight"].double(), cfg["rms_norm_eps"]), w["lm_head.weight"].double())
+    assert torch.allclose(llama.forward(dead, cfg, toks), want, atol=1e-12, rtol=0)
+    # one layer alive again: its contribution arrives through the later layers' residual, not through their norms
+    alive = dict(dead)
+    alive["model.layers.0.mlp.down_proj.weight"] = w["model.layers.0.mlp.down_proj.weight"]
+    h = F.rms_norm(x, (cfg["hidden_size"],), w["model.layers.0.post_attention_layernorm.weight"].double(), cfg["rms_norm_eps"])
+    x1 = x + llama.swiglu(h, *(w[f"model.layers.0.mlp.{n}_proj.weight"].double() for n in ("gate", "up", "down")))
+    want = F.linear(F.rms_norm(x1, (cfg["hidden_size"],), w["model.norm.weight"].double(), cfg["rms_norm_eps"]), w["lm_head.weight"].double())
+    assert torch.allclose(llama.forward(alive, cfg, toks), want, atol=1e-12, rtol=0)
+
+
 def test_float32_arithmetic_agrees_with_float64(tiny):
     cfg, w = tiny["B"]
     toks = helpers.random_tokens(cfg["vocab_size"], 40, seed=2)
