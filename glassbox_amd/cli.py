@@ -289,7 +289,8 @@ def cmd_bench_kernels(a) -> int:
     reference's matmul (crates/glassbox-bench/src/main.rs:509-536).  Every product runs as the engine runs it
     (bfloat16: with the workspace that lets it divide k; the feed-forward's first product with its SiLU-multiply
     epilogue, the projections that end a part adding into the 32-bit residual).  The weights are rotated through
-    copies of more than 512 MB in all, so that no launch finds them in a cache."""
+    copies of more than 512 MB in all, so that no launch finds them in a cache, and the launches are replayed from
+    a HIP graph, so that short kernels are not timed at the pace of their launches."""
     import torch
     from . import ops
     from .weights import compute_dtype
@@ -317,14 +318,23 @@ def cmd_bench_kernels(a) -> int:
                 ops.gemm(x, ws[i % copies], out, accumulate=mode == "add", silu_mul=silu, workspace=work)
             for i in range(3):
                 run(i)
-            iters = int(min(200, max(5, 2e11 / (2.0 * n_out * k * max(m, 64)))))
+            # the launches of a round are replayed from a graph: issued one by one from here, short kernels would be
+            # timed at the pace of their launches
+            iters = int(min(64, max(4, 2e11 / (2.0 * n_out * k * max(m, 64)))))
+            torch.cuda.synchronize()
+            graph = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(graph):
+                for i in range(iters):
+                    run(i)
+            graph.replay()
             start, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
             torch.cuda.synchronize()
             start.record()
-            for i in range(iters):
-                run(i)
+            for _ in range(3):
+                graph.replay()
             end.record()
             torch.cuda.synchronize()
+            iters *= 3
             us = start.elapsed_time(end) * 1e3 / iters
             res = {"product": name, "n": n_out, "k": k, "rows": m, "us": us, "weight_gb_s": w_bytes / us / 1e3,
                    "tflop_s": 2.0 * n_out * k * m / us / 1e6}

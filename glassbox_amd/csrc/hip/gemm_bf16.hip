@@ -354,7 +354,12 @@ __device__ __forceinline__ void lds_wait(bf16x8 (&fa)[NA], bf16x8 (&fb)[NB]) {
 #pragma unroll
   for (int j = 0; j < NB; ++j) asm volatile("" : "+v"(fb[j]));
 }
-template <int LEFT> __device__ __forceinline__ void vm_wait() { __builtin_amdgcn_s_waitcnt(0x0F70 | LEFT); }
+// waits until at most LEFT of this wave's loads from memory are on their way (the counter's six bits lie in two
+// places of the instruction's operand: bits 3:0 and 15:14; the other counters are left alone)
+template <int LEFT> __device__ __forceinline__ void vm_wait() {
+  static_assert(LEFT >= 0 && LEFT < 64, "the counter has six bits");
+  __builtin_amdgcn_s_waitcnt(0x0F70 | (LEFT & 15) | ((LEFT >> 4) << 14));
+}
 
 template <int EPI, typename CT>
 __global__ __launch_bounds__(512, 1) void gemm_ring_kernel(const bf16* __restrict__ a, int lda, const bf16* __restrict__ w, int ldw,
@@ -572,6 +577,222 @@ int launch_ring(const bf16* a, int lda, const bf16* w, int ldw, CT* c, int ldc, 
   return launched("gemm_bf16 (ring)");
 }
 
+// ----------------------------------------------------------------------- stream
+// Products of 17 to a few hundred rows (the mixed steps of serving: a portion of a prompt beside decoded tokens,
+// a new turn behind a long history).  They are bound by reading W once, like decoding, but A no longer fits a
+// wave's registers; and with the wide tiles above few workgroups exist, each with little on its way from memory
+// (a chip-wide 5 TB/s at 2 us of latency wants some 40 KB in flight on every compute unit).
+//
+// Here a workgroup owns all 128 rows of a row tile and only 32 or 64 rows of W (TN = 1, 2), so that even the QKV
+// product of a 2,048-wide model has a workgroup for most compute units without dividing k.  Four waves compute,
+// each 32 rows of A by all of the workgroup's columns.  Both operands go from memory straight into LDS
+// (global_load_lds, 16 bytes a lane) in k-steps of 64 through two rings: six stages of A (16 KB each; A comes
+// from the second-level cache, every workgroup reads the same rows), asked for by the computing waves, and 14 or 7
+// stages of W (4 or 8 KB each: some 50 KB on their way from memory per compute unit), asked for by a fifth wave
+// that does nothing else.  A wave's loads retire in the order of issue: if one wave asked for both, waiting for
+// a stage of A would also wait for every stage of W asked for before it, and W would be three k-steps ahead,
+// not thirteen.  A row of a k-step is 128 bytes = 8 pieces; piece p of row r lies at position p ^ (r & 7), which
+// spreads the 16-byte operand reads of a wave over all banks.  Waits are written by hand as in the ring kernel.
+constexpr int SBK = 64, SBM = 128, SA_STAGES = 6;
+// Measured on SmolLM2-1.7B shapes (each product alone, replayed from a graph): up to 64 rows the skinny kernel is as
+// fast or faster (it keeps A in registers); from about 200 rows on the wide tiles that divide k are (a workgroup here
+// reads two LDS operands for every MFMA); between, this kernel gains 10 to 25 %.
+constexpr int STREAM_MIN_ROWS = 64, STREAM_MAX_ROWS = 128;
+constexpr int SLA = SBM / 8 / 4;  // a computing wave's load instructions per stage of A (an instruction moves 8 rows x 8 pieces)
+template <int TN> struct StreamShape {
+  static constexpr int BN = 32 * TN, W_STAGES = TN == 1 ? 14 : 7, LW = BN / 8;  // LW: the loading wave's instructions per stage
+};
+
+template <int TN, int EPI, typename CT>
+__global__ __launch_bounds__(320, 1) void gemm_stream_kernel(const bf16* __restrict__ a, int lda, const bf16* __restrict__ w,
+                                                             int ldw, CT* __restrict__ c, int ldc, int M, int N, int K,
+                                                             int k_slice) {
+  using S = StreamShape<TN>;
+  constexpr int BN = S::BN, SW = S::W_STAGES, LW = S::LW, DA = SA_STAGES - 1, DW = SW - 1;
+  static_assert((DW - 1) * LW < 64 && (DA - 1) * SLA < 64, "a wave counts at most 63 loads on their way");
+  if (k_slice > 0) {  // split k: workgroup z of a tile sums its own slice of k into its own copy of C
+    const int z = blockIdx.z;
+    a += (size_t)z * k_slice;
+    w += (size_t)z * k_slice;
+    c += (size_t)z * M * ldc;
+    K = min(k_slice, K - z * k_slice);
+  }
+  __shared__ __attribute__((aligned(16))) bf16 As[SA_STAGES][SBM * SBK];
+  __shared__ __attribute__((aligned(16))) bf16 Ws[SW][BN * SBK];
+  const int tid = threadIdx.x, lane = tid % 64, wave = tid / 64;
+  const int bx = blockIdx.x, m0 = blockIdx.y * SBM;
+  const int half = N / 2;  // EPI_SILU_MUL: number of gate rows
+  const int steps = K / SBK;
+  // Every workgroup of a row tile reads the same rows of A.  If all walked k from 0 they would ask the same few
+  // channels of the second-level cache for the same lines at the same time; so each starts somewhere else and
+  // walks round (the order of a cell's sum depends on its column tile, never on the rows of the step).
+  const int rot = (int)((blockIdx.x * 13u + blockIdx.z * 5u) % (unsigned)steps);
+  auto k_of = [&](int step) {
+    const int t = step + rot;
+    return (t >= steps ? t - steps : t) * SBK;
+  };
+
+  if (wave == 4) {
+    // ------------------------------------------------------------ the wave that asks for W
+    // row of W behind row r of the workgroup's W tile; with EPI_SILU_MUL (TN = 2) the first 32 rows are gate rows
+    // and the second 32 the up rows that belong to them; rows beyond N are read from a row that exists
+    auto w_row = [&](int r) -> int {
+      if (EPI == EPI_SILU_MUL) {
+        const int n = bx * 32 + r % 32;
+        return n < half ? (r / 32 ? half + n : n) : 0;
+      }
+      return min(bx * BN + r, N - 1);
+    };
+    const bf16* wsrc[LW];
+#pragma unroll
+    for (int t = 0; t < LW; ++t) {
+      const int row = t * 8 + lane / 8, piece = (lane % 8) ^ (row & 7);
+      wsrc[t] = w + (size_t)w_row(row) * ldw + piece * 8;
+    }
+    auto load_w = [&](int step) {
+#pragma unroll
+      for (int t = 0; t < LW; ++t)
+        __builtin_amdgcn_global_load_lds((glb_void*)(wsrc[t] + k_of(step)), (lds_void*)&Ws[step % SW][t * 8 * SBK], 16, 0, 0);
+    };
+    for (int t = 0; t < DW && t < steps; ++t) load_w(t);
+    // stage 0 has landed once at most the loads asked for after it are on their way
+    if (steps >= DW)
+      vm_wait<(DW - 1) * LW>();
+    else
+      vm_wait<0>();
+    __builtin_amdgcn_s_barrier();
+    for (int s = 0; s < steps; ++s) {
+      // everybody has passed the barrier of k-step s - 1: the buffer of stage s - 1 is free
+      const bool more = s + DW < steps;
+      if (more) load_w(s + DW);
+      if (s + 1 < steps) {
+        if (more)
+          vm_wait<(DW - 1) * LW>();  // stage s + 1 has landed: only what was asked for after it is on its way
+        else
+          vm_wait<0>();
+        __builtin_amdgcn_s_barrier();
+      }
+    }
+    return;
+  }
+
+  // ---------------------------------------------------------------- the waves that compute
+  // a load instruction moves 8 rows x 8 pieces; rows beyond M are read from a row that exists
+  const bf16* asrc[SLA];
+#pragma unroll
+  for (int t = 0; t < SLA; ++t) {
+    const int row = (wave * SLA + t) * 8 + lane / 8, piece = (lane % 8) ^ (row & 7);
+    asrc[t] = a + (size_t)min(m0 + row, M - 1) * lda + piece * 8;
+  }
+  auto load_a = [&](int step) {
+#pragma unroll
+    for (int t = 0; t < SLA; ++t)
+      __builtin_amdgcn_global_load_lds((glb_void*)(asrc[t] + k_of(step)),
+                                       (lds_void*)&As[step % SA_STAGES][(wave * SLA + t) * 8 * SBK], 16, 0, 0);
+  };
+  f32x16 acc[TN];
+#pragma unroll
+  for (int j = 0; j < TN; ++j)
+#pragma unroll
+    for (int r = 0; r < 16; ++r) acc[j][r] = 0.f;
+
+  // operand of MFMA step kk (0..3): row lane % 32 of a 32-row tile, piece 2 kk + lane / 32
+  uint32_t off[4];
+#pragma unroll
+  for (int kk = 0; kk < 4; ++kk) off[kk] = 2 * ((lane % 32) * SBK + (((2 * kk + lane / 32) ^ (lane & 7)) * 8));
+  const uint32_t abase = (uint32_t)(uintptr_t)(lds_void*)&As[0][0] + 2 * wave * 32 * SBK;
+  const uint32_t wbase = (uint32_t)(uintptr_t)(lds_void*)&Ws[0][0];
+  constexpr uint32_t A_STAGE = 2 * SBM * SBK, W_STAGE = 2 * BN * SBK, TILE = 2 * 32 * SBK;
+
+  bf16x8 fa[2][4], fw[2][4 * TN];  // two sets: the operands of k-step s + 1 arrive under the MFMAs of k-step s
+  auto read_operands = [&](int s, int set) {
+#pragma unroll
+    for (int kk = 0; kk < 4; ++kk) {
+      fa[set][kk] = lds_read16(abase + (s % SA_STAGES) * A_STAGE + off[kk]);
+#pragma unroll
+      for (int j = 0; j < TN; ++j) fw[set][kk * TN + j] = lds_read16(wbase + (s % SW) * W_STAGE + j * TILE + off[kk]);
+    }
+  };
+  using Set0 = std::integral_constant<int, 0>;
+  using Set1 = std::integral_constant<int, 1>;
+
+  for (int t = 0; t < DA && t < steps; ++t) load_a(t);
+  if (steps >= DA)
+    vm_wait<(DA - 1) * SLA>();
+  else
+    vm_wait<0>();
+  __builtin_amdgcn_s_barrier();
+  read_operands(0, 0);
+  // k-step s, its operands in register set `mine`
+  auto step = [&](int s, auto mine) {
+    constexpr int set = decltype(mine)::value;
+    // everybody has passed the barrier of k-step s - 1: the buffer of stage s - 1 is free
+    const bool more = s + DA < steps;
+    if (more) load_a(s + DA);
+    lds_wait<0>(fa[set], fw[set]);  // all of this wave's reads of stage s have arrived
+    if (s + 1 < steps) {
+      if (more)
+        vm_wait<(DA - 1) * SLA>();  // this wave's part of stage s + 1 has landed
+      else
+        vm_wait<0>();
+      __builtin_amdgcn_s_barrier();
+      read_operands(s + 1, set ^ 1);
+    }
+#pragma unroll
+    for (int kk = 0; kk < 4; ++kk)
+#pragma unroll
+      for (int j = 0; j < TN; ++j) acc[j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa[set][kk], fw[set][kk * TN + j], acc[j], 0, 0, 0);
+  };
+  for (int s = 0; s < steps; s += 2) {
+    step(s, Set0{});
+    if (s + 1 < steps) step(s + 1, Set1{});
+  }
+
+  // accumulator layout of a 32x32 tile: lane holds column lane%32, rows 8*(r/4) + 4*(lane/32) + r%4
+  const int row0 = m0 + wave * 32 + 4 * (lane / 32);
+  if (EPI == EPI_SILU_MUL) {
+    const int gn = bx * 32 + lane % 32;
+    if (gn >= half) return;
+#pragma unroll
+    for (int r = 0; r < 16; ++r) {
+      const int gm = row0 + 8 * (r / 4) + r % 4;
+      const float g = acc[0][r], u = acc[TN - 1][r];
+      if (gm < M) c[(size_t)gm * ldc + gn] = (CT)(g / (1.0f + __expf(-g)) * u);
+    }
+    return;
+  }
+#pragma unroll
+  for (int j = 0; j < TN; ++j) {
+    const int gn = bx * BN + j * 32 + lane % 32;
+    if (gn >= N) continue;
+#pragma unroll
+    for (int r = 0; r < 16; ++r) {
+      const int gm = row0 + 8 * (r / 4) + r % 4;
+      if (gm < M) store_c<CT>(c + (size_t)gm * ldc + gn, acc[j][r], EPI == EPI_ACCUMULATE);
+    }
+  }
+}
+
+inline bool stream_takes(const void* a, int lda, const void* w, int ldw, int K) {
+  return K % SBK == 0 && lda % 8 == 0 && ldw % 8 == 0 && (uintptr_t)a % 16 == 0 && (uintptr_t)w % 16 == 0;
+}
+
+template <int EPI, typename CT>
+int launch_stream(const bf16* a, int lda, const bf16* w, int ldw, CT* c, int ldc, int M, int N, int K, int k_slice, int slices,
+                  hipStream_t stream) {
+  const int cols = EPI == EPI_SILU_MUL ? N / 2 : N;
+  // the SiLU-multiply needs a gate tile and its up tile in one wave; otherwise narrow tiles while they are few
+  const int tn = EPI == EPI_SILU_MUL ? 2 : ((cols + 31) / 32) * ((M + SBM - 1) / SBM) * slices > 512 ? 2 : 1;
+  const int bn = EPI == EPI_SILU_MUL ? 32 : 32 * tn;
+  const dim3 grid((cols + bn - 1) / bn, (M + SBM - 1) / SBM, slices), block(320);
+  GB_REQUIRE(grid.y <= 65535 && grid.z <= 65535, "gemm_bf16: M=%d needs more than 65535 row tiles", M);
+  if (tn == 2)
+    hipLaunchKernelGGL((gemm_stream_kernel<2, EPI, CT>), grid, block, 0, stream, a, lda, w, ldw, c, ldc, M, N, K, k_slice);
+  else if constexpr (EPI != EPI_SILU_MUL)
+    hipLaunchKernelGGL((gemm_stream_kernel<1, EPI, CT>), grid, block, 0, stream, a, lda, w, ldw, c, ldc, M, N, K, k_slice);
+  return launched("gemm_bf16 (stream)");
+}
+
 // ------------------------------------------------------------------------ split k
 // A product with few tiles (17 to a few hundred rows, or few rows of W) leaves most compute units idle
 // and, as a skinny product, makes every workgroup read all of A.  Here the tiled kernel's workgroups
@@ -582,10 +803,11 @@ struct SplitPlan {
   int bm, slices, k_slice;
   size_t floats;  // of workspace
   bool ring;      // the ring kernel's 256 x 256 tiles, if the operands allow (else the tiled kernel's, same slices)
+  bool stream;    // the stream kernel's 128 x 32 tiles, if the operands allow (else the tiled kernel's, same slices)
 };
 
 inline SplitPlan split_plan(int M, int N, int K) {
-  SplitPlan p{M <= 64 ? 64 : 128, 1, 0, 0, false};
+  SplitPlan p{M <= 64 ? 64 : 128, 1, 0, 0, false, false};
   // many rows, a long k and few 256 x 256 tiles (the down projection of a prompt portion): slices of k fill the
   // chip with the ring kernel's tiles once; a slice keeps 1,024 of k or more
   if (M >= 1024 && K >= 4096 && K % TBK == 0 && N % 8 == 0) {
@@ -603,6 +825,23 @@ inline SplitPlan split_plan(int M, int N, int K) {
       p.slices = 1, p.k_slice = 0;
     }
   }
+  if (M > STREAM_MIN_ROWS && M <= STREAM_MAX_ROWS && K % SBK == 0 && N % 8 == 0) {
+    // the stream kernel's range: its tiles are narrow, so only products with few rows of W divide k at all
+    // (the O and down projections); a slice keeps 512 of k or more
+    const int tiles = ((N + 31) / 32) * ((M + SBM - 1) / SBM);
+    if (tiles >= 128) return p;  // enough narrow tiles: no slices at all
+    if (K < 4096) {              // a long k (the down projection) is left to the wide tiles' slices below: measured faster
+      int want = (256 + tiles - 1) / tiles;
+      if (want > K / 512) want = K / 512;
+      if (want < 2) return p;
+      p.k_slice = ((K + want - 1) / want + SBK - 1) / SBK * SBK;
+      p.slices = (K + p.k_slice - 1) / p.k_slice;
+      if (p.slices < 2) return SplitPlan{p.bm, 1, 0, 0, false, false};
+      p.floats = (size_t)p.slices * M * N;
+      p.stream = true;
+      return p;
+    }
+  }
   const int tiles = ((N + 127) / 128) * ((M + p.bm - 1) / p.bm);
   if (tiles >= 192 || N % 8 != 0) return p;
   // measured on SmolLM2-1.7B shapes: a long k (the down projection) always gains; a short one where the
@@ -616,7 +855,7 @@ inline SplitPlan split_plan(int M, int N, int K) {
   if (want < 2) return p;
   p.k_slice = ((K + want - 1) / want + TBK - 1) / TBK * TBK;
   p.slices = (K + p.k_slice - 1) / p.k_slice;
-  if (p.slices < 2) return SplitPlan{p.bm, 1, 0, 0, false};
+  if (p.slices < 2) return SplitPlan{p.bm, 1, 0, 0, false, false};
   p.floats = (size_t)p.slices * M * N;
   return p;
 }
@@ -728,11 +967,15 @@ int launch_split(const bf16* a, int lda, const bf16* w, int ldw, CT* c, int ldc,
   const dim3 grid((N + 127) / 128, (M + plan.bm - 1) / plan.bm, plan.slices), block(256);
   const bool kfull = K % TBK == 0;
   const bool ring = plan.ring && ring_takes(a, lda, w, ldw, K);
+  const bool streams = plan.stream && stream_takes(a, lda, w, ldw, K);
+  if (streams) {
+    if (int rc = launch_stream<EPI_STORE, float>(a, lda, w, ldw, ws, N, M, N, K, plan.k_slice, plan.slices, stream)) return rc;
+  }
   if (ring)
     hipLaunchKernelGGL((gemm_ring_kernel<EPI_STORE, float>), dim3((N + RBN - 1) / RBN, (M + RBM - 1) / RBM, plan.slices), dim3(512),
                        0, stream, a, lda, w, ldw, ws, N, M, N, K, plan.k_slice);
 #define GB_S(WM, FULL)                                                                                                   \
-  if (!ring && (plan.bm == 64 * WM) && kfull == FULL)                                                                    \
+  if (!ring && !streams && (plan.bm == 64 * WM) && kfull == FULL)                                                                   \
     hipLaunchKernelGGL((gemm_tiled_kernel<WM, 2, 1, EPI_STORE, FULL, float>), grid, block, 0, stream, a, lda, w, ldw, ws, \
                        N, M, N, K, plan.k_slice);
   GB_S(1, true) GB_S(1, false) GB_S(2, true) GB_S(2, false)
@@ -1270,7 +1513,21 @@ extern "C" int gb_gemm_bf16(const void* a, int lda, const void* w, int ldw, void
 #undef GB_SP
     }
   }
-  if (M <= 64) {
+  if (M > STREAM_MIN_ROWS && M <= STREAM_MAX_ROWS && !gamma && !parts && !emit_h && stream_takes(a, lda, w, ldw, K) &&
+      (epilogue != EPI_SILU_MUL || N % 16 == 0) && ((ncols + 31) / 32) * ((M + SBM - 1) / SBM) >= 128) {
+    const bf16* A = (const bf16*)a;
+#define GB_ST(EPI, CT) return launch_stream<EPI, CT>(A, lda, W, ldw, (CT*)c, ldc, M, N, K, 0, 1, stream)
+    if (epilogue == EPI_ACCUMULATE) GB_ST(EPI_ACCUMULATE, float);
+    if (epilogue == EPI_SILU_MUL && c_dtype == kBF16) GB_ST(EPI_SILU_MUL, bf16);
+    if (epilogue == EPI_SILU_MUL) GB_ST(EPI_SILU_MUL, float);
+    if (c_dtype == kF32) GB_ST(EPI_STORE, float);
+    GB_ST(EPI_STORE, bf16);
+#undef GB_ST
+  }
+  // 33 to 64 rows by very many rows of W (the vocabulary product of a large decode batch): measured twice as fast
+  // through the tiles below as through the skinny kernel with four column blocks (49,152 x 2,048: 102 -> about 50 us)
+  const bool wide_head = M > 32 && N >= 32768 && !gamma && !parts;
+  if (M <= 64 && !wide_head) {
     const int gf = gamma_dtype == kF32;
     if (fold_pays(M, N) && epilogue != EPI_SILU_MUL && !parts) {
       if (gamma) return launch_fold<EPI_STORE, true, bf16>(a, lda, W, ldw, (bf16*)c, ldc, M, N, K, gamma, gf, eps, extra, stream);

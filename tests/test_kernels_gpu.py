@@ -215,12 +215,13 @@ def test_gemm_bf16_that_divides_k_does_the_next_norm(M, N, K, gamma_dtype):
         ops.gemm(to_dev(a), to_dev(w), res, accumulate=True, emit=(to_dev(g), h, eps))       # no workspace
 
 
-@pytest.mark.parametrize("M,N,K", [(17, 96, 4096), (33, 2048, 2048), (64, 2048, 8192), (64, 6144, 2048), (100, 2048, 4160),
-                                   (200, 528, 8200), (64, 16384, 2048), (40, 1008, 4104), (512, 2048, 8192),
+@pytest.mark.parametrize("M,N,K", [(17, 96, 4096), (33, 2048, 2048), (64, 2048, 8192), (100, 2048, 4160),
+                                   # a k that is no multiple of 64: the tiled kernel's slices
+                                   (200, 528, 8200), (40, 1008, 4104),
                                    # a thousand rows and more: slices of k through the 256 x 256 tiles
                                    (2048, 2048, 8192), (1100, 1008, 4160), (1024, 528, 5120),
                                    # some hundred rows, a k of 2,048 and very few tiles
-                                   (128, 2048, 2048), (512, 2048, 2048), (300, 1008, 2112)])
+                                   (128, 2048, 2048), (300, 1008, 2112), (256, 1024, 2048)])
 @pytest.mark.parametrize("mode", ["bf16", "f32", "f32+", "silu"])
 def test_gemm_bf16_divides_k_over_workgroups(M, N, K, mode):
     """With a workspace, a product of few tiles has several workgroups a tile, each over a slice of k,
@@ -250,6 +251,46 @@ def test_gemm_bf16_divides_k_over_workgroups(M, N, K, mode):
     assert torch.equal(outs[0], outs[1])
     with pytest.raises(ops.KernelError, match="workspace"):
         ops.gemm(to_dev(a), to_dev(w), outs[0], accumulate=(mode == "f32+"), silu_mul=(mode == "silu"), workspace=ws[:8])
+
+
+@pytest.mark.parametrize("M,N,K", [(65, 6144, 2048), (128, 16384, 2048), (96, 4096, 8192),
+                                   # one, two, three k-steps: fewer than either ring is deep; and more than both
+                                   (100, 4096, 64), (128, 4128, 128), (100, 5000, 192), (70, 4100, 1024), (128, 8200, 1088),
+                                   # so many narrow tiles that a workgroup takes 64 columns
+                                   (128, 24600, 320), (96, 49152, 512),
+                                   # 33 to 64 rows by very many rows of W: the wide tiles, not the skinny kernel
+                                   (64, 49152, 256), (40, 33000, 192)])
+@pytest.mark.parametrize("mode", ["bf16", "f32", "f32+", "silu"])
+def test_gemm_bf16_streams_products_of_some_hundred_rows(M, N, K, mode):
+    """65 to 128 rows, a k that is a multiple of 64: tiles of 128 rows by 32 or 64 columns, both operands through
+    rings in LDS, no slices of k where the narrow tiles alone fill the chip (with or without a workspace on offer).
+    Against float64, the same bits on every run, rows and columns beyond the last tile's edge untouched."""
+    from glassbox_amd import ops
+    if mode == "silu" and N % 16:
+        N -= N % 16
+    assert ops.gemm_split_floats(M, N, K) == 0
+    a, w = rnd(M, K, seed=1).bfloat16(), (rnd(N, K, seed=2) / math.sqrt(K)).bfloat16()
+    c0 = rnd(M, N, seed=3)
+    prod = a.double() @ w.double().T
+    if mode == "silu":
+        want = prod[:, :N // 2] / (1 + torch.exp(-prod[:, :N // 2])) * prod[:, N // 2:]
+    else:
+        want = prod + (c0.double() if mode == "f32+" else 0)
+    cols = want.shape[1]
+    outs = []
+    for _ in range(2):
+        # a frame of untouched cells around the result: two more rows, a longer row stride
+        dtype = torch.float32 if mode in ("f32", "f32+") else torch.bfloat16
+        frame = torch.full((M + 2, cols + 8), 7.0, device=DEV, dtype=dtype)
+        c = frame[:M, :cols]
+        if mode == "f32+":
+            c.copy_(to_dev(c0))
+        ops.gemm(to_dev(a), to_dev(w), c, accumulate=(mode == "f32+"), silu_mul=(mode == "silu"))
+        assert (frame[M:] == 7.0).all() and (frame[:, cols:] == 7.0).all()
+        outs.append(c.clone())
+    tol = 1e-4 * math.sqrt(K) + (2 ** -8) * want.abs().max().item() * (mode in ("bf16", "silu"))
+    assert (outs[0].cpu().double() - want).abs().max().item() <= tol
+    assert torch.equal(outs[0], outs[1])
 
 
 def test_gemm_bf16_split_k_is_the_same_on_every_run():
