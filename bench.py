@@ -50,8 +50,11 @@ def main() -> int:
     ap.add_argument("--layers", type=int, default=None, help="fewer layers than the model has (both numbers are reported)")
     ap.add_argument("--dtype", default="bfloat16", choices=["bfloat16", "float32"])
     ap.add_argument("--no-points", action="store_true", help="skip the batch 1 and 64 points")
-    ap.add_argument("--only", choices=["decode", "prefill"], default=None,
-                    help="for profiling: run only the decode steps (after their prefill) or only the 2,048-token prefill")
+    ap.add_argument("--only", choices=["decode", "prefill", "portion"], default=None,
+                    help="for profiling: run only the decode steps (after their prefill), only the 2,048-token prefill, or "
+                         "only a portion of --portion-tokens tokens behind a cached context of --context tokens (a new "
+                         "turn behind a long history, the tail of a prompt)")
+    ap.add_argument("--portion-tokens", type=int, default=128)
     ap.add_argument("--no-graph", action="store_true", help="run decode steps without HIP graph replay")
     ap.add_argument("--reps", type=int, default=3, help="times the K timed steps are repeated (mean and spread are reported)")
     ap.add_argument("--no-scheduler", action="store_true", help="skip the figure through Scheduler.step")
@@ -99,6 +102,23 @@ def main() -> int:
         dt = time.perf_counter() - t0
         eng.end_request(name)
         return dt
+    if a.only == "portion":
+        # a step of a few hundred rows: the history is cached in portions of 2,048, then the timed step brings the rest
+        hist = a.context - a.portion_tokens
+        times = []
+        for rep in range(4):
+            toks = torch.randint(0, vocab, (a.context,), generator=g).tolist()
+            for at in range(0, hist, PREFILL_TOKENS):
+                eng.step([("p", toks[at:min(at + PREFILL_TOKENS, hist)], [])])
+            torch.cuda.synchronize()
+            t0 = time.perf_counter()
+            eng.step([("p", toks[hist:], [a.portion_tokens - 1])])
+            torch.cuda.synchronize()
+            times.append(time.perf_counter() - t0)
+            eng.end_request("p")
+        print(json.dumps({"portion_ms": round(min(times[1:]) * 1e3, 3), "tokens": a.portion_tokens, "context": a.context,
+                          "all_ms": [round(t * 1e3, 3) for t in times]}))
+        return 0
     if a.only == "decode":
         pf = float("nan")
     else:

@@ -1514,7 +1514,7 @@ extern "C" int gb_gemm_bf16(const void* a, int lda, const void* w, int ldw, void
     }
   }
   if (M > STREAM_MIN_ROWS && M <= STREAM_MAX_ROWS && !gamma && !parts && !emit_h && stream_takes(a, lda, w, ldw, K) &&
-      (epilogue != EPI_SILU_MUL || N % 16 == 0) && ((ncols + 31) / 32) * ((M + SBM - 1) / SBM) >= 128) {
+      (epilogue != EPI_SILU_MUL || N % 16 == 0) && ((ncols + 31) / 32) * ((M + SBM - 1) / SBM) >= 128 && N < 32768) {
     const bf16* A = (const bf16*)a;
 #define GB_ST(EPI, CT) return launch_stream<EPI, CT>(A, lda, W, ldw, (CT*)c, ldc, M, N, K, 0, 1, stream)
     if (epilogue == EPI_ACCUMULATE) GB_ST(EPI_ACCUMULATE, float);
