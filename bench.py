@@ -229,7 +229,7 @@ def main() -> int:
                    "head_dim": cfg.head_size, "intermediate": I, "vocab": vocab, "rope_theta": cfg.rope_theta,
                    "rms_norm_eps": cfg.rms_norm_eps, "tied": cfg.tie_word_embeddings, "global_batch": a.batch,
                    "seq_len": a.context, "page_size": eng.page_size, "parallelism": "single GPU",
-                   "graph": not a.no_graph},
+                   "graph": eng.decode_graphs is not None},
         "reps": {"n": a.reps, "ms_per_step": [round(m, 4) for m in ms], "mean_ms": round(statistics.mean(ms), 4),
                  "sd_ms": round(statistics.stdev(ms), 4) if len(ms) > 1 else 0.0},
         "meta": {"gpu": torch.cuda.get_device_name(0), "commit": commit(),
