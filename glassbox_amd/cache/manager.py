@@ -98,6 +98,7 @@ class CacheManager:
             page_size, n, mk([g.kind for g in groups]), mk([g.window for g in groups]),
             mk([g.num_pages for g in groups]), num_state_slots, 1 if share_prefixes else 0))
         self._table_buf = (C.c_int32 * 64)()
+        self._copies_buf = (C.c_int32 * (3 * 64))()
 
     def __del__(self):
         h, self._h = getattr(self, "_h", None), None
@@ -239,8 +240,10 @@ class CacheManager:
 
     def take_copies(self) -> List[Tuple[int, int, int]]:
         """Pending device copies (group, src, dst); group -1 means a state slot."""
-        buf = (C.c_int32 * (3 * 64))()
+        buf = self._copies_buf
         n = self._lib.gbh_cache_take_copies(self._h, buf, 64)
+        if n == 0:
+            return []
         if n > 64:
             raise CacheError("more pending copies than the buffer holds")
         return [(buf[3 * i], buf[3 * i + 1], buf[3 * i + 2]) for i in range(n)]

@@ -362,7 +362,7 @@ template <int LEFT> __device__ __forceinline__ void vm_wait() {
 }
 
 template <int EPI, typename CT>
-__global__ __launch_bounds__(512, 1) void gemm_ring_kernel(const bf16* __restrict__ a, int lda, const bf16* __restrict__ w, int ldw,
+__global__ __launch_bounds__(RGM * RGN * 64, 1) void gemm_ring_kernel(const bf16* __restrict__ a, int lda, const bf16* __restrict__ w, int ldw,
                                                            CT* __restrict__ c, int ldc, int M, int N, int K, int k_slice) {
   int bx = blockIdx.x, by = blockIdx.y;
   if (k_slice > 0) {  // split k: workgroup z of a tile sums its own slice of k into its own copy of C
@@ -393,8 +393,9 @@ __global__ __launch_bounds__(512, 1) void gemm_ring_kernel(const bf16* __restric
   // first column tile holds gate rows and its second the up rows that belong to them
   auto w_row = [&](int r) -> int {
     if (EPI == EPI_SILU_MUL) {
-      const int n = bx * (RBN / 2) + (r / 64) * 32 + r % 32;
-      return n < half ? ((r % 64) / 32 ? half + n : n) : 0;
+      const int j = (r % (RTN * 32)) / 32;  // column tile of its wave: even ones hold gate rows, odd ones their up rows
+      const int n = bx * (RBN / 2) + (r / (RTN * 32)) * (RTN / 2 * 32) + (j / 2) * 32 + r % 32;
+      return n < half ? (j % 2 ? half + n : n) : 0;
     }
     return min(bx * RBN + r, N - 1);
   };
@@ -466,7 +467,7 @@ __global__ __launch_bounds__(512, 1) void gemm_ring_kernel(const bf16* __restric
   // between the two MFMA steps: by then this wave has read all it needs of stage s, and once every wave has,
   // stage s + 1 (whose loads were waited for) may be read and the buffer of stage s overwritten (by the loads of
   // k-step s + 1).  So the first operands of k-step s + 1 arrive under the second MFMA step of k-step s.
-  static_assert(RLPS == 4 && RING_STAGES == 4, "the wait counts below are written for four loads a stage, four stages");
+  static_assert(RING_STAGES == 4 && RLPS % 2 == 0, "the wait counts below are written for four stages and an even number of loads a stage");
   auto step = [&](int s, auto more) {
     const int stage = s % RING_STAGES, nstage = (s + RING_STAGES - 1) % RING_STAGES, nk0 = (s + RING_STAGES - 1) * RBK;
     read_operands(stage, 1);
@@ -510,16 +511,19 @@ __global__ __launch_bounds__(512, 1) void gemm_ring_kernel(const bf16* __restric
 
   // accumulator layout of a 32x32 tile: lane holds column lane%32, rows 8*(r/4) + 4*(lane/32) + r%4
   if (EPI == EPI_SILU_MUL) {
-    const int gn = bx * (RBN / 2) + wn * 32 + lane % 32;
-    if (gn >= half) return;
 #pragma unroll
-    for (int i = 0; i < RTM; ++i)
+    for (int p = 0; p < RTN / 2; ++p) {
+      const int gn = bx * (RBN / 2) + wn * (RTN / 2 * 32) + p * 32 + lane % 32;
+      if (gn >= half) continue;
 #pragma unroll
-      for (int r = 0; r < 16; ++r) {
-        const int gm = m0 + wm * RTM * 32 + i * 32 + 8 * (r / 4) + 4 * (lane / 32) + r % 4;
-        const float g = acc[i][0][r], u = acc[i][1][r];
-        if (gm < M) c[(size_t)gm * ldc + gn] = (CT)(g / (1.0f + __expf(-g)) * u);
-      }
+      for (int i = 0; i < RTM; ++i)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+          const int gm = m0 + wm * RTM * 32 + i * 32 + 8 * (r / 4) + 4 * (lane / 32) + r % 4;
+          const float g = acc[i][2 * p][r], u = acc[i][2 * p + 1][r];
+          if (gm < M) c[(size_t)gm * ldc + gn] = (CT)(g / (1.0f + __expf(-g)) * u);
+        }
+    }
     return;
   }
   if constexpr (EPI == EPI_ACCUMULATE) {
@@ -571,7 +575,7 @@ inline bool ring_pays(int epi, const void* a, int lda, const void* w, int ldw, i
 template <int EPI, typename CT>
 int launch_ring(const bf16* a, int lda, const bf16* w, int ldw, CT* c, int ldc, int M, int N, int K, hipStream_t stream) {
   const int cols = EPI == EPI_SILU_MUL ? N / 2 : N, bn = EPI == EPI_SILU_MUL ? RBN / 2 : RBN;
-  const dim3 grid((cols + bn - 1) / bn, (M + RBM - 1) / RBM), block(512);
+  const dim3 grid((cols + bn - 1) / bn, (M + RBM - 1) / RBM), block(RGM * RGN * 64);
   GB_REQUIRE(grid.y <= 65535, "gemm_bf16: M=%d needs more than 65535 row tiles", M);
   hipLaunchKernelGGL((gemm_ring_kernel<EPI, CT>), grid, block, 0, stream, a, lda, w, ldw, c, ldc, M, N, K, 0);
   return launched("gemm_bf16 (ring)");
@@ -972,7 +976,7 @@ int launch_split(const bf16* a, int lda, const bf16* w, int ldw, CT* c, int ldc,
     if (int rc = launch_stream<EPI_STORE, float>(a, lda, w, ldw, ws, N, M, N, K, plan.k_slice, plan.slices, stream)) return rc;
   }
   if (ring)
-    hipLaunchKernelGGL((gemm_ring_kernel<EPI_STORE, float>), dim3((N + RBN - 1) / RBN, (M + RBM - 1) / RBM, plan.slices), dim3(512),
+    hipLaunchKernelGGL((gemm_ring_kernel<EPI_STORE, float>), dim3((N + RBN - 1) / RBN, (M + RBM - 1) / RBM, plan.slices), dim3(RGM * RGN * 64),
                        0, stream, a, lda, w, ldw, ws, N, M, N, K, plan.k_slice);
 #define GB_S(WM, FULL)                                                                                                   \
   if (!ring && !streams && (plan.bm == 64 * WM) && kfull == FULL)                                                                   \

@@ -105,6 +105,9 @@ class Scheduler:
         self.itl: List[float] = []
         self._arrival: Dict[int, float] = {}
         self._last_token: Dict[int, float] = {}
+        # what every step hands to the host library, made once: events come back through these
+        self._event_cap = 4096
+        self._event_bufs = ((C.c_int64 * self._event_cap)(), (C.c_int32 * self._event_cap)(), (C.c_int32 * self._event_cap)())
 
     def __del__(self):
         h, self._h = getattr(self, "_h", None), None
@@ -168,7 +171,8 @@ class Scheduler:
             entries.append((ids[i], flat[at:at + counts[i]], [counts[i] - 1] if wants[i] else []))
             batch_desc.append((ids[i], "decode" if decodes[i] else "prefill", counts[i]))
             at += counts[i]
-        logits = self.engine.run_reserved(entries)
+        # prompt ids were checked when the request was submitted and sampled ids lie below the vocabulary by construction
+        logits = self.engine.run_reserved(entries, validated=True)
         rows = logits.shape[0]
         # sampling parameters of every wanted row: temperature, top_p, min_p, penalty, uniform | top_k, skip
         fl, it = np.empty((5, max(1, rows)), np.float32), np.empty((2, max(1, rows)), np.int32)
@@ -204,8 +208,8 @@ class Scheduler:
 
     def _drain_events(self) -> List[int]:
         finished = []
-        cap = 4096
-        ids, kinds, vals = (C.c_int64 * cap)(), (C.c_int32 * cap)(), (C.c_int32 * cap)()
+        cap = self._event_cap
+        ids, kinds, vals = self._event_bufs
         now = time.perf_counter()
         while True:
             n = self._lib.gbh_sched_take_events(self._h, ids, kinds, vals, cap)

@@ -33,7 +33,7 @@ class ToyEngine:
     def reset_state(self, sid):
         pass
 
-    def run_reserved(self, entries):
+    def run_reserved(self, entries, validated=False):
         rows = []
         for sid, toks, want in entries:
             start = self.cache.seq_len(sid)
