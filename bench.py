@@ -222,7 +222,8 @@ def main() -> int:
         "metric": f"decode tok/s at batch {a.batch}, {NAMES[a.shapes]}, context {a.context} "
                   "(prefill tok/s at 2,048 tokens beside it)",
         "value": round(value, 1), "unit": "tok/s", "n_gpus": 1, "steps": a.steps, "warmup": a.warmup,
-        "ms_per_step": round(step_s * 1e3, 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "ms_per_step": round(step_s * 1e3, 4), "ms_per_step_sd": round(statistics.stdev(ms), 4) if len(ms) > 1 else 0.0,
+        "repetitions": a.reps, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "bf16" if a.dtype == "bfloat16" else "fp32", "data": "synthetic token ids, random N(0, 0.02) weights",
         "config": {"model": NAMES[a.shapes], "layers": cfg.num_hidden_layers, "layers_of_model": MODEL["num_hidden_layers"],
                    "hidden": d, "heads": cfg.num_attention_heads, "kv_heads": cfg.num_key_value_heads,

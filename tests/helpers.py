@@ -44,13 +44,25 @@ class ModelDirs:
         self.base = base
         self._made: Dict[Tuple, str] = {}
 
-    def get(self, name: str, seed: int = 0, norm_init: str = "uniform", dtype=torch.float32) -> str:
+    def get(self, name: str, seed: int = 0, norm_init: str = "uniform", dtype=torch.float32, sharp: float = 1.0) -> str:
+        """``sharp`` > 1: query and key projections are scaled by it, so that scores spread out and single keys stand
+        out among their neighbours: with weights of 0.02 every softmax is nearly flat, and a key read from a wrong
+        page or slot would change an output by a hundredth of what it changes here."""
         from glassbox_amd.config import config_from_dict
-        from glassbox_amd.weights import write_random_model
-        key = (name, seed, norm_init, str(dtype))
+        from glassbox_amd.weights import SafetensorsFile, save_file, write_random_model
+        key = (name, seed, norm_init, str(dtype), sharp)
         if key not in self._made:
             folder = os.path.join(self.base, "_".join(str(k).replace(".", "_") for k in key))
             write_random_model(config_from_dict(TINY[name]), folder, seed, norm_init=norm_init, dtype=dtype)
+            if sharp != 1.0:
+                path = os.path.join(folder, "model.safetensors")
+                f = SafetensorsFile(path)
+                tensors = {n: f.tensor(n).clone() for n in f.names()}
+                f.close()
+                for n in tensors:
+                    if n.endswith(("q_proj.weight", "k_proj.weight")):
+                        tensors[n] = (tensors[n].float() * sharp).to(tensors[n].dtype)
+                save_file(tensors, path)
             self._made[key] = folder
         return self._made[key]
 
@@ -103,25 +115,26 @@ class Bf16Bound:
     def __init__(self):
         self._made: Dict[Tuple, float] = {}
 
-    def get(self, folder: str, requests: Dict[str, List[int]], page_size: int = 16) -> float:
+    def get(self, folder: str, requests: Dict[str, List[int]], page_size: int = 16,
+            plain_rel: float = TOL_BF16_PLAIN_REL) -> float:
         from glassbox_amd.engine import Engine
         key = (folder, page_size, tuple(sorted((r, tuple(t)) for r, t in requests.items())))
         if key not in self._made:
             eng = Engine(folder, dtype="bfloat16", max_tokens=sum(len(t) + 64 for t in requests.values()), max_seqs=2,
                          kernels="plain", page_size=page_size)
-            self._made[key] = self.measure(eng, requests, lambda r: oracle(folder, requests[r], "bfloat16"))
+            self._made[key] = self.measure(eng, requests, lambda r: oracle(folder, requests[r], "bfloat16"), plain_rel)
         return self._made[key]
 
     @staticmethod
-    def measure(plain_engine, requests: Dict[str, List[int]], want_of) -> float:
+    def measure(plain_engine, requests: Dict[str, List[int]], want_of, plain_rel: float = TOL_BF16_PLAIN_REL) -> float:
         """Twice the largest error of ``plain_engine`` (bfloat16, plain kernels) over the requests run whole;
-        ``want_of(request)`` gives the plain implementation's logits."""
+        ``want_of(request)`` gives the plain implementation's logits.  ``plain_rel`` bounds that engine's own error."""
         got = replay(plain_engine, schedule_whole(requests))
         worst = 0.0
         for r in requests:
             want = want_of(r)
             err = float(np.abs(got[r] - want).max())
-            limit = TOL_BF16_PLAIN_REL * max(1.0, float(np.abs(want).max()))
+            limit = plain_rel * max(1.0, float(np.abs(want).max()))
             assert err <= limit, f"plain kernels in bfloat16, request {r}: {err:.3e} from the plain implementation (limit {limit:.3e})"
             worst = max(worst, err)
         return 2.0 * worst

@@ -174,6 +174,43 @@ def test_shared_prefixes_recomputation_and_forks(model_dirs, bf16_bound, name, d
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("name", ["B", "D"])
+def test_sharp_attention_shows_a_wrong_key(model_dirs, bf16_bound, name, dtype):
+    """With small random weights every softmax is nearly flat and one wrong key among a hundred changes little.  Here
+    the query and key projections are scaled so that scores spread over several units and a few keys carry a row's
+    attention: mixed steps over an exact-fit pool, and a request cut at every page's edge, must still give the plain
+    implementation's logits.  (The test checks first that attention is sharp: the largest probability of a late token
+    is many times the uniform one.)"""
+    import math
+    import torch
+    from plain import llama as plain_llama
+    from glassbox_amd.engine import Engine
+    folder = model_dirs.get(name, sharp=8.0)
+    cfg, w = plain_llama.load_folder(folder)
+    requests = make_requests_det(name, more=True)
+    # how sharp: the first layer's attention of the longest request's last token
+    toks = max(requests.values(), key=len)
+    x = w["model.embed_tokens.weight"].double()[torch.tensor(toks)]
+    h = plain_llama.rms_norm(x, w["model.layers.0.input_layernorm.weight"].double(), cfg["rms_norm_eps"])
+    nh, nkv, hd = cfg["num_attention_heads"], cfg["num_key_value_heads"], cfg["head_dim"]
+    q = plain_llama.rope((h @ w["model.layers.0.self_attn.q_proj.weight"].double().T).reshape(len(toks), nh, hd), range(len(toks)), cfg["rope_theta"])
+    k = plain_llama.rope((h @ w["model.layers.0.self_attn.k_proj.weight"].double().T).reshape(len(toks), nkv, hd), range(len(toks)), cfg["rope_theta"])
+    prob = torch.softmax((k[:, 0, :] @ q[-1, 0, :]) / math.sqrt(hd), 0)
+    assert prob.max().item() > 10.0 / len(toks), f"attention is not sharp: largest probability {prob.max().item():.3f} over {len(toks)} keys"
+    # scores of several units carry bfloat16's rounding of queries and keys into the probabilities: the plain kernels'
+    # own error is 2 to 4e-2 here (measured), four times that of the flat model; a wrong key would cost tenths
+    tol = helpers.TOL_F32 if dtype == "float32" else bf16_bound.get(folder, requests, plain_rel=8e-2)
+    steps, peak = helpers.schedule_mixed(requests, seed=7)
+    eng = Engine(folder, dtype=dtype, max_tokens=peak, max_seqs=4)
+    got = helpers.replay(eng, steps)
+    check(folder, requests, got, dtype, f"sharp attention, mixed (pool {peak})", tol)
+    got = helpers.replay(eng, helpers.schedule_chunks(make_requests_det(name), sizes=(16, 15, 17, 1, 32, 31, 2)))
+    check(folder, make_requests_det(name), got, dtype, "sharp attention, portions that end at and beside page edges", tol)
+    eng.cache.check_invariants()
+    assert eng.cache.used_pages() == 0
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 @pytest.mark.parametrize("name,page_size", [("B", 32), ("D", 64), ("C", 48)])
 def test_other_page_sizes(model_dirs, bf16_bound, name, page_size, dtype):
     """Pages of 32 and 64 tokens through the whole engine (the tuned attention kernels take powers of two), and of
