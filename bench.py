@@ -56,6 +56,7 @@ def main() -> int:
                          "turn behind a long history, the tail of a prompt)")
     ap.add_argument("--portion-tokens", type=int, default=128)
     ap.add_argument("--no-graph", action="store_true", help="run decode steps without HIP graph replay")
+    ap.add_argument("--page-size", type=int, default=16, help="tokens a page of the cache (16 as in the reference)")
     ap.add_argument("--reps", type=int, default=3, help="times the K timed steps are repeated (mean and spread are reported)")
     ap.add_argument("--no-scheduler", action="store_true", help="skip the figure through Scheduler.step")
     ap.add_argument("--prefill-tokens", type=int, default=PREFILL_TOKENS,
@@ -81,7 +82,7 @@ def main() -> int:
     init_random(model, seed=0, dtype=a.dtype, device="cuda:0")
     batches = [a.batch] + ([] if a.no_points else [b for b in (1, 64) if b != a.batch])
     max_tokens = max(max(batches) * (a.context + 64), a.prefill_tokens + 64)
-    eng = Engine(model, dtype=a.dtype, max_tokens=max_tokens, max_seqs=max(batches), page_size=16,
+    eng = Engine(model, dtype=a.dtype, max_tokens=max_tokens, max_seqs=max(batches), page_size=a.page_size,
                  graph_decode=False if a.no_graph else None)
     vocab = cfg.vocab_size
     g = torch.Generator().manual_seed(1)
