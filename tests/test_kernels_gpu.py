@@ -754,6 +754,37 @@ def test_tuned_decode_finds_one_far_key_in_every_chunk_position():
             assert (out.cpu().float()[0] - want).abs().max().item() < 2e-2, f"key at {target} was not found"
 
 
+def test_tuned_decode_over_tens_of_thousands_of_keys():
+    """Contexts of 40,000 and 33,333 keys beside one of 5: some hundred and sixty chunks a request for the second
+    pass to merge, block tables of 2,500 pages.  Against the plain kernel on random keys, and with one key made to
+    stand out near the start, in the middle and at the end."""
+    from types import SimpleNamespace
+    from glassbox_amd import ops
+    nh, nkv, hd, page = 4, 2, 64, 16
+    ctx_lens = [40000, 33333, 5]
+    k_pages, v_pages, tables, ks, vs = paged_setup(ctx_lens, nkv, hd, page, seed=5, dtype=torch.bfloat16)
+    q = (rnd(3, nh * hd, seed=6) * 0.7).bfloat16()
+    ctx = BareContext([1, 1, 1], ctx_lens, tables, max_context=40960)
+    assert -(-40960 // ops.decode_chunk(3, nkv, 40960)) > 100
+    cache = SimpleNamespace(k_pages=to_dev(ops.pack_keys(k_pages)), v_pages=to_dev(v_pages), group=0)
+    out, twin = (torch.zeros(3, nh * hd, device=DEV, dtype=torch.bfloat16) for _ in range(2))
+    ops.attention_decode(to_dev(q), out, ctx, cache, nh, 1 / math.sqrt(hd), 0)
+    ops.attention_plain(to_dev(q), twin, ctx.positions, torch.tensor([0, 1, 2], dtype=torch.int32, device=DEV), ctx.tables[0],
+                        cache.k_pages, cache.v_pages, nh, 1 / math.sqrt(hd), 0)
+    assert ((out.float() - twin.float()).abs() <= 2 ** -7 * (1 + twin.float().abs())).all()
+    qq = q.float().reshape(3, nh, hd)
+    qq[:, 1::2] = qq[:, 0::2]
+    qq = qq.reshape(3, nh * hd).bfloat16()
+    for target in (3, 20479, 20480, 39999):
+        kp = k_pages.clone()
+        for kvh in range(nkv):
+            kp[tables[0, target // page], kvh, target % page, :] = (qq[0].float().reshape(nh, hd)[2 * kvh] * 40).bfloat16()
+        cache = SimpleNamespace(k_pages=to_dev(ops.pack_keys(kp)), v_pages=to_dev(v_pages), group=0)
+        ops.attention_decode(to_dev(qq), out, ctx, cache, nh, 1 / math.sqrt(hd), 0)
+        want = vs[0][target].float().repeat_interleave(2, 0).reshape(-1)
+        assert (out.cpu().float()[0] - want).abs().max().item() < 2e-2, f"key at {target} of 40,000 was not found"
+
+
 @pytest.mark.parametrize("nh,nkv,hd,window", [(8, 2, 64, 0), (4, 4, 128, 0), (6, 3, 32, 700), (8, 8, 96, 0)])
 def test_tuned_prefill_short_portions_over_long_contexts(nh, nkv, hd, window):
     """Few pairs of blocks and long contexts: several workgroups share a pair's keys and a second pass adds their
