@@ -56,6 +56,8 @@ def main() -> int:
                          "turn behind a long history, the tail of a prompt)")
     ap.add_argument("--portion-tokens", type=int, default=128)
     ap.add_argument("--no-graph", action="store_true", help="run decode steps without HIP graph replay")
+    ap.add_argument("--no-layer-tapes", action="store_true",
+                    help="walk every layer through the parts' Python (by default layers of a kind share one walk a step)")
     ap.add_argument("--page-size", type=int, default=16, help="tokens a page of the cache (16 as in the reference)")
     ap.add_argument("--reps", type=int, default=3, help="times the K timed steps are repeated (mean and spread are reported)")
     ap.add_argument("--no-scheduler", action="store_true", help="skip the figure through Scheduler.step")
@@ -83,7 +85,7 @@ def main() -> int:
     batches = [a.batch] + ([] if a.no_points else [b for b in (1, 64) if b != a.batch])
     max_tokens = max(max(batches) * (a.context + 64), a.prefill_tokens + 64)
     eng = Engine(model, dtype=a.dtype, max_tokens=max_tokens, max_seqs=max(batches), page_size=a.page_size,
-                 graph_decode=False if a.no_graph else None)
+                 graph_decode=False if a.no_graph else None, layer_tapes=not a.no_layer_tapes)
     vocab = cfg.vocab_size
     g = torch.Generator().manual_seed(1)
 
@@ -106,7 +108,7 @@ def main() -> int:
     if a.only == "portion":
         # a step of a few hundred rows: the history is cached in portions of 2,048, then the timed step brings the rest
         hist = a.context - a.portion_tokens
-        times = []
+        times, host = [], []
         for rep in range(4):
             toks = torch.randint(0, vocab, (a.context,), generator=g).tolist()
             for at in range(0, hist, PREFILL_TOKENS):
@@ -114,11 +116,12 @@ def main() -> int:
             torch.cuda.synchronize()
             t0 = time.perf_counter()
             eng.step([("p", toks[hist:], [a.portion_tokens - 1])])
+            host.append(time.perf_counter() - t0)              # the launches are made: what the step costs the host
             torch.cuda.synchronize()
             times.append(time.perf_counter() - t0)
             eng.end_request("p")
         print(json.dumps({"portion_ms": round(min(times[1:]) * 1e3, 3), "tokens": a.portion_tokens, "context": a.context,
-                          "all_ms": [round(t * 1e3, 3) for t in times]}))
+                          "host_ms": round(min(host[1:]) * 1e3, 3), "all_ms": [round(t * 1e3, 3) for t in times]}))
         return 0
     if a.only == "decode":
         pf = float("nan")

@@ -38,7 +38,7 @@ HOST_FLAGS = ["-O2", "-std=c++17", "-fPIC", "-shared", "-Wall"]
 
 #: name -> (compiler kind, sources relative to csrc, extra dependencies hashed with them)
 LIBRARIES: Dict[str, tuple] = {
-    "host": ("host", ["host/cache_manager.cpp", "host/scheduler.cpp", "host/c_api.cpp"],
+    "host": ("host", ["host/cache_manager.cpp", "host/scheduler.cpp", "host/c_api.cpp", "host/launch_tape.cpp"],
              ["host/cache_manager.h", "host/scheduler.h", "host/sampler.h"]),
     "elementwise": ("hip", ["hip/elementwise.hip"], ["hip/common.h"]),
     "gemm_f32": ("hip", ["hip/gemm_f32.hip"], ["hip/common.h"]),

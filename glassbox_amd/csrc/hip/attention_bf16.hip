@@ -910,3 +910,7 @@ extern "C" int gb_attention_prefill_bf16(const void* q, int q_stride, void* out,
   }
   return 0;
 }
+
+// the launches of a layer can be recorded and made again for the layers like it (common.h)
+GB_TAPED(gb_attention_decode_bf16)
+GB_TAPED(gb_attention_prefill_bf16)

@@ -102,3 +102,6 @@ extern "C" int gb_attention_plain(const void* q, int q_stride, void* out, int ou
     return fail("attention_plain: unknown dtype %d", dtype);
   return launched("attention_plain");
 }
+
+// the launches of a layer can be recorded and made again for the layers like it (common.h)
+GB_TAPED(gb_attention_plain)

@@ -10,7 +10,10 @@
 #include <cstdarg>
 #include <cstdint>
 #include <cstdio>
+#include <cstring>
 #include <string>
+#include <type_traits>
+#include <utility>
 
 namespace gb {
 
@@ -112,6 +115,35 @@ inline int launched(const char* what) {
   do {                        \
     if (!(cond)) return gb::fail(__VA_ARGS__); \
   } while (0)
+
+// A launch can be recorded as its entry point and its arguments and made again later, with other operands in
+// the places of some pointers, without a walk through the bindings.  Recorded arguments lie in 64-bit slots:
+// integers sign-extended, the bits of a float in the low half, pointers as they are.  GB_TAPED(entry) gives an
+// entry point `<entry>_taped(slots)` that unpacks the slots by the entry point's own parameter types and calls it.
+namespace gb {
+template <class T> inline T from_slot(unsigned long long v) {
+  if constexpr (std::is_pointer_v<T>) {
+    return reinterpret_cast<T>(static_cast<uintptr_t>(v));
+  } else if constexpr (std::is_floating_point_v<T>) {
+    const uint32_t bits = static_cast<uint32_t>(v);
+    float f;
+    std::memcpy(&f, &bits, sizeof f);
+    return static_cast<T>(f);
+  } else {
+    return static_cast<T>(static_cast<long long>(v));
+  }
+}
+template <class... A, std::size_t... I>
+inline int call_slots(int (*f)(A...), const unsigned long long* slots, std::index_sequence<I...>) {
+  return f(from_slot<A>(slots[I])...);
+}
+template <class... A> inline int call_slots(int (*f)(A...), const unsigned long long* slots) {
+  return call_slots(f, slots, std::index_sequence_for<A...>{});
+}
+}  // namespace gb
+
+#define GB_TAPED(entry) \
+  extern "C" int entry##_taped(const unsigned long long* slots) { return gb::call_slots(&entry, slots); }
 
 #define GB_DEFINE_LAST_ERROR \
   extern "C" const char* gb_last_error() { return gb::last_error().c_str(); }

@@ -534,3 +534,11 @@ extern "C" int gb_copy_rows(void* base, long long row_bytes, const int32_t* src,
   hipLaunchKernelGGL(copy_rows_kernel, dim3(count), dim3(256), 0, stream, (uint32_t*)base, (size_t)(row_bytes / 4), src, dst);
   return launched("copy_rows");
 }
+
+// the launches of a layer can be recorded and made again for the layers like it (common.h)
+GB_TAPED(gb_embed)
+GB_TAPED(gb_rmsnorm)
+GB_TAPED(gb_rope_table)
+GB_TAPED(gb_rope_store)
+GB_TAPED(gb_silu_mul)
+GB_TAPED(gb_copy_rows)

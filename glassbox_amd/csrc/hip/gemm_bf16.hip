@@ -1596,3 +1596,7 @@ extern "C" int gb_gemm_bf16_rope(const void* a, int lda, const void* w, int ldw,
   return launch_skinny<EPI_ROPE, false, bf16>(a, lda, (const bf16*)w, ldw, (bf16*)c, ldc, M, N, K, nullptr, 0, eps, extra,
                                               stream, rope);
 }
+
+// the launches of a layer can be recorded and made again for the layers like it (common.h)
+GB_TAPED(gb_gemm_bf16)
+GB_TAPED(gb_gemm_bf16_rope)

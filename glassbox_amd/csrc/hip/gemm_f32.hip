@@ -77,3 +77,6 @@ extern "C" int gb_gemm_f32(const float* a, int lda, const float* w, int ldw, flo
   hipLaunchKernelGGL(gemm_f32_kernel, grid, dim3(256), 0, stream, a, lda, w, ldw, c, ldc, M, N, K, accumulate);
   return launched("gemm_f32");
 }
+
+// the launches of a layer can be recorded and made again for the layers like it (common.h)
+GB_TAPED(gb_gemm_f32)

@@ -57,7 +57,8 @@ class Workspace:
 class StepContext:
     def __init__(self, *, device, dtype, page_size: int, workspace: Workspace, n: int, num_seqs: int,
                  token_ids, positions, tok_seq, slots: List[torch.Tensor], tables: List[torch.Tensor],
-                 q_start, q_len, pos0, state_slots, want, host: dict, kernels: str = "auto"):
+                 q_start, q_len, pos0, state_slots, want, host: dict, kernels: str = "auto",
+                 layer_tapes: bool = True):
         self.device, self.dtype, self.page_size, self.workspace = device, dtype, page_size, workspace
         self.n, self.num_seqs = n, num_seqs
         self.token_ids, self.positions, self.tok_seq = token_ids, positions, tok_seq
@@ -73,6 +74,8 @@ class StepContext:
         self.tuned = kernels != "plain"
         #: whether norms may be computed inside the matrix products around them
         self.fuse_norms = self.tuned
+        #: whether layers of a kind share one walk through the parts (``parts.tape``)
+        self.layer_tapes = layer_tapes
         self.memo: dict = {}
 
     def buffer(self, name: str, shape, dtype) -> torch.Tensor:

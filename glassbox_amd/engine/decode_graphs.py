@@ -96,7 +96,7 @@ class _Shape:
         self.ctx = StepContext(device=engine.device, dtype=engine.dtype, page_size=P, workspace=workspace, n=rows,
                                num_seqs=rows, token_ids=d[0], positions=d[1], tok_seq=d[2], slots=d_slots,
                                tables=d_tables, q_start=d[3], q_len=d[4], pos0=d[1], state_slots=d[5], want=d[6],
-                               host=host, kernels=engine.kernels)
+                               host=host, kernels=engine.kernels, layer_tapes=engine.layer_tapes)
         self.copied = torch.cuda.Event()
         self.runs = 0
         self.graph = None

@@ -52,11 +52,13 @@ class Engine:
     default where the arithmetic is bfloat16 and every part of the model allows it.
     kernels: "auto", or "plain": every part takes its plain kernels, one per operation and nothing fused, which
     is what the tuned kernels are compared with.
+    layer_tapes: layers of the same parts and sizes share one walk through the parts' Python a step: the first is
+    walked and its launches recorded, the others made again from native code (parts.tape); False walks every layer.
     """
 
     def __init__(self, model, dtype="bfloat16", max_tokens: int = 4096, max_seqs: int = 32, page_size: int = 16,
                  prefix_caching: bool = False, device: str = "cuda:0", kernels: str = "auto",
-                 graph_decode: Optional[bool] = None):
+                 graph_decode: Optional[bool] = None, layer_tapes: bool = True):
         ops.require_gpu()
         self.dtype = compute_dtype(dtype)
         self.device = torch.device(device)
@@ -74,6 +76,7 @@ class Engine:
         if kernels not in ("auto", "plain"):
             raise EngineError(f"kernels={kernels!r}: 'auto' (tuned and fused kernels where they apply) or 'plain'")
         self.kernels = kernels
+        self.layer_tapes = bool(layer_tapes)
         num_pages = max(1, -(-int(max_tokens) // self.page_size))
 
         # page groups: cache layers whose mixers keep the same span of positions share page numbers
@@ -303,4 +306,4 @@ class Engine:
                            num_seqs=S, token_ids=cut(0, n), positions=cut(n, n), tok_seq=cut(2 * n, n), slots=slots,
                            tables=tables, q_start=cut(3 * n, S), q_len=cut(3 * n + S, S), pos0=cut(3 * n + 2 * S, S),
                            state_slots=cut(3 * n + 3 * S, S), want=cut(3 * n + 4 * S, W), host=host,
-                           kernels=self.kernels)
+                           kernels=self.kernels, layer_tapes=self.layer_tapes)

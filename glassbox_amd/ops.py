@@ -10,7 +10,8 @@ from __future__ import annotations
 
 import ctypes as C
 import functools
-from typing import Optional
+import struct
+from typing import List, Optional, Sequence
 
 import torch
 
@@ -101,9 +102,136 @@ def _lib(name: str):
     return lib
 
 
-def _check(lib, rc: int) -> None:
-    if rc != 0:
+def _launch(lib, entry, *args) -> None:
+    """Calls a kernel's entry point; every launch of a step goes through here, which is where a layer's
+    launches are recorded (``start_tape``)."""
+    if entry(*args) != 0:
         raise KernelError(lib.gb_last_error().decode())
+    if _tape is not None:
+        _tape.add(lib, entry, args)
+
+
+# ------------------------------------------------------------------ recorded launches
+# The layers of a model mostly differ in nothing but their tensors.  A step walks the first of a kind through the
+# parts' Python while the launches it makes are recorded, and makes the same launches again for every later layer
+# of that kind from native code, with the recorded layer's tensors replaced by the later layer's
+# (csrc/host/launch_tape.cpp).  ``parts.model.DecoderModel.forward`` decides which layers are of a kind.
+TAPE_COUNTS = {"recorded_layers": 0, "replayed_layers": 0, "replayed_launches": 0}
+_tape: Optional["LaunchTape"] = None
+_tape_entries: dict = {}
+_host = None
+
+
+def _host_lib():
+    global _host
+    if _host is None:
+        lib = build.load("host")
+        lib.gbh_tape_run.argtypes = [_vp, _i, _vp, _vp, _vp, _i]
+        lib.gbh_tape_run.restype = _i
+        if lib.gbh_tape_entry_bytes() != 24 + 8 * lib.gbh_tape_max_args():
+            raise KernelError("the host library's recorded launches are not laid out as the bindings pack them")
+        _host = lib
+    return _host
+
+
+def _tape_entry(lib, entry):
+    """How to pack a launch of ``entry``: (struct, address of its taped form, pointer mask), or False if the
+    library has no taped form of it."""
+    held = _tape_entries.get(id(entry))   # ctypes functions do not hash; the entry is held so that its id stays its own
+    hit = held[1] if held is not None and held[0] is entry else None
+    if hit is None:
+        max_args = _host_lib().gbh_tape_max_args()
+        try:
+            taped = getattr(lib, entry.__name__ + "_taped")
+        except AttributeError:
+            taped = None
+        if taped is None or len(entry.argtypes) > max_args:
+            hit = False
+        else:
+            codes, mask = "", 0
+            for i, t in enumerate(entry.argtypes):
+                if t is _vp:
+                    codes += "Q"
+                    mask |= 1 << i
+                elif t is _f:
+                    codes += "f4x"      # the float's bits in the low half of the slot
+                else:
+                    codes += "q"
+            pad = 8 * (max_args - len(entry.argtypes))
+            hit = (struct.Struct("<QQII" + codes + (f"{pad}x" if pad else "")), C.cast(taped, _vp).value, mask,
+                   len(entry.argtypes))
+        _tape_entries[id(entry)] = (entry, hit)
+    return hit
+
+
+class LaunchTape:
+    """The launches made between ``start_tape()`` and ``stop_tape()``, packed as the native runner reads them."""
+
+    def __init__(self):
+        self.data = bytearray()
+        self.libs: list = []          # the library of each launch: it holds the message if a replay refuses
+        self.usable = True            # False once a launch was made that cannot be made again natively
+        self._c = None
+
+    def __len__(self):
+        return len(self.libs)
+
+    def add(self, lib, entry, args) -> None:
+        how = _tape_entry(lib, entry)
+        if how is False:
+            self.usable = False
+            return
+        st, address, mask, n = how
+        self.data += st.pack(address, mask, n, 0, *[0 if a is None else a for a in args])
+        self.libs.append(lib)
+
+    def pointer(self):
+        if self._c is None:
+            self._c = (C.c_char * max(1, len(self.data))).from_buffer(self.data)
+        return C.addressof(self._c)
+
+
+class TapeOperands:
+    """The tensors of a layer, in a fixed order, as the address ranges the native runner maps between layers."""
+
+    def __init__(self, tensors: Sequence[torch.Tensor]):
+        n = len(tensors)
+        ptrs, sizes = [], []
+        for t in tensors:
+            span = 1 + sum((s - 1) * st for s, st in zip(t.shape, t.stride())) if t.numel() else 0
+            ptrs.append(t.data_ptr())
+            sizes.append(span * t.element_size())
+        self.sizes = tuple(sizes)
+        self.ptrs = (C.c_uint64 * max(1, n))(*ptrs)
+        self.bytes = (C.c_uint64 * max(1, n))(*sizes)
+        self.count = n
+        self.keep = list(tensors)
+
+
+def start_tape() -> LaunchTape:
+    global _tape
+    if _tape is not None:
+        raise KernelError("launches are being recorded already")
+    _host_lib()
+    _tape = LaunchTape()
+    return _tape
+
+
+def stop_tape() -> None:
+    global _tape
+    _tape = None
+
+
+def run_tape(tape: LaunchTape, recorded: TapeOperands, target: TapeOperands) -> None:
+    """Makes the recorded launches again with the tensors of ``recorded`` replaced, one for one, by those of ``target``."""
+    if not tape.usable or recorded.sizes != target.sizes:
+        raise KernelError("run_tape: the layer's tensors do not match those of the recorded layer")
+    rc = _host_lib().gbh_tape_run(tape.pointer(), len(tape), C.addressof(recorded.ptrs), C.addressof(recorded.bytes),
+                                  C.addressof(target.ptrs), recorded.count)
+    if rc != 0:
+        raise KernelError(tape.libs[rc - 1].gb_last_error().decode())
+    TAPE_COUNTS["replayed_layers"] += 1
+    TAPE_COUNTS["replayed_launches"] += len(tape)
 
 
 _raw_stream = getattr(torch._C, "_cuda_getCurrentRawStream", None)
@@ -196,7 +324,7 @@ def embed(table: torch.Tensor, ids: torch.Tensor, out: torch.Tensor) -> None:
     if out.dtype != torch.float32 or not out.is_contiguous() or not table.is_contiguous() or table.shape[1] != d:
         raise KernelError("embed: out must be contiguous float32 [n, d] and table [vocab, d]")
     lib = _lib("elementwise")
-    _check(lib, lib.gb_embed(_p(table), dtype_code(table), _p(ids), _p(out), n, d, table.shape[0], _stream()))
+    _launch(lib, lib.gb_embed, _p(table), dtype_code(table), _p(ids), _p(out), n, d, table.shape[0], _stream())
 
 
 def rmsnorm(x: torch.Tensor, gamma: torch.Tensor, eps: float, out: torch.Tensor,
@@ -212,8 +340,8 @@ def rmsnorm(x: torch.Tensor, gamma: torch.Tensor, eps: float, out: torch.Tensor,
         raise KernelError("rmsnorm: fewer input rows than output rows")
     _i32(rows, "rows", m)
     lib = _lib("elementwise")
-    _check(lib, lib.gb_rmsnorm(_p(x), _p(gamma), dtype_code(gamma), _p(rows), _p(out), dtype_code(out), m, d,
-                               float(eps), _stream()))
+    _launch(lib, lib.gb_rmsnorm, _p(x), _p(gamma), dtype_code(gamma), _p(rows), _p(out), dtype_code(out), m, d,
+                               float(eps), _stream())
 
 
 def rope_table(positions: torch.Tensor, inv_freq: torch.Tensor, cos: torch.Tensor, sin: torch.Tensor) -> None:
@@ -226,7 +354,7 @@ def rope_table(positions: torch.Tensor, inv_freq: torch.Tensor, cos: torch.Tenso
     if inv_freq.numel() != half or sin.shape != cos.shape:
         raise KernelError("rope_table: table shapes do not match")
     lib = _lib("elementwise")
-    _check(lib, lib.gb_rope_table(_p(positions), _p(inv_freq), _p(cos), _p(sin), n, half, _stream()))
+    _launch(lib, lib.gb_rope_table, _p(positions), _p(inv_freq), _p(cos), _p(sin), n, half, _stream())
 
 
 def rope_store(qkv: torch.Tensor, cos: Optional[torch.Tensor], sin: Optional[torch.Tensor],
@@ -263,10 +391,10 @@ def rope_store(qkv: torch.Tensor, cos: Optional[torch.Tensor], sin: Optional[tor
         if not 0 <= v_rows <= n:
             raise KernelError("rope_store: the first portion row lies outside the batch")
     lib = _lib("elementwise")
-    _check(lib, lib.gb_rope_store(_p(qkv), dtype_code(qkv), stride, _p(cos), _p(sin), _p(slots), _p(k_pages),
+    _launch(lib, lib.gb_rope_store, _p(qkv), dtype_code(qkv), stride, _p(cos), _p(sin), _p(slots), _p(k_pages),
                                   _p(v_pages), n, n_heads, n_kv_heads, head_dim, page_size, 1 if rotate else 0,
                                   int(v_rows), _p(q_start), _p(q_len), _p(pos0), int(seq_base), int(n_seqs),
-                                  int(max_q_len), _stream()))
+                                  int(max_q_len), _stream())
 
 
 def silu_mul(gate_up: torch.Tensor, out: torch.Tensor) -> None:
@@ -276,7 +404,7 @@ def silu_mul(gate_up: torch.Tensor, out: torch.Tensor) -> None:
             or gate_up.dtype != out.dtype:
         raise KernelError("silu_mul: gate_up must be contiguous [n, 2I] and out [n, I] of one type")
     lib = _lib("elementwise")
-    _check(lib, lib.gb_silu_mul(_p(gate_up), _p(out), dtype_code(out), n, inter, _stream()))
+    _launch(lib, lib.gb_silu_mul, _p(gate_up), _p(out), dtype_code(out), n, inter, _stream())
 
 
 def copy_rows(base: torch.Tensor, src: torch.Tensor, dst: torch.Tensor) -> None:
@@ -289,7 +417,7 @@ def copy_rows(base: torch.Tensor, src: torch.Tensor, dst: torch.Tensor) -> None:
     _i32(dst, "dst", count)
     row_bytes = base[0].numel() * base.element_size()
     lib = _lib("elementwise")
-    _check(lib, lib.gb_copy_rows(_p(base), row_bytes, _p(src), _p(dst), count, _stream()))
+    _launch(lib, lib.gb_copy_rows, _p(base), row_bytes, _p(src), _p(dst), count, _stream())
 
 
 # ------------------------------------------------------------------------ products
@@ -356,14 +484,14 @@ def gemm(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor, accumulate: bool =
         if emit is not None or rms_parts is not None:
             raise KernelError("gemm: one way of fusing the norm at a time")
         lib = _lib("gemm_bf16")
-        _check(lib, lib.gb_gemm_bf16(_p(a), lda, _p(w), ldw, _p(out), ldc, BF16, M, N, K, 2 if silu_mul else 0,
+        _launch(lib, lib.gb_gemm_bf16, _p(a), lda, _p(w), ldw, _p(out), ldc, BF16, M, N, K, 2 if silu_mul else 0,
                                      _p(gamma), dtype_code(gamma), float(eps), None, 0, None, 0, None, None, 0,
-                                     None, 0, _stream()))
+                                     None, 0, _stream())
     elif a.dtype == torch.float32 and w.dtype == torch.float32:
         if out.dtype != torch.float32:
             raise KernelError("gemm: 32-bit operands need a 32-bit result")
         lib = _lib("gemm_f32")
-        _check(lib, lib.gb_gemm_f32(_p(a), lda, _p(w), ldw, _p(out), ldc, M, N, K, 1 if accumulate else 0, _stream()))
+        _launch(lib, lib.gb_gemm_f32, _p(a), lda, _p(w), ldw, _p(out), ldc, M, N, K, 1 if accumulate else 0, _stream())
     elif a.dtype == torch.bfloat16 and w.dtype == torch.bfloat16:
         if accumulate and out.dtype != torch.float32:
             raise KernelError("gemm: accumulation is into a 32-bit result")
@@ -399,11 +527,11 @@ def gemm(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor, accumulate: bool =
             if (M > 8 or accumulate or parts.dtype != torch.float32 or not parts.is_contiguous()
                     or parts.numel() < n_parts * 8 or n_parts <= 0):
                 raise KernelError("gemm: partial sums of a norm go with at most 8 rows and a storing product")
-        _check(lib, lib.gb_gemm_bf16(_p(a), lda, _p(w), ldw, _p(out), ldc, dtype_code(out), M, N, K,
+        _launch(lib, lib.gb_gemm_bf16, _p(a), lda, _p(w), ldw, _p(out), ldc, dtype_code(out), M, N, K,
                                      2 if silu_mul else (1 if accumulate else 0), None, 0, float(eps),
                                      _p(e_gamma), dtype_code(e_gamma) if e_gamma is not None else 0, _p(e_h), e_ldh,
                                      _p(e_ss), _p(parts), int(n_parts), _p(workspace),
-                                     workspace.numel() if workspace is not None else 0, _stream()))
+                                     workspace.numel() if workspace is not None else 0, _stream())
     else:
         raise KernelError(f"gemm: operand types {a.dtype} and {w.dtype} do not match a kernel")
 
@@ -448,10 +576,10 @@ def gemm_rope(a: torch.Tensor, w: torch.Tensor, qkv: torch.Tensor, n_heads: int,
         if rms is not None or M > 8 or parts.dtype != torch.float32 or not parts.is_contiguous() or parts.numel() < n_parts * 8:
             raise KernelError("gemm_rope: partial sums of a norm go with at most 8 rows and no gamma")
     lib = _lib("gemm_bf16")
-    _check(lib, lib.gb_gemm_bf16_rope(_p(a), _rows(a, "a"), _p(w), _rows(w, "w"), _p(qkv), _rows(qkv, "qkv"), M, N, K,
+    _launch(lib, lib.gb_gemm_bf16_rope, _p(a), _rows(a, "a"), _p(w), _rows(w, "w"), _p(qkv), _rows(qkv, "qkv"), M, N, K,
                                       _p(gamma), dtype_code(gamma) if gamma is not None else 0, float(eps), _p(parts),
                                       int(n_parts), _p(cos), _p(sin), _p(slots), _p(k_pages), _p(v_pages), n_heads,
-                                      n_kv_heads, head_dim, page_size, _stream()))
+                                      n_kv_heads, head_dim, page_size, _stream())
 
 
 # ----------------------------------------------------------------------- attention
@@ -475,9 +603,9 @@ def attention_plain(q: torch.Tensor, out: torch.Tensor, positions: torch.Tensor,
     if tables.dtype != torch.int32 or tables.dim() != 2 or tables.stride(1) != 1:
         raise KernelError("attention: block tables must be int32 [requests, pages]")
     lib = _lib("attention_plain")
-    _check(lib, lib.gb_attention_plain(_p(q), _rows(q, "q"), _p(out), _rows(out, "out"), dtype_code(q), _p(positions),
+    _launch(lib, lib.gb_attention_plain, _p(q), _rows(q, "q"), _p(out), _rows(out, "out"), dtype_code(q), _p(positions),
                                        _p(tok_seq), _p(tables), tables.stride(0), _p(k_pages), _p(v_pages), n,
-                                       n_heads, nkv, hd, page_size, float(scale), int(window), _stream()))
+                                       n_heads, nkv, hd, page_size, float(scale), int(window), _stream())
 
 
 def tuned_attention_supports(k_pages: torch.Tensor, n_heads: int, window: int) -> bool:
@@ -515,10 +643,10 @@ def attention_decode(q: torch.Tensor, out: torch.Tensor, ctx, cache, n_heads: in
     ws_acc = ctx.buffer("attn_ws_acc", (n_dec * n_heads * splits * hd,), torch.float32)
     ws_ml = ctx.buffer("attn_ws_ml", (n_dec * n_heads * splits * 2,), torch.float32)
     lib = _lib("attention_bf16")
-    _check(lib, lib.gb_attention_decode_bf16(_p(q), _rows(q, "q"), _p(out), _rows(out, "out"), _p(ws_acc), _p(ws_ml),
+    _launch(lib, lib.gb_attention_decode_bf16, _p(q), _rows(q, "q"), _p(out), _rows(out, "out"), _p(ws_acc), _p(ws_ml),
                                              _p(ctx.positions), _p(tables), tables.stride(0), _p(k_pages), _p(v_pages),
                                              n_dec, n_heads, nkv, hd, page, float(scale), int(window), chunk,
-                                             max_context, _stream()))
+                                             max_context, _stream())
 
 
 @functools.lru_cache(maxsize=4096)
@@ -542,11 +670,11 @@ def attention_prefill(q: torch.Tensor, out: torch.Tensor, ctx, cache, n_heads: i
     first_row, n_rows = n_dec, q.shape[0] - n_dec
     parts = _prefill_parts(max_q, max_ctx, n_heads, S - n_dec, hd)
     ws = ctx.buffer("attn_parts", (parts * n_rows * n_heads * (hd + 2),), torch.float32) if parts > 1 else None
-    _check(lib, lib.gb_attention_prefill_bf16(_p(q), _rows(q, "q"), _p(out), _rows(out, "out"), _p(ctx.q_start),
+    _launch(lib, lib.gb_attention_prefill_bf16, _p(q), _rows(q, "q"), _p(out), _rows(out, "out"), _p(ctx.q_start),
                                               _p(ctx.q_len), _p(ctx.pos0), n_dec, S - n_dec, max_q, max_ctx, _p(tables),
                                               tables.stride(0), _p(k_pages), _p(v_pages), n_heads, nkv, hd, page,
                                               float(scale), int(window), first_row, n_rows, _p(ws),
-                                              ws.numel() if ws is not None else 0, _stream()))
+                                              ws.numel() if ws is not None else 0, _stream())
 
 
 # ------------------------------------------------------------------------ sampling
@@ -561,7 +689,7 @@ def argmax(logits: torch.Tensor, out: torch.Tensor) -> None:
     rows, vocab = _logit_rows(logits)
     _i32(out, "out", rows)
     lib = _lib("sampling")
-    _check(lib, lib.gb_argmax(_p(logits), _p(out), rows, vocab, _stream()))
+    _launch(lib, lib.gb_argmax, _p(logits), _p(out), rows, vocab, _stream())
 
 
 def penalize(logits: torch.Tensor, rows: torch.Tensor, tokens: torch.Tensor, counts: torch.Tensor,
@@ -574,7 +702,7 @@ def penalize(logits: torch.Tensor, rows: torch.Tensor, tokens: torch.Tensor, cou
     if penalties.dtype != torch.float32 or penalties.numel() < pairs:
         raise KernelError("penalize: penalties must be float32, one per pair")
     lib = _lib("sampling")
-    _check(lib, lib.gb_penalize(_p(logits), vocab, _p(rows), _p(tokens), _p(counts), _p(penalties), pairs, _stream()))
+    _launch(lib, lib.gb_penalize, _p(logits), vocab, _p(rows), _p(tokens), _p(counts), _p(penalties), pairs, _stream())
 
 
 def sample(logits: torch.Tensor, temperature: torch.Tensor, top_k: torch.Tensor, top_p: torch.Tensor,
@@ -589,5 +717,5 @@ def sample(logits: torch.Tensor, temperature: torch.Tensor, top_k: torch.Tensor,
     _i32(out_token, "out_token", rows)
     _i32(out_candidates, "out_candidates", rows)
     lib = _lib("sampling")
-    _check(lib, lib.gb_sample(_p(logits), rows, vocab, _p(temperature), _p(top_k), _p(top_p), _p(min_p), _p(uniform),
-                              _p(out_token), _p(out_candidates), _stream()))
+    _launch(lib, lib.gb_sample, _p(logits), rows, vocab, _p(temperature), _p(top_k), _p(top_p), _p(min_p), _p(uniform),
+                              _p(out_token), _p(out_candidates), _stream())

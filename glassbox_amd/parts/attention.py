@@ -39,6 +39,7 @@ def paged_attention(ctx, q: torch.Tensor, out: torch.Tensor, cache: LayerCache, 
 
 class PagedAttention(Mixer):
     replayable = True
+    taped = True
 
     def __init__(self, width: int, n_heads: int, n_kv_heads: int, head_dim: int, position: PositionEncoding,
                  window: int = 0, shares_kv: bool = False, scale: Optional[float] = None):
@@ -69,6 +70,9 @@ class PagedAttention(Mixer):
 
     def all_replayable(self) -> bool:
         return self.replayable and self.position.all_replayable()
+
+    def all_taped(self) -> bool:
+        return self.taped and self.position.all_taped()
 
     def load(self, tensors):
         if self.shares_kv:

@@ -23,6 +23,8 @@ Interfaces (all activations are [tokens, width] tensors on the device;
   Part.problems(dtype, page_size)                   what the kernels would refuse, asked when the engine is built
   Part.replayable                                   class attribute: the part's launches may be replayed
                                                     from a HIP graph (see Part)
+  Part.taped                                        class attribute: the part's launches may be recorded and
+                                                    made again for the next layer like it (see Part)
 
 Optional, for steps of few rows (each part says by a class attribute whether it takes part):
   ``accepts_fused_norm``: forward(..., norm=) takes the un-normed residual and either the norm's
@@ -93,8 +95,20 @@ class Part:
     #: part that reads the context's host lists, synchronises or allocates leaves this False.
     replayable = False
 
+    #: True if ``forward`` does all of its device work through ``glassbox_amd.ops`` and decides what to launch by
+    #: nothing but the step (``ctx``), the arguments of ``forward`` and the part's own constants, which are
+    #: attributes holding numbers, strings, truth values or tuples of them (names that begin with an underscore are
+    #: the part's working state and do not count); its tensors are attributes too.  The
+    #: launches of one layer then serve every layer of the same parts and constants in the same step, with the
+    #: tensors exchanged, and the model walks only the first of them through Python (``parts.tape``).  A part that
+    #: launches anything by other means (a torch operator), or decides by anything else, leaves this False.
+    taped = False
+
     def all_replayable(self) -> bool:
         return self.replayable and all(c.all_replayable() for c in self.children().values())
+
+    def all_taped(self) -> bool:
+        return self.taped and all(c.all_taped() for c in self.children().values())
 
     def tensor_specs(self) -> Dict[str, TensorSpec]:
         return {}

@@ -18,6 +18,7 @@ from .base import Block, CacheSpec, FeedForward, LayerCache, Mixer, Norm, Normed
 
 class PreNormBlock(Block):
     replayable = True
+    taped = True
 
     def __init__(self, mixer_norm: Norm, mixer: Mixer, ffn_norm: Norm, ffn: FeedForward,
                  names=("input_layernorm", "self_attn", "post_attention_layernorm", "mlp")):

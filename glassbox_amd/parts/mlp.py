@@ -12,6 +12,7 @@ from .base import FeedForward, PreNormed, TensorSpec, emit_target, needs_multipl
 
 class SwiGLU(FeedForward):
     replayable = True
+    taped = True
 
     def __init__(self, width: int, intermediate: int):
         self.width, self.intermediate = width, intermediate

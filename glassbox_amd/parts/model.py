@@ -17,6 +17,7 @@ import torch
 
 from .base import CacheSpec, LayerCache, Norm, Part, StateSpec
 from .embedding import Embedding, LMHead
+from .tape import LayerTapes
 
 
 @dataclass(frozen=True)
@@ -42,6 +43,8 @@ class DecoderModel(Part):
         self.vocab_size = embedding.vocab
         self.width = embedding.width
         self._check_schedule()
+        self._tape_sites: dict = {}                    # what parts.tape keeps of each schedule entry
+        self._taped: Optional[List[bool]] = None       # which blocks allow it
 
     # structure ------------------------------------------------------------------
     def children(self) -> Dict[str, Part]:
@@ -84,6 +87,9 @@ class DecoderModel(Part):
         x = ctx.buffer("x", (ctx.n, self.width), torch.float32)
         self.embedding.forward(ctx, x)
         pre = None   # what the block before prepared of this block's first norm
+        if self._taped is None:
+            self._taped = [b.all_taped() for b in self.blocks]
+        tapes = LayerTapes(ctx, self._tape_sites) if getattr(ctx, "layer_tapes", False) and any(self._taped) else None
         for i, call in enumerate(self.schedule):
             if call.cache is not None:
                 cache = caches[call.cache]
@@ -93,17 +99,25 @@ class DecoderModel(Part):
             else:
                 cache = None
             block = self.blocks[call.block]
-            if hasattr(block, "entry_norm"):
+            handover = hasattr(block, "entry_norm")
+            more = {}
+            if handover:
                 after = self.blocks[self.schedule[i + 1].block] if i + 1 < len(self.schedule) else None
-                emit = after.entry_norm(ctx, ctx.n) if hasattr(after, "entry_norm") else None
-                pre = block.forward(ctx, x, cache, pre=pre, emit=emit)
+                more = {"pre": pre, "emit": after.entry_norm(ctx, ctx.n) if hasattr(after, "entry_norm") else None}
+            if tapes is not None and self._taped[call.block]:
+                # the first layer of a kind walks through its parts and is recorded; the others are replayed
+                out = tapes.forward(i, block, x, cache, more)
             else:
-                block.forward(ctx, x, cache)
-                pre = None
+                out = block.forward(ctx, x, cache, **more)
+            pre = out if handover else None
         if ctx.want.numel() == 0:
             return ctx.buffer("logits", (0, self.vocab_size), torch.float32)
         rows = self.final_norm.forward(ctx, x, rows=ctx.want, out_name="h_out")
         return self.head.forward(ctx, rows)
+
+    def load_tree(self, tensors, prefix: str = "") -> None:
+        super().load_tree(tensors, prefix)
+        self._tape_sites.clear()   # they hold the tensors that were loaded before
 
     def streamed_matrices(self) -> List[torch.Tensor]:
         """Every tensor a step reads whole, once each: those of the scheduled blocks (a block named twice, or a

@@ -12,6 +12,7 @@ from .base import Norm, TensorSpec
 
 class RMSNorm(Norm):
     replayable = True
+    taped = True
 
     def __init__(self, width: int, eps: float):
         self.width = width

@@ -18,6 +18,7 @@ from .base import PositionEncoding
 
 class Rotary(PositionEncoding):
     replayable = True
+    taped = True
 
     def __init__(self, head_dim: int, theta: float):
         if head_dim % 2:
@@ -59,6 +60,7 @@ class Rotary(PositionEncoding):
 class NoPosition(PositionEncoding):
     """Keys and queries as they are; only the cache write."""
     replayable = True
+    taped = True
 
     def fuse_spec(self, ctx, head_dim: int):
         return (None, None)

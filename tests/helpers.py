@@ -27,6 +27,11 @@ TINY_C = dict(architectures=["LlamaForCausalLM"], hidden_size=80, intermediate_s
 TINY_D = dict(architectures=["LlamaForCausalLM"], hidden_size=160, intermediate_size=208, num_hidden_layers=2,
               num_attention_heads=4, num_key_value_heads=2, head_dim=128, vocab_size=200, rope_theta=50000.0,
               rms_norm_eps=2e-6, tie_word_embeddings=False, max_position_embeddings=1024)
+# six layers, so that a step has layers that follow a layer like them (the engine walks the first of a kind through
+# the parts and makes its launches again for the rest); three heads to a group, the smallest head the tuned kernels take
+TINY_E = dict(architectures=["LlamaForCausalLM"], hidden_size=72, intermediate_size=120, num_hidden_layers=6,
+              num_attention_heads=6, num_key_value_heads=2, head_dim=16, vocab_size=150, rope_theta=20000.0,
+              rms_norm_eps=4e-6, tie_word_embeddings=False, max_position_embeddings=512)
 # two layers of SmolLM2-360M's widths (a width of 960, 15 heads in 5 groups): large enough that the
 # products take their many-step paths and attention crosses many pages, small enough for the plain oracle
 MID_M = dict(architectures=["LlamaForCausalLM"], hidden_size=960, intermediate_size=2560, num_hidden_layers=2,
@@ -36,7 +41,7 @@ MID_M = dict(architectures=["LlamaForCausalLM"], hidden_size=960, intermediate_s
 WIDE_W = dict(architectures=["LlamaForCausalLM"], hidden_size=2048, intermediate_size=8192, num_hidden_layers=1,
               num_attention_heads=32, num_key_value_heads=32, vocab_size=1000, rope_theta=130000.0,
               rms_norm_eps=1e-5, tie_word_embeddings=True, max_position_embeddings=8192)
-TINY = {"A": TINY_A, "B": TINY_B, "C": TINY_C, "D": TINY_D, "M": MID_M, "W": WIDE_W}
+TINY = {"A": TINY_A, "B": TINY_B, "C": TINY_C, "D": TINY_D, "E": TINY_E, "M": MID_M, "W": WIDE_W}
 
 
 class ModelDirs:

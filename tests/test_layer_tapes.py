@@ -1,0 +1,141 @@
+"""Recorded launches (ops.LaunchTape, csrc/host/launch_tape.cpp) and what makes two layers of a kind
+(parts.tape), without a GPU: the entry points recorded here are callbacks."""
+import ctypes as C
+import struct
+from types import SimpleNamespace
+
+import pytest
+import torch
+
+from glassbox_amd import ops
+from glassbox_amd.parts import tape as layer_tape
+from glassbox_amd.parts.attention import PagedAttention
+from glassbox_amd.parts.base import LayerCache
+from glassbox_amd.parts.block import PreNormBlock
+from glassbox_amd.parts.mlp import SwiGLU
+from glassbox_amd.parts.norm import RMSNorm
+from glassbox_amd.parts.rotary import Rotary
+
+
+class Entry:
+    """What the bindings know of an entry point: its name and the types of its arguments."""
+
+    def __init__(self, name, argtypes):
+        self.__name__, self.argtypes = name, list(argtypes)
+
+
+def fake_entry(name, argtypes, seen, refuse_at=None):
+    """A stand-in for a library with one entry point ``name`` and its taped form, which notes its slots."""
+    @C.CFUNCTYPE(C.c_int, C.POINTER(C.c_uint64))
+    def taped(slots):
+        seen.append([slots[i] for i in range(len(argtypes))])
+        return 1 if refuse_at is not None and len(seen) - 1 == refuse_at else 0
+    lib = SimpleNamespace(gb_last_error=lambda: b"refused on purpose")
+    setattr(lib, name + "_taped", taped)
+    entry = Entry(name, argtypes)
+    return lib, entry
+
+
+def as_float(slot):
+    return struct.unpack("<f", struct.pack("<I", slot & 0xFFFFFFFF))[0]
+
+
+def as_int(slot):
+    return struct.unpack("<q", struct.pack("<Q", slot))[0]
+
+
+def test_a_replayed_launch_moves_pointers_between_tensors_and_keeps_the_rest():
+    seen = []
+    lib, entry = fake_entry("fake_a", [C.c_void_p, C.c_int, C.c_float, C.c_void_p, C.c_longlong, C.c_void_p, C.c_void_p], seen)
+    w1, w2 = torch.zeros(64, dtype=torch.float32), torch.zeros(64, dtype=torch.float32)
+    p1, p2 = torch.zeros(8, 16, dtype=torch.bfloat16), torch.zeros(8, 16, dtype=torch.bfloat16)
+    shared = torch.zeros(32)
+    tape = ops.LaunchTape()
+    tape.add(lib, entry, (w1.data_ptr() + 40, -3, 1.5, None, 1 << 40, p1.data_ptr(), shared.data_ptr()))
+    tape.add(lib, entry, (p1.data_ptr() + 255, 7, -0.25, w1.data_ptr(), -1, w1.data_ptr() + 256, shared.data_ptr() + 4))
+    assert len(tape) == 2 and tape.usable
+    ops.run_tape(tape, ops.TapeOperands([w1, p1]), ops.TapeOperands([w2, p2]))
+    a, b = seen
+    assert a[0] == w2.data_ptr() + 40 and as_int(a[1]) == -3 and as_float(a[2]) == 1.5 and a[3] == 0
+    assert as_int(a[4]) == 1 << 40 and a[5] == p2.data_ptr() and a[6] == shared.data_ptr()
+    assert b[0] == p2.data_ptr() + 255 and as_int(b[1]) == 7 and as_float(b[2]) == -0.25 and b[3] == w2.data_ptr()
+    assert as_int(b[4]) == -1
+    # one past the end of a tensor is not inside it: the pointer stays (unless the tensors happen to touch)
+    if w1.data_ptr() + 256 != p1.data_ptr():
+        assert b[5] == w1.data_ptr() + 256
+    assert b[6] == shared.data_ptr() + 4
+
+
+def test_a_replay_stops_at_the_launch_that_is_refused_and_says_why():
+    seen = []
+    lib, entry = fake_entry("fake_b", [C.c_void_p, C.c_int], seen, refuse_at=1)
+    t = torch.zeros(4)
+    tape = ops.LaunchTape()
+    for i in range(3):
+        tape.add(lib, entry, (t.data_ptr(), i))
+    with pytest.raises(ops.KernelError, match="refused on purpose"):
+        ops.run_tape(tape, ops.TapeOperands([t]), ops.TapeOperands([t]))
+    assert [as_int(s[1]) for s in seen] == [0, 1]
+
+
+def test_a_launch_without_a_taped_form_spoils_the_tape_and_other_sizes_are_refused():
+    lib = SimpleNamespace()
+    entry = Entry("fake_c", [C.c_int])
+    tape = ops.LaunchTape()
+    tape.add(lib, entry, (1,))
+    assert not tape.usable
+    seen = []
+    lib, entry = fake_entry("fake_d", [C.c_void_p], seen)
+    tape = ops.LaunchTape()
+    tape.add(lib, entry, (0,))
+    with pytest.raises(ops.KernelError, match="do not match"):
+        ops.run_tape(tape, ops.TapeOperands([torch.zeros(4)]), ops.TapeOperands([torch.zeros(5)]))
+    assert not seen
+
+
+def block(width=32, heads=4, kv=2, hd=8, inter=48, eps=1e-5, theta=10000.0, window=0, rotary=None):
+    rotary = rotary or Rotary(hd, theta)
+    return PreNormBlock(RMSNorm(width, eps), PagedAttention(width, heads, kv, hd, rotary, window=window),
+                        RMSNorm(width, eps), SwiGLU(width, inter))
+
+
+def load_random(b):
+    for part in (b.mixer_norm, b.mixer, b.ffn_norm, b.ffn):
+        part.load({name: torch.randn(spec.shape) for name, spec in part.tensor_specs().items()})
+
+
+def test_layers_are_of_a_kind_by_classes_and_constants():
+    shared = Rotary(8, 10000.0)
+    a, b = block(rotary=shared), block(rotary=shared)
+    assert a.all_taped()
+    assert layer_tape.signature(a) == layer_tape.signature(b)
+    assert layer_tape.signature(a) == layer_tape.signature(block())            # a rotary of its own with the same constants
+    for other in (block(eps=1e-6), block(theta=500000.0), block(window=64), block(heads=2), block(inter=64)):
+        assert layer_tape.signature(other) != layer_tape.signature(a)
+
+    class OtherFeedForward(SwiGLU):
+        pass
+    c = PreNormBlock(RMSNorm(32, 1e-5), PagedAttention(32, 4, 2, 8, shared), RMSNorm(32, 1e-5), OtherFeedForward(32, 48))
+    assert layer_tape.signature(c) != layer_tape.signature(a)
+    assert not c.all_taped() or OtherFeedForward.taped   # a subclass inherits what its base said
+
+    class Untaped(SwiGLU):
+        taped = False
+    d = PreNormBlock(RMSNorm(32, 1e-5), PagedAttention(32, 4, 2, 8, shared), RMSNorm(32, 1e-5), Untaped(32, 48))
+    assert not d.all_taped()
+
+
+def test_a_layers_tensors_come_in_one_order_and_include_cache_and_the_next_norm():
+    a, b = block(), block()
+    load_random(a)
+    load_random(b)
+    ta, tb = layer_tape.tensors_of(a), layer_tape.tensors_of(b)
+    assert len(ta) == len(tb) == 6                                   # two gammas, qkv, o, gate/up, down
+    assert [t.shape for t in ta] == [t.shape for t in tb]
+    assert all(x.data_ptr() != y.data_ptr() for x, y in zip(ta, tb))
+    assert any(t is a.mixer.wqkv for t in ta) and any(t is a.ffn.w_down for t in ta)
+    cache = LayerCache(torch.zeros(3, 2, 1, 16, 8), torch.zeros(3, 2, 8, 16), 0, torch.zeros(4, 5))
+    assert [t.data_ptr() for t in layer_tape.tensors_of(cache)] == [cache.k_pages.data_ptr(), cache.v_pages.data_ptr(),
+                                                                    cache.state.data_ptr()]
+    gamma = torch.ones(32)
+    assert layer_tape.tensors_of((gamma, 1e-5))[0] is gamma and layer_tape.tensors_of(None) == []

@@ -22,6 +22,7 @@ REQUESTS = {
     "B": {"b0": 1, "b1": 33, "b2": 64, "b3": 94, "b4": 200, "b5": 40},
     "C": {"c0": 3, "c1": 47, "c2": 130, "c3": 65, "c4": 257},
     "D": {"d0": 2, "d1": 31, "d2": 150, "d3": 64, "d4": 301},
+    "E": {"e0": 4, "e1": 35, "e2": 96, "e3": 161, "e4": 48},
 }
 # more requests than are live at once, so that finished requests' pages are handed out again
 MORE = {
@@ -29,6 +30,7 @@ MORE = {
     "B": {"b6": 150, "b7": 17, "b8": 256, "b9": 77},
     "C": {"c5": 90, "c6": 33, "c7": 200, "c8": 16, "c9": 129},
     "D": {"d5": 70, "d6": 129, "d7": 18, "d8": 260},
+    "E": {"e5": 66, "e6": 19, "e7": 180, "e8": 97},
 }
 
 
@@ -66,7 +68,7 @@ def engines(model_dirs):
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
-@pytest.mark.parametrize("name", ["A", "B", "C", "D"])
+@pytest.mark.parametrize("name", ["A", "B", "C", "D", "E"])
 @pytest.mark.parametrize("mode", ["whole", "tail32", "chunks"])
 def test_single_request_splits(engines, model_dirs, bf16_bound, name, dtype, mode):
     folder = model_dirs.get(name)
@@ -81,7 +83,7 @@ def test_single_request_splits(engines, model_dirs, bf16_bound, name, dtype, mod
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
-@pytest.mark.parametrize("name", ["A", "B", "C", "D"])
+@pytest.mark.parametrize("name", ["A", "B", "C", "D", "E"])
 def test_mixed_batches_with_page_reuse(model_dirs, bf16_bound, name, dtype):
     from glassbox_amd.engine import Engine
     folder = model_dirs.get(name)
