@@ -259,10 +259,13 @@ def test_gemm_bf16_divides_k_over_workgroups(M, N, K, mode):
                                    # so many narrow tiles that a workgroup takes 64 columns
                                    (128, 24600, 320), (96, 32760, 512),
                                    # 33 to 64 rows by very many rows of W: the wide tiles, not the skinny kernel
-                                   (64, 49152, 256), (40, 33000, 192)])
+                                   (64, 49152, 256), (40, 33000, 192),
+                                   # a narrow model's products: few narrow tiles and a k too short to divide; and up to
+                                   # 256 rows (two row tiles) where the wide tiles would be fewer still
+                                   (96, 2560, 960), (200, 5120, 960), (256, 2500, 448), (129, 2100, 128)])
 @pytest.mark.parametrize("mode", ["bf16", "f32", "f32+", "silu"])
 def test_gemm_bf16_streams_products_of_some_hundred_rows(M, N, K, mode):
-    """65 to 128 rows, a k that is a multiple of 64: tiles of 128 rows by 32 or 64 columns, both operands through
+    """65 to 128 rows (to 256 in a narrow model), a k that is a multiple of 64: tiles of 128 rows by 32 or 64 columns, both operands through
     rings in LDS, no slices of k where the narrow tiles alone fill the chip (with or without a workspace on offer).
     Against float64, the same bits on every run, rows and columns beyond the last tile's edge untouched."""
     from glassbox_amd import ops
