@@ -299,20 +299,31 @@ int launch_tiled(const bf16* a, int lda, const bf16* w, int ldw, CT* c, int ldc,
   tiled_plan(M, N, &wn, &depth);
   if (EPI == EPI_SILU_MUL) wn = 2;  // a wave's two column tiles are gate and up
   const int cols = EPI == EPI_SILU_MUL ? N / 2 : N, bn = EPI == EPI_SILU_MUL ? 64 : 64 * wn;
-  const dim3 grid((cols + bn - 1) / bn, (M + 127) / 128), block(256);
+  // Tiles of 64 rows where those of 128 would leave a third of the compute units without a workgroup (the
+  // products of a narrow model at some hundred rows): a workgroup's time is its k-steps' arithmetic, and half the
+  // rows halve it.
+  const bool low = M > 64 && ((cols + bn - 1) / bn) * ((M + 127) / 128) < 168;
+  const int bm = low ? 64 : 128;
+  const dim3 grid((cols + bn - 1) / bn, (M + bm - 1) / bm), block(256);
   GB_REQUIRE(grid.y <= 65535, "gemm_bf16: M=%d needs more than 65535 row tiles", M);
   const bool kfull = K % TBK == 0;  // then no load needs a check against K
-#define GB_T(B, D)                                                                                                          \
+#define GB_T(WM, B, D)                                                                                                      \
   if (wn == (B) && depth == (D)) {                                                                                          \
     if (kfull)                                                                                                              \
-      hipLaunchKernelGGL((gemm_tiled_kernel<2, (B), (D), EPI, true, CT>), grid, block, 0, stream, a, lda, w, ldw, c, ldc, M, \
+      hipLaunchKernelGGL((gemm_tiled_kernel<WM, (B), (D), EPI, true, CT>), grid, block, 0, stream, a, lda, w, ldw, c, ldc, M, \
                          N, K, 0);                                                                                          \
     else                                                                                                                    \
-      hipLaunchKernelGGL((gemm_tiled_kernel<2, (B), (D), EPI, false, CT>), grid, block, 0, stream, a, lda, w, ldw, c, ldc,   \
+      hipLaunchKernelGGL((gemm_tiled_kernel<WM, (B), (D), EPI, false, CT>), grid, block, 0, stream, a, lda, w, ldw, c, ldc,  \
                          M, N, K, 0);                                                                                       \
   }
-  GB_T(2, 1) GB_T(2, 2)
-  if (EPI != EPI_SILU_MUL) { GB_T((EPI == EPI_SILU_MUL ? 2 : 1), 1) GB_T((EPI == EPI_SILU_MUL ? 2 : 1), 2) }
+  if (low) {
+    depth = wn == 1 ? 2 : 1;
+    GB_T(1, 2, 1)
+    if (EPI != EPI_SILU_MUL) { GB_T(1, (EPI == EPI_SILU_MUL ? 2 : 1), 2) }
+  } else {
+    GB_T(2, 2, 1) GB_T(2, 2, 2)
+    if (EPI != EPI_SILU_MUL) { GB_T(2, (EPI == EPI_SILU_MUL ? 2 : 1), 1) GB_T(2, (EPI == EPI_SILU_MUL ? 2 : 1), 2) }
+  }
 #undef GB_T
   return launched("gemm_bf16 (tiled)");
 }
@@ -861,6 +872,8 @@ inline SplitPlan split_plan(int M, int N, int K) {
   p.slices = (K + p.k_slice - 1) / p.k_slice;
   if (p.slices < 2) return SplitPlan{p.bm, 1, 0, 0, false, false};
   p.floats = (size_t)p.slices * M * N;
+  // tiles of 64 rows where even with the slices a third of the compute units would have no workgroup
+  if (tiles * p.slices < 168) p.bm = 64;
   return p;
 }
 
@@ -1521,7 +1534,8 @@ extern "C" int gb_gemm_bf16(const void* a, int lda, const void* w, int ldw, void
   // long enough k the plan above has divided it instead); up to 256 rows where the wide tiles would be few and k is
   // too short to divide (the products of a narrow model: SmolLM2-360M's gate/up of 256 rows, 16.3 -> 11.2 us).
   const int narrow_tiles = ((ncols + 31) / 32) * ((M + SBM - 1) / SBM), wide_tiles = ((N + 127) / 128) * ((M + 127) / 128);
-  const bool narrow_pays = M <= STREAM_MAX_ROWS ? narrow_tiles >= 64 : (M <= 2 * STREAM_MAX_ROWS && narrow_tiles >= 64 && wide_tiles < 128 && K < 2048);
+  const bool narrow_pays = M <= STREAM_MAX_ROWS ? narrow_tiles >= 64
+                                               : (M <= 2 * STREAM_MAX_ROWS && epilogue == EPI_SILU_MUL && narrow_tiles >= 64 && wide_tiles < 128 && K < 2048);
   if (M > STREAM_MIN_ROWS && narrow_pays && !gamma && !parts && !emit_h && stream_takes(a, lda, w, ldw, K) &&
       (epilogue != EPI_SILU_MUL || N % 16 == 0) && N < 32768) {
     const bf16* A = (const bf16*)a;

@@ -63,7 +63,7 @@ def test_gemm_bf16(N, K, M, out):
 
 @pytest.mark.parametrize("I,K,M", [(8, 32, 1), (176, 64, 5), (144, 80, 16), (200, 2048, 17), (8192, 2048, 8), (88, 4104, 64),
                                    # more than 64 rows: the tiled kernel's epilogue
-                                   (176, 64, 130), (72, 264, 65), (1024, 520, 300), (2560, 960, 200), (1000, 2048, 129)])
+                                   (176, 64, 130), (72, 264, 65), (1024, 520, 300), (2560, 960, 200), (2560, 960, 400), (1000, 2048, 129)])
 def test_gemm_bf16_fused_silu_mul(I, K, M):
     """Stacked gate/up rows with the activation applied in the product's epilogue
     (crates/glassbox-core/src/model.rs:335-340), against the formula in float64."""
