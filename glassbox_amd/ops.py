@@ -170,6 +170,7 @@ class LaunchTape:
     def __init__(self):
         self.data = bytearray()
         self.libs: list = []          # the library of each launch: it holds the message if a replay refuses
+        self.names: List[str] = []    # the entry point of each launch
         self.usable = True            # False once a launch was made that cannot be made again natively
         self._c = None
 
@@ -184,6 +185,7 @@ class LaunchTape:
         st, address, mask, n = how
         self.data += st.pack(address, mask, n, 0, *[0 if a is None else a for a in args])
         self.libs.append(lib)
+        self.names.append(entry.__name__)
 
     def pointer(self):
         if self._c is None:

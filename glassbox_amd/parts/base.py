@@ -98,7 +98,8 @@ class Part:
     #: True if ``forward`` does all of its device work through ``glassbox_amd.ops`` and decides what to launch by
     #: nothing but the step (``ctx``), the arguments of ``forward`` and the part's own constants, which are
     #: attributes holding numbers, strings, truth values or tuples of them (names that begin with an underscore are
-    #: the part's working state and do not count); its tensors are attributes too.  The
+    #: the part's working state and do not count); its tensors are attributes too; what it computes once a step for
+    #: all layers it keeps in ``ctx.memo`` (a walk that adds to the memo is not recorded).  The
     #: launches of one layer then serve every layer of the same parts and constants in the same step, with the
     #: tensors exchanged, and the model walks only the first of them through Python (``parts.tape``).  A part that
     #: launches anything by other means (a torch operator), or decides by anything else, leaves this False.

@@ -15,6 +15,8 @@ What makes two layers of a kind is decided here, from the parts themselves, and 
 * the blocks have one ``signature``: the same classes, arranged alike, with the same constants (every
   attribute that is a number, a string, a truth value or a tuple or list of such, but for those whose names begin
   with an underscore);
+* the walk of the recorded layer added nothing to the step's memo (``ctx.memo``: what a part computes once a step
+  for all layers, like the rotation's table, is not among the launches of the layers after it);
 * they are called alike: what the block before prepared of the first norm, whether the block after asks for its
   norm to be prepared, the kind and shapes of the cache layer, the residual buffer;
 * their tensors (the attributes of the parts that are tensors, the cache layer's pages and state, the gamma of a
@@ -194,13 +196,16 @@ class LayerTapes:
             site.forget()
             return result
         # the first layer of its kind in this step (or a buffer of the step has grown since that one was recorded)
+        memo = len(ctx.memo)
         tape = ops.start_tape()
         try:
             result = block.forward(ctx, x, cache, **kwargs)
         finally:
             ops.stop_tape()
         site.forget()   # the walk may have made tensors that the parts keep
-        if tape.usable and len(tape) and ctx.workspace.epoch == epoch:
+        # a walk that added to the step's memo did work that is done once a step (the rotation's table): its launches
+        # are not those of the layers after it, so the next layer of the kind is walked and recorded instead
+        if tape.usable and len(tape) and ctx.workspace.epoch == epoch and len(ctx.memo) == memo:
             self.records[key] = _Record(tape, site.tensors(), result, epoch)
             ops.TAPE_COUNTS["recorded_layers"] += 1
         return result

@@ -118,3 +118,24 @@ def test_layers_of_two_kinds_are_recorded_apart_and_a_block_named_twice_is_repla
         assert np.array_equal(got[True][r], got[False][r]), f"request {r}: replayed layers changed the logits"
     # and the windowed layers did matter: the same model without windows says something else
     assert len(eng.group_keys) == 2
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_what_is_done_once_a_step_is_not_replayed(model_dirs, monkeypatch, dtype):
+    """The first layer's walk computes the rotation's table for the whole step.  Its launches are therefore not
+    those of the layers after it: no replayed layer may compute the table again (steps of 40 rows, where nothing is
+    handed over between layers and the first layer is of the same kind as the rest)."""
+    from glassbox_amd import ops
+    from glassbox_amd.engine import Engine
+    folder = model_dirs.get("E")
+    replayed = []
+    real = ops.run_tape
+    monkeypatch.setattr(ops, "run_tape", lambda tape, a, b: (replayed.append(list(tape.names)), real(tape, a, b))[1])
+    eng = Engine(folder, dtype=dtype, max_tokens=512, max_seqs=4, graph_decode=False)
+    toks = helpers.random_tokens(helpers.TINY["E"]["vocab_size"], 120, seed=9)
+    eng.step([("a", toks[:40], [39])])
+    eng.step([("a", toks[40:80], [39])])
+    eng.step([("a", toks[80:81], [0]), ("b", toks[:39], [])])
+    assert len(replayed) >= 3 * 3, "layers were not replayed"
+    assert all("gb_rope_table" not in names for names in replayed)
+    assert all(any(n.startswith("gb_gemm") for n in names) for names in replayed)
