@@ -1065,7 +1065,7 @@ __device__ __forceinline__ bf16x8 load_a(const void* a, int lda, int m, int k, b
   return out;
 }
 
-template <int MT, int WAVES, int ITERS, int RT, int EPI, bool RMS, typename CT>
+template <int MT, int WAVES, int ITERS, int RT, int EPI, bool RMS, typename CT, bool HALF = false>
 __global__ __launch_bounds__(WAVES * 64) void gemm_skinny_kernel(const void* __restrict__ a, int lda,
                                                                  const bf16* __restrict__ w, int ldw, CT* __restrict__ c,
                                                                  int ldc, int M, int N, int K, const void* __restrict__ gamma,
@@ -1098,10 +1098,12 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_skinny_kernel(const void* __r
       // a tile is 8 pairs of one head: its dims d0..d0+7 and those hd/2 further on
       const int per_head = rope.hd / 16, head = tile / per_head, d0 = (tile % per_head) * 8;
       row = head * rope.hd + (r < 8 ? d0 + r : rope.hd / 2 + d0 + (r - 8));
+    } else if (HALF) {
+      row = tile * 8 + (r & 7);  // a workgroup owns 8 rows of W: the tile's lower half stays empty
     } else {
       row = tile * 16 + r;
     }
-    row_ok[rt] = EPI == EPI_SILU_MUL ? (tile * 8 + (r & 7) < N / 2) : row < N;
+    row_ok[rt] = EPI == EPI_SILU_MUL ? (tile * 8 + (r & 7) < N / 2) : HALF ? (r < 8 && row < N) : row < N;
     wrow[rt] = w + (size_t)(row_ok[rt] ? row : 0) * ldw;
   }
 
@@ -1269,10 +1271,12 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_skinny_kernel(const void* __r
     // accumulating: all of a thread's old values are asked for before any is added to (behind the checks one
     // by one, every read would wait for the one before it)
     float old[RT][MT];
+    if (HALF && nrow >= 8) return;
+    constexpr int ROWS = HALF ? 8 : 16;  // rows of W a tile owns
     if (EPI == EPI_ACCUMULATE) {
 #pragma unroll
       for (int rt = 0; rt < RT; ++rt) {
-        const int n = (blockIdx.x * RT + rt) * 16 + nrow;
+        const int n = (blockIdx.x * RT + rt) * ROWS + nrow;
 #pragma unroll
         for (int t = 0; t < MT; ++t) {
           const int m = t * 16 + l % 16;
@@ -1282,7 +1286,7 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_skinny_kernel(const void* __r
     }
 #pragma unroll
     for (int rt = 0; rt < RT; ++rt) {
-      const int n = (blockIdx.x * RT + rt) * 16 + nrow;
+      const int n = (blockIdx.x * RT + rt) * ROWS + nrow;
 #pragma unroll
       for (int t = 0; t < MT; ++t) {
         const int m = t * 16 + l % 16;
@@ -1440,6 +1444,21 @@ int launch_skinny_mt(int tiles, const void* a, int lda, const bf16* w, int ldw, 
                      hipStream_t stream) {
   int waves, iters, rt;
   skinny_plan(tiles, K, MT, &waves, &iters, &rt);
+  if constexpr ((EPI == EPI_STORE || EPI == EPI_ACCUMULATE) && !RMS) {
+    // Few rows of W (a narrow model's O and down projections, beyond the 8 rows of A that the folded kernel takes):
+    // workgroups of 8 rows of W, half of each tile left empty, so that twice as many compute units draw on memory.
+    if (tiles < 256 && extra.parts == nullptr) {
+      const int halves = (N + 7) / 8;
+#define GB_HALF(WV, IT)                                                                                                    \
+  if (waves == WV && iters == (IT))                                                                                        \
+    hipLaunchKernelGGL((gemm_skinny_kernel<MT, WV, (IT), 1, EPI, RMS, CT, true>), dim3(halves), dim3(WV * 64), 0, stream, a, \
+                       lda, w, ldw, c, ldc, M, N, K, gamma, gamma_f32, eps, extra.parts, extra.n_parts, rope);
+      GB_HALF(4, 1) GB_HALF(16, 1)
+      if (MT == 1) { GB_HALF(4, MT == 1 ? 2 : 1) GB_HALF(16, MT == 1 ? 2 : 1) }
+#undef GB_HALF
+      return launched("gemm_bf16 (skinny, half tiles)");
+    }
+  }
 #define GB_CFG(WV, IT, RT)                                                                                                 \
   if (waves == WV && iters == (IT) && rt == RT)                                                                            \
     hipLaunchKernelGGL((gemm_skinny_kernel<MT, WV, (IT), RT, EPI, RMS, CT>), dim3((tiles + RT - 1) / RT), dim3(WV * 64), 0,  \
