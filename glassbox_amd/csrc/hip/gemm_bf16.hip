@@ -36,13 +36,15 @@ __device__ __forceinline__ bf16x8 zero8() {
   return z;
 }
 
-// What a product of at most 8 rows may do for the RMS norm that follows it or precedes it.
-//  * emit (the folded kernel, accumulating into the float32 residual): besides the new residual r it
-//    writes h[m, n] = bf16(gamma[n] * r[m, n]), the operand of the next product, and for every tile of 8
-//    columns the sums over them of r[m, n]^2 to ss[tile * 8 + m]: the next norm's pass over the residual
-//    is done where the residual is made.
+// What a product of at most 64 rows may do for the RMS norm that follows it or precedes it.
+//  * emit (the folded kernel for up to 8 rows, the skinny kernel beyond; accumulating into the float32 residual):
+//    besides the new residual r it writes h[m, n] = bf16(gamma[n] * r[m, n]), the operand of the next product, and
+//    for every tile of columns (8 or 16: gb_gemm_bf16_emit_parts says how many tiles) the sums over them of
+//    r[m, n]^2 to ss[tile * stride + m]: the next norm's pass over the residual is done where the residual is made.
+//    stride = parts_stride(M): 8 for up to 8 rows, 64 beyond.
 //  * parts (the skinny kernel): the rows of A are such an h; the product is scaled by
 //    1 / sqrt(sum of the n_parts partial sums of row m / K + eps), added up in the order of the tiles.
+__host__ __device__ __forceinline__ int parts_stride(int M) { return M <= 8 ? 8 : 64; }
 struct NormExtras {
   const void* emit_gamma;
   int emit_gamma_f32;
@@ -970,12 +972,20 @@ __global__ __launch_bounds__(256) void splitk_reduce_norm_kernel(const float* __
 inline bool fold_pays(int M, int N) { return M <= 8 && (N + 15) / 16 < 256; }
 
 // What an accumulating product of these sizes can do for the RMS norm that reads the residual after it:
-// 0 nothing; 1 (the folded kernel, at most 8 rows) the operand bf16(gamma * r) and partial sums, see NormExtras;
+// 0 nothing; 1 (the folded kernel for at most 8 rows, the skinny kernel up to 64) the operand bf16(gamma * r) and
+// partial sums, see NormExtras;
 // 2 (a product that divides k, given its workspace) the whole norm, in the pass that adds the slices.
 inline int emit_mode(int M, int N, int K) {
   if (fold_pays(M, N)) return 1;
   if (M > 16 && N % 4 == 0 && N <= SPLIT_NORM_MAX && split_plan(M, N, K).slices > 1) return 2;
+  if (M <= 64 && !(M > 32 && N >= 32768)) return 1;  // the skinny kernel
   return 0;
+}
+// Tiles of columns for which an emitting product of these sizes writes partial sums.
+inline int emit_parts(int M, int N) {
+  if (fold_pays(M, N)) return (N + 7) / 8;
+  if (M > 64) return 0;
+  return (N + 15) / 16 < 256 ? (N + 7) / 8 : (N + 15) / 16;  // the skinny kernel: half tiles while the tiles are few
 }
 
 template <int EPI, typename CT>
@@ -1065,25 +1075,51 @@ __device__ __forceinline__ bf16x8 load_a(const void* a, int lda, int m, int k, b
   return out;
 }
 
+// (Up to 16 rows, sixteen waves, two row tiles and two loads in flight: the kernel needs exactly 64 registers a lane,
+// with which two workgroups share a compute unit, one's loads on their way while the other adds up and stores.  One
+// register more and only one fits: decode steps of one to eight requests were 4 % slower.)
 template <int MT, int WAVES, int ITERS, int RT, int EPI, bool RMS, typename CT, bool HALF = false>
 __global__ __launch_bounds__(WAVES * 64) void gemm_skinny_kernel(const void* __restrict__ a, int lda,
                                                                  const bf16* __restrict__ w, int ldw, CT* __restrict__ c,
                                                                  int ldc, int M, int N, int K, const void* __restrict__ gamma,
-                                                                 int gamma_f32, float eps, const float* __restrict__ parts,
-                                                                 int n_parts, RopeExtras rope) {
+                                                                 int gamma_f32, float eps, NormExtras extra, RopeExtras rope) {
   __shared__ float part[WAVES][RT][MT][64][4];
   __shared__ float sspart[RMS ? WAVES : 1][MT][64];
-  __shared__ float red[64][8];
+  constexpr int PJ = WAVES * 64 / (MT * 16) < 64 ? WAVES * 64 / (MT * 16) : 64;  // threads that share a row's partial sums
+  __shared__ float red[RMS ? 1 : PJ][MT * 16];  // (with RMS the rows bring no partial sums)
+  __shared__ float emit_sq[4][RT][MT][16];
+  const float* __restrict__ parts = extra.parts;
+  const int n_parts = extra.n_parts;
   const int tid = threadIdx.x, lane = tid % 64, wave = tid / 64;
   const int r = lane % 16, q = lane / 16;
+  // Partial sums of squares of the rows, one per tile of the product that made them: some threads a row add up
+  // every so-manieth, the epilogue adds up theirs, both in a fixed order.  Up to 8 rows (8 floats a tile): J8 threads a
+  // row, few terms each.  Beyond (64 floats a tile): PJ threads a row, and where a thread has many terms, four loads
+  // at a time are asked for before any is added (one after the other they would each wait).  The first form is kept
+  // as it is on purpose: with it the sixteen-wave kernel needs 64 registers and fits twice on a compute unit, with
+  // the general form alone the compiler keeps one or two more through the main loop.
+  constexpr int J8 = WAVES * 8 < 64 ? WAVES * 8 : 64;
+  float* red8 = &red[0][0];  // [J8][8]
   if (!RMS && parts != nullptr) {
-    // partial sums of squares of the (at most 8) rows, one per tile of the product that made them:
-    // 64 threads a row add up every 64th, the epilogue adds up those 64, both in a fixed order
-    for (int t = tid; t < 512; t += WAVES * 64) {
-      const int m = t & 7, j = t >> 3;
+    if (M <= 8) {
+      for (int t = tid; t < 8 * J8; t += WAVES * 64) {
+        const int m = t & 7, j = t >> 3;
+        float sum = 0.f;
+        for (int p = j; p < n_parts; p += J8) sum += parts[p * 8 + m];
+        red8[j * 8 + m] = sum;
+      }
+    } else {
+      const int m = tid % (MT * 16), j = tid / (MT * 16);
       float sum = 0.f;
-      for (int p = j; p < n_parts; p += 64) sum += parts[p * 8 + m];
-      red[j][m] = sum;
+      if (m < M && j < PJ)
+        for (int p = j; p < n_parts; p += 4 * PJ) {
+          float got[4];
+#pragma unroll
+          for (int u = 0; u < 4; ++u) got[u] = p + u * PJ < n_parts ? parts[(p + u * PJ) * 64 + m] : 0.f;
+#pragma unroll
+          for (int u = 0; u < 4; ++u) sum += got[u];
+        }
+      if (j < PJ) red[j][m] = sum;
     }
   }
   const bf16* wrow[RT];
@@ -1190,10 +1226,17 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_skinny_kernel(const void* __r
 #pragma unroll
         for (int qq = 0; qq < 4; ++qq) tot += sspart[wv][t][l % 16 + 16 * qq];
       scale = 1.0f / sqrtf(tot / (float)K + eps);
-    } else if (parts != nullptr && l % 16 < 8) {
+    } else if (parts != nullptr) {
       float tot = 0.f;
+      if (M <= 8) {
+        if (l % 16 < 8) {
 #pragma unroll 8
-      for (int j = 0; j < 64; ++j) tot += red[j][l % 16];
+          for (int j = 0; j < J8; ++j) tot += red8[j * 8 + l % 16];
+        }
+      } else {
+#pragma unroll 8
+        for (int j = 0; j < PJ; ++j) tot += red[j][t * 16 + l % 16];
+      }
       scale = 1.0f / sqrtf(tot / (float)K + eps);
     }
 #pragma unroll
@@ -1271,7 +1314,9 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_skinny_kernel(const void* __r
     // accumulating: all of a thread's old values are asked for before any is added to (behind the checks one
     // by one, every read would wait for the one before it)
     float old[RT][MT];
-    if (HALF && nrow >= 8) return;
+    const bool emits = EPI == EPI_ACCUMULATE && extra.emit_h != nullptr;
+    const bool empty = HALF && nrow >= 8;  // the lower half of a half tile
+    if (empty && !emits) return;
     constexpr int ROWS = HALF ? 8 : 16;  // rows of W a tile owns
     if (EPI == EPI_ACCUMULATE) {
 #pragma unroll
@@ -1280,17 +1325,47 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_skinny_kernel(const void* __r
 #pragma unroll
         for (int t = 0; t < MT; ++t) {
           const int m = t * 16 + l % 16;
-          old[rt][t] = (m < M && n < N) ? (float)c[(size_t)m * ldc + n] : 0.f;
+          old[rt][t] = (!empty && m < M && n < N) ? (float)c[(size_t)m * ldc + n] : 0.f;
         }
       }
     }
+    float sq[RT][MT];
 #pragma unroll
     for (int rt = 0; rt < RT; ++rt) {
       const int n = (blockIdx.x * RT + rt) * ROWS + nrow;
 #pragma unroll
       for (int t = 0; t < MT; ++t) {
         const int m = t * 16 + l % 16;
-        if (m < M && n < N) c[(size_t)m * ldc + n] = (CT)(EPI == EPI_ACCUMULATE ? old[rt][t] + v[rt][t] : v[rt][t]);
+        sq[rt][t] = 0.f;
+        if (!empty && m < M && n < N) {
+          const float now = EPI == EPI_ACCUMULATE ? old[rt][t] + v[rt][t] : v[rt][t];
+          c[(size_t)m * ldc + n] = (CT)now;
+          if (emits) {
+            const float g = extra.emit_gamma_f32 ? ((const float*)extra.emit_gamma)[n] : (float)((const bf16*)extra.emit_gamma)[n];
+            extra.emit_h[(size_t)m * extra.emit_ldh + n] = (bf16)(g * now);
+            sq[rt][t] = now * now;
+          }
+        }
+      }
+    }
+    if (emits) {
+      // sum of squares over a tile's columns, per row: a row's 16 cells lie in four neighbouring lanes of each of
+      // the four waves that are still here; added in a fixed order
+#pragma unroll
+      for (int rt = 0; rt < RT; ++rt)
+#pragma unroll
+        for (int t = 0; t < MT; ++t) {
+          float x = sq[rt][t];
+          x += __shfl_xor(x, 1, kWave);
+          x += __shfl_xor(x, 2, kWave);
+          if (e == 0) emit_sq[wave][rt][t][l % 16] = x;
+        }
+      __syncthreads();  // the four waves that are still here
+      const int stride = parts_stride(M);
+      for (int i = tid; i < RT * MT * 16; i += 256) {
+        const int rt = i / (MT * 16), t = i / 16 % MT, mm = i % 16, m = t * 16 + mm;
+        const float tot = emit_sq[0][rt][t][mm] + emit_sq[1][rt][t][mm] + emit_sq[2][rt][t][mm] + emit_sq[3][rt][t][mm];
+        if (m < M) extra.emit_ss[(size_t)(blockIdx.x * RT + rt) * stride + m] = tot;
       }
     }
   }
@@ -1452,7 +1527,7 @@ int launch_skinny_mt(int tiles, const void* a, int lda, const bf16* w, int ldw, 
 #define GB_HALF(WV, IT)                                                                                                    \
   if (waves == WV && iters == (IT))                                                                                        \
     hipLaunchKernelGGL((gemm_skinny_kernel<MT, WV, (IT), 1, EPI, RMS, CT, true>), dim3(halves), dim3(WV * 64), 0, stream, a, \
-                       lda, w, ldw, c, ldc, M, N, K, gamma, gamma_f32, eps, extra.parts, extra.n_parts, rope);
+                       lda, w, ldw, c, ldc, M, N, K, gamma, gamma_f32, eps, extra, rope);
       GB_HALF(4, 1) GB_HALF(16, 1)
       if (MT == 1) { GB_HALF(4, MT == 1 ? 2 : 1) GB_HALF(16, MT == 1 ? 2 : 1) }
 #undef GB_HALF
@@ -1462,7 +1537,7 @@ int launch_skinny_mt(int tiles, const void* a, int lda, const bf16* w, int ldw, 
 #define GB_CFG(WV, IT, RT)                                                                                                 \
   if (waves == WV && iters == (IT) && rt == RT)                                                                            \
     hipLaunchKernelGGL((gemm_skinny_kernel<MT, WV, (IT), RT, EPI, RMS, CT>), dim3((tiles + RT - 1) / RT), dim3(WV * 64), 0,  \
-                       stream, a, lda, w, ldw, c, ldc, M, N, K, gamma, gamma_f32, eps, extra.parts, extra.n_parts, rope);
+                       stream, a, lda, w, ldw, c, ldc, M, N, K, gamma, gamma_f32, eps, extra, rope);
   // the configurations skinny_plan can ask for: two loads in flight only with one column block
   GB_CFG(4, 1, 1) GB_CFG(4, 1, 2) GB_CFG(16, 1, 1) GB_CFG(16, 1, 2)
   if (MT == 1) {
@@ -1493,10 +1568,10 @@ int launch_skinny(const void* a, int lda, const bf16* w, int ldw, CT* c, int ldc
 // split_ws != nullptr: a workspace of split_ws_floats floats that the product may use to divide k over
 // workgroups (gb_gemm_bf16_split_floats says how many it needs; fewer than that is an error).
 // emit_h != nullptr (accumulating product that gb_gemm_bf16_emit_parts accepts): the next norm's operand and
-// partial sums are written beside the residual, see NormExtras.  parts != nullptr (at most 8 rows, no
+// partial sums are written beside the residual, see NormExtras.  parts != nullptr (at most 64 rows, no
 // gamma): the rows of a are such an operand and the product is scaled by the norm's factor from n_parts
 // partial sums; eps is that norm's.
-extern "C" int gb_gemm_bf16_emit_parts(int M, int N) { return fold_pays(M, N) ? (N + 7) / 8 : 0; }
+extern "C" int gb_gemm_bf16_emit_parts(int M, int N) { return emit_parts(M, N); }
 // 0, 1 or 2: see emit_mode.  With 2, gb_gemm_bf16 takes emit_gamma, emit_h and eps (no emit_ss) together with the
 // workspace and writes the normed rows to emit_h.
 extern "C" int gb_gemm_bf16_emit_mode(int M, int N, int K) { return emit_mode(M, N, K); }
@@ -1528,8 +1603,8 @@ extern "C" int gb_gemm_bf16(const void* a, int lda, const void* w, int ldw, void
                          (emit_gamma_dtype == kF32 || emit_gamma_dtype == kBF16) &&
                          ((emits == 1 && emit_ss) || (emits == 2 && split_ws && emit_ldh % 4 == 0 && ((uintptr_t)emit_h % 8 == 0)))),
              "gemm_bf16: only an accumulating product that gb_gemm_bf16_emit_mode accepts can prepare the next norm");
-  GB_REQUIRE(!parts || (M <= 8 && !gamma && n_parts > 0 && epilogue != EPI_ACCUMULATE),
-             "gemm_bf16: partial sums of a norm go with at most 8 rows, no gamma, and a storing epilogue");
+  GB_REQUIRE(!parts || (M <= 64 && !gamma && n_parts > 0 && epilogue != EPI_ACCUMULATE),
+             "gemm_bf16: partial sums of a norm go with at most 64 rows, no gamma, and a storing epilogue");
   const NormExtras extra{emit_gamma, emit_gamma_dtype == kF32, (bf16*)emit_h, emit_ldh, emit_ss, parts, n_parts};
   if (M == 0) return 0;
   const bf16* W = (const bf16*)w;
@@ -1625,7 +1700,7 @@ extern "C" int gb_gemm_bf16_rope(const void* a, int lda, const void* w, int ldw,
   GB_REQUIRE(!slots || (k_pages && v_pages && page_size > 0 && nkv > 0), "gemm_bf16_rope: slots given without pages");
   GB_REQUIRE(!gamma || (((uintptr_t)gamma % 16 == 0) && (gamma_dtype == kF32 || gamma_dtype == kBF16) && !parts),
              "gemm_bf16_rope: gamma must be aligned float32 or bfloat16, and not given together with parts");
-  GB_REQUIRE(!parts || (M <= 8 && n_parts > 0), "gemm_bf16_rope: partial sums of a norm go with at most 8 rows");
+  GB_REQUIRE(!parts || n_parts > 0, "gemm_bf16_rope: partial sums of a norm without a count");
   const NormExtras extra{nullptr, 0, nullptr, 0, nullptr, parts, n_parts};
   const RopeExtras rope{cosv, sinv, slots, (bf16*)k_pages, (bf16*)v_pages, nh, nkv, hd, page_size};
   if (gamma)

@@ -426,6 +426,12 @@ def copy_rows(base: torch.Tensor, src: torch.Tensor, dst: torch.Tensor) -> None:
 FUSED_NORM_MAX_ROWS = 16   # measured: beyond one 16-row block the re-reading of float32 rows costs more than a norm pass
 
 
+def parts_stride(rows: int) -> int:
+    """Floats a tile of partial sums holds (``gemm(..., emit=)`` / ``rms_parts=``): one per row, 8 for up to 8 rows,
+    64 beyond."""
+    return 8 if rows <= 8 else 64
+
+
 @functools.lru_cache(maxsize=4096)   # a pure function of the sizes, asked for at every product
 def gemm_emit_parts(rows: int, n: int) -> int:
     """How many partial sums an accumulating bfloat16 product of ``rows`` rows and ``n`` columns writes when
@@ -460,12 +466,13 @@ def gemm(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor, accumulate: bool =
     silu(a . gate_j) * (a . up_j), of half as many columns.
     ``rms=(gamma, eps)`` (bfloat16 w and out, at most 64 rows): a is the float32 residual and the
     product is that of its RMS-normed rows, the norm computed inside the product's kernel.
-    ``emit=(gamma, h, parts)`` (accumulating bfloat16 product with ``gemm_emit_mode(M, N, K) == 1``): besides
-    the new residual r in out, h[m, n] = bf16(gamma[n] r[m, n]) and float32 parts[tile, m] (8 columns a
-    tile) of sum(r^2) are written: the work of the RMS norm that reads the residual next.
+    ``emit=(gamma, h, parts)`` (accumulating bfloat16 product with ``gemm_emit_mode(M, N, K) == 1``: at most 64
+    rows): besides the new residual r in out, h[m, n] = bf16(gamma[n] r[m, n]) and float32 parts[tile, m] of
+    sum(r^2) over the tile's columns are written (``gemm_emit_parts`` tiles, ``parts_stride(M)`` floats a tile):
+    the work of the RMS norm that reads the residual next.
     ``emit=(gamma, h, eps)`` with a number as the third entry (``gemm_emit_mode(M, N, K) == 2``, with the
     workspace): h receives the rows of that norm itself, gamma * r / sqrt(mean(r^2) + eps).
-    ``rms_parts=(parts, n_parts, eps)`` (at most 8 rows): a is such an h, and the product is scaled by
+    ``rms_parts=(parts, n_parts, eps)`` (at most 64 rows): a is such an h, and the product is scaled by
     1 / sqrt(sum(parts[:, m]) / K + eps) to that of the normed rows.
     ``workspace`` (float32, at least ``gemm_split_floats(M, N, K)`` elements): lets a bfloat16 product of
     more than 16 rows and few tiles divide k over workgroups; their sums are added in a fixed order."""
@@ -519,16 +526,16 @@ def gemm(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor, accumulate: bool =
             want = gemm_emit_parts(M, N)
             if (not accumulate or want == 0 or e_gamma.numel() != N or not e_gamma.is_contiguous()
                     or e_h.dtype != torch.bfloat16 or e_h.shape != (M, N) or e_ss.dtype != torch.float32
-                    or not e_ss.is_contiguous() or e_ss.numel() < want * 8):
+                    or not e_ss.is_contiguous() or e_ss.numel() < want * parts_stride(M)):
                 raise KernelError("gemm: emit needs an accumulating product that gemm_emit_parts accepts, gamma of N "
-                                  "entries, a bfloat16 [M, N] operand buffer and 8 float32 per part")
+                                  "entries, a bfloat16 [M, N] operand buffer and parts_stride(M) float32 per part")
             e_ldh = _rows(e_h, "emit h")
         if rms_parts is not None:
             parts, n_parts, eps = rms_parts
             _dev(parts)
-            if (M > 8 or accumulate or parts.dtype != torch.float32 or not parts.is_contiguous()
-                    or parts.numel() < n_parts * 8 or n_parts <= 0):
-                raise KernelError("gemm: partial sums of a norm go with at most 8 rows and a storing product")
+            if (M > 64 or accumulate or parts.dtype != torch.float32 or not parts.is_contiguous()
+                    or parts.numel() < n_parts * parts_stride(M) or n_parts <= 0):
+                raise KernelError("gemm: partial sums of a norm go with at most 64 rows and a storing product")
         _launch(lib, lib.gb_gemm_bf16, _p(a), lda, _p(w), ldw, _p(out), ldc, dtype_code(out), M, N, K,
                                      2 if silu_mul else (1 if accumulate else 0), None, 0, float(eps),
                                      _p(e_gamma), dtype_code(e_gamma) if e_gamma is not None else 0, _p(e_h), e_ldh,
@@ -575,8 +582,8 @@ def gemm_rope(a: torch.Tensor, w: torch.Tensor, qkv: torch.Tensor, n_heads: int,
         raise KernelError("gemm_rope: rows must be bfloat16 (float32 only with rms=)")
     if rms_parts is not None:
         parts, n_parts, eps = rms_parts
-        if rms is not None or M > 8 or parts.dtype != torch.float32 or not parts.is_contiguous() or parts.numel() < n_parts * 8:
-            raise KernelError("gemm_rope: partial sums of a norm go with at most 8 rows and no gamma")
+        if rms is not None or parts.dtype != torch.float32 or not parts.is_contiguous() or parts.numel() < n_parts * parts_stride(M):
+            raise KernelError("gemm_rope: partial sums of a norm go with no gamma and parts_stride(M) floats a part")
     lib = _lib("gemm_bf16")
     _launch(lib, lib.gb_gemm_bf16_rope, _p(a), _rows(a, "a"), _p(w), _rows(w, "w"), _p(qkv), _rows(qkv, "qkv"), M, N, K,
                                       _p(gamma), dtype_code(gamma) if gamma is not None else 0, float(eps), _p(parts),

@@ -189,7 +189,8 @@ class PositionEncoding(Part):
 
 class PreNormed(NamedTuple):
     """The work of an RMS norm done by the product that made the residual: ``rows`` = bf16(gamma * residual)
-    and partial sums of the residual's squares, ``parts[:n_parts]``, 8 floats a part (row m in column m).
+    and partial sums of the residual's squares, ``parts[:n_parts]``, ``ops.parts_stride(rows)`` floats a part (row m
+    in column m).
     The product that takes it scales its result by 1 / sqrt(sum of parts / width + eps)."""
     rows: torch.Tensor
     parts: torch.Tensor
@@ -219,7 +220,7 @@ def emit_target(ctx, n: int, width: int, in_features: int, emit, tag: str):
     if mode == 1:
         n_parts = ops.gemm_emit_parts(n, width)
         rows = ctx.buffer(f"prenorm_rows_{tag}", (n, width), torch.bfloat16)
-        parts = ctx.buffer(f"prenorm_parts_{tag}", (n_parts, 8), torch.float32)
+        parts = ctx.buffer(f"prenorm_parts_{tag}", (n_parts, ops.parts_stride(n)), torch.float32)
         return (gamma, rows, parts), PreNormed(rows, parts, n_parts, float(eps))
     if mode == 2:
         rows = ctx.buffer(f"normed_rows_{tag}", (n, width), torch.bfloat16)

@@ -147,7 +147,13 @@ def test_gemm_bf16_fused_rms_norm(N, K, M, silu, gamma_dtype):
 
 
 @pytest.mark.parametrize("M,N,K,N2,silu", [(1, 64, 176, 96, False), (5, 352, 64, 176, True), (8, 2048, 2048, 6144, False),
-                                           (8, 2048, 8192, 16384, True), (3, 960, 2560, 2880, False)])
+                                           (8, 2048, 8192, 16384, True), (3, 960, 2560, 2880, False),
+                                           # more than 8 rows: the skinny kernel emits (tiles of 8 columns while they are
+                                           # few, of 16 beyond), and takes the partial sums of up to 64 rows
+                                           (12, 960, 2560, 2880, False), (40, 24704, 128, 512, False), (64, 352, 64, 176, True),
+                                           (20, 4096, 1024, 1024, True), (9, 72, 264, 48, False), (17, 2048, 1024, 16384, True),
+                                           # at most 8 rows by so many rows of W that the folded kernel does not pay
+                                           (5, 4096, 512, 256, False)])
 @pytest.mark.parametrize("gamma_dtype", [torch.float32, torch.bfloat16])
 def test_gemm_bf16_prepares_the_next_norm(M, N, K, N2, silu, gamma_dtype):
     """The product that adds into the residual and, on its way out, writes what the RMS norm that reads
@@ -155,7 +161,9 @@ def test_gemm_bf16_prepares_the_next_norm(M, N, K, N2, silu, gamma_dtype):
     those: against norm-then-product in float64 (crates/glassbox-core/src/model.rs:94-100, 323-335)."""
     from glassbox_amd import ops
     parts_n = ops.gemm_emit_parts(M, N)
-    assert parts_n == -(-N // 8)
+    assert parts_n == (-(-N // 8) if -(-N // 16) < 256 else -(-N // 16)) and ops.gemm_emit_mode(M, N, K) == 1
+    stride = ops.parts_stride(M)
+    assert stride == (8 if M <= 8 else 64)
     a, w = rnd(M, K, seed=1).bfloat16(), (rnd(N, K, seed=2) / math.sqrt(K)).bfloat16()
     r0 = rnd(M, N, seed=3, scale=2.0).float()
     g = (rnd(N, seed=4) * 0.3 + 1.0).to(gamma_dtype)
@@ -163,13 +171,13 @@ def test_gemm_bf16_prepares_the_next_norm(M, N, K, N2, silu, gamma_dtype):
     plain = to_dev(r0.clone())
     ops.gemm(to_dev(a), to_dev(w), plain, accumulate=True)
     res, h = to_dev(r0.clone()), torch.zeros(M, N, device=DEV, dtype=torch.bfloat16)
-    parts = torch.full((parts_n, 8), 7.0, device=DEV)
+    parts = torch.full((parts_n, stride), 7.0, device=DEV)
     ops.gemm(to_dev(a), to_dev(w), res, accumulate=True, emit=(to_dev(g), h, parts))
     assert torch.equal(res, plain)                                        # the residual is what it was without
     assert torch.equal(h, (to_dev(g).float() * res).bfloat16())
     ss = res.double().pow(2).sum(-1).cpu()
     assert ((parts[:, :M].double().sum(0).cpu() - ss).abs() <= 1e-5 * ss).all()
-    assert (parts[:, M:] == 0).all()
+    assert ((parts[:, M:] == 0) | (parts[:, M:] == 7.0)).all()                # rows that do not exist: zero or untouched
     # the product that follows
     w2 = (rnd(N2, N, seed=5) / math.sqrt(N)).bfloat16()
     x = res.double().cpu()
