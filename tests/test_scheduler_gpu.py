@@ -104,7 +104,7 @@ def test_preemption_and_shared_beginnings_at_the_level_of_logits(model_dirs, bf1
 
 
 def test_seeded_temperature_replies_are_the_plain_samplers(model_dirs):
-    """The second tiny configuration as BASELINE names it: prompts of 1, 9, 40 and 70 tokens, portions of sixteen,
+    """The second tiny configuration with the workload it is quoted with: prompts of 1, 9, 40 and 70 tokens, portions of sixteen,
     24 tokens at temperature 0.8, seeded.  In 32-bit every token is the one the plain sampler draws from the plain
     implementation's logits with the same generator (crates/glassbox-core/src/sampler.rs:97-164); the comparison
     of a request ends where a draw falls within 1e-5 of a boundary between two tokens."""
