@@ -313,13 +313,12 @@ __global__ void rope_store_kernel(T* __restrict__ qkv, int row_stride, const flo
 // The same for head sizes that are a multiple of 16, bfloat16, with 16-byte aligned rows: a lane takes a whole
 // piece of 8 dimensions and its partner piece hd/2 further on as 16-byte words, so that a key's pieces go to
 // their places in the page (key_piece()) in one store each.  hd / 16 lanes a head.
-__global__ void rope_store_pieces_kernel(bf16* __restrict__ qkv, int row_stride, const float* __restrict__ cosv,
-                                         const float* __restrict__ sinv, const int32_t* __restrict__ slots,
-                                         bf16* __restrict__ k_pages, bf16* __restrict__ v_pages, int nh, int nkv, int hd,
-                                         int page_size, int rotate, int v_rows) {
-  const int t = blockIdx.x;
+__device__ __forceinline__ void rope_store_pieces(int t, int idx, bf16* __restrict__ qkv, int row_stride,
+                                                  const float* __restrict__ cosv, const float* __restrict__ sinv,
+                                                  const int32_t* __restrict__ slots, bf16* __restrict__ k_pages,
+                                                  bf16* __restrict__ v_pages, int nh, int nkv, int hd, int page_size,
+                                                  int rotate, int v_rows) {
   const int half = hd / 2, lanes = half / 8;  // lanes a head
-  const int idx = blockIdx.y * blockDim.x + threadIdx.x;
   const int unit = idx / lanes, j = (idx % lanes) * 8;
   const int units = nh + nkv + ((slots && t < v_rows) ? nkv : 0);  // rows from v_rows on: values are stored by tiles
   if (unit >= units) return;
@@ -359,21 +358,26 @@ __global__ void rope_store_pieces_kernel(bf16* __restrict__ qkv, int row_stride,
   }
 }
 
+__global__ void rope_store_pieces_kernel(bf16* __restrict__ qkv, int row_stride, const float* __restrict__ cosv,
+                                         const float* __restrict__ sinv, const int32_t* __restrict__ slots,
+                                         bf16* __restrict__ k_pages, bf16* __restrict__ v_pages, int nh, int nkv, int hd,
+                                         int page_size, int rotate, int v_rows) {
+  rope_store_pieces(blockIdx.x, blockIdx.y * blockDim.x + threadIdx.x, qkv, row_stride, cosv, sinv, slots, k_pages, v_pages, nh,
+                    nkv, hd, page_size, rotate, v_rows);
+}
+
 // Values of prompt portions, sixteen positions at a time: the transposed page holds the sixteen slots
 // of one dimension side by side, so a tile of 16 tokens x hd is turned in LDS and written as whole
 // 16-byte words instead of two bytes at a time.  grid (groups of 16 positions, kv heads, requests
 // from seq_base on); request s has q_len[s] rows from row q_start[s] on, the first at position pos0[s].
 template <typename T>
-__global__ void store_values_kernel(const T* __restrict__ qkv, int row_stride, const int32_t* __restrict__ slots,
-                                    T* __restrict__ v_pages, const int32_t* __restrict__ q_start,
-                                    const int32_t* __restrict__ q_len, const int32_t* __restrict__ pos0, int seq_base,
-                                    int nh, int nkv, int hd, int page_size) {
-  extern __shared__ unsigned char tile_bytes[];
-  T* tile = reinterpret_cast<T*>(tile_bytes);  // [16][hd + 2]
-  const int ld = hd + 2;
-  const int seq = seq_base + blockIdx.z, kvh = blockIdx.y;
+__device__ __forceinline__ void store_values_tile(int group, int kvh, int seq, T* tile, const T* __restrict__ qkv,
+                                                  int row_stride, const int32_t* __restrict__ slots, T* __restrict__ v_pages,
+                                                  const int32_t* __restrict__ q_start, const int32_t* __restrict__ q_len,
+                                                  const int32_t* __restrict__ pos0, int nh, int nkv, int hd, int page_size) {
+  const int ld = hd + 2;  // tile: [16][hd + 2]
   const int first = pos0[seq], n = q_len[seq];
-  const int p_lo = (first / 16 + blockIdx.x) * 16;  // the group's first position
+  const int p_lo = (first / 16 + group) * 16;  // the group's first position
   const int j_lo = p_lo - first;                     // its token index in the portion (may be negative)
   if (j_lo >= n) return;
   const int row0 = q_start[seq];
@@ -418,6 +422,37 @@ __global__ void store_values_kernel(const T* __restrict__ qkv, int row_stride, c
   }
 }
 
+template <typename T>
+__global__ void store_values_kernel(const T* __restrict__ qkv, int row_stride, const int32_t* __restrict__ slots,
+                                    T* __restrict__ v_pages, const int32_t* __restrict__ q_start,
+                                    const int32_t* __restrict__ q_len, const int32_t* __restrict__ pos0, int seq_base,
+                                    int nh, int nkv, int hd, int page_size) {
+  extern __shared__ unsigned char tile_bytes[];
+  store_values_tile<T>(blockIdx.x, blockIdx.y, seq_base + blockIdx.z, reinterpret_cast<T*>(tile_bytes), qkv, row_stride, slots,
+                       v_pages, q_start, q_len, pos0, nh, nkv, hd, page_size);
+}
+
+// Both at once for bfloat16 steps with prompt portions: the first `rope_blocks` workgroups rotate and write keys
+// (and the values of single-token rows), the rest turn the portions' values tile by tile.  The two have nothing to
+// wait for in each other, and one launch costs a step of some hundred rows less than two.
+__global__ void rope_and_values_kernel(bf16* __restrict__ qkv, int row_stride, const float* __restrict__ cosv,
+                                       const float* __restrict__ sinv, const int32_t* __restrict__ slots,
+                                       bf16* __restrict__ k_pages, bf16* __restrict__ v_pages, int nh, int nkv, int hd,
+                                       int page_size, int rotate, int v_rows, int rope_blocks, int rope_y,
+                                       const int32_t* __restrict__ q_start, const int32_t* __restrict__ q_len,
+                                       const int32_t* __restrict__ pos0, int seq_base, int groups) {
+  extern __shared__ unsigned char tile_bytes[];
+  const int b = blockIdx.x;
+  if (b < rope_blocks) {
+    rope_store_pieces(b / rope_y, (b % rope_y) * blockDim.x + threadIdx.x, qkv, row_stride, cosv, sinv, slots, k_pages, v_pages,
+                      nh, nkv, hd, page_size, rotate, v_rows);
+    return;
+  }
+  const int v = b - rope_blocks;
+  store_values_tile<bf16>(v % groups, v / groups % nkv, seq_base + v / (groups * nkv), reinterpret_cast<bf16*>(tile_bytes), qkv,
+                          row_stride, slots, v_pages, q_start, q_len, pos0, nh, nkv, hd, page_size);
+}
+
 // Rows v_rows .. n-1 are prompt portions described by q_start, q_len and pos0 of requests seq_base ..
 // seq_base + n_seqs - 1 (the longest has max_q_len rows): their values are stored tile by tile.  With
 // v_rows == n there are none.
@@ -435,6 +470,21 @@ extern "C" int gb_rope_store(void* qkv, int dtype, int row_stride, const float* 
   const bool tiles = slots && v_rows < n && n_seqs > 0 && q_start && q_len && pos0 && page_size % 16 == 0 && hd % 8 == 0 &&
                      (uintptr_t)v_pages % 16 == 0 && (uintptr_t)qkv % 16 == 0 && row_stride % 8 == 0;
   if (!tiles) v_rows = n;
+  const bool pairs_of_two = hd % 4 == 0 && row_stride % 2 == 0 && (uintptr_t)qkv % 8 == 0 && (uintptr_t)k_pages % 8 == 0 &&
+                            (!rotate || ((uintptr_t)cosv % 8 == 0 && (uintptr_t)sinv % 8 == 0));
+  const bool pieces = dtype == kBF16 && hd % 16 == 0 && row_stride % 8 == 0 && (uintptr_t)qkv % 16 == 0 &&
+                      (uintptr_t)k_pages % 16 == 0 && (!rotate || ((uintptr_t)cosv % 16 == 0 && (uintptr_t)sinv % 16 == 0));
+  if (tiles && pieces) {  // one launch for both
+    const int units = nh + 2 * nkv, lanes = units * (hd / 16);
+    const int threads = lanes >= 256 ? 256 : 64;
+    const int rope_y = (lanes + threads - 1) / threads, groups = (max_q_len + 15) / 16 + 1;
+    const long long blocks = (long long)n * rope_y + (long long)groups * nkv * n_seqs;
+    GB_REQUIRE(blocks < (1ll << 31), "rope_store: %lld workgroups are too many for one launch", blocks);
+    hipLaunchKernelGGL(rope_and_values_kernel, dim3((unsigned)blocks), dim3(threads), 16 * (hd + 2) * sizeof(bf16), stream,
+                       (bf16*)qkv, row_stride, cosv, sinv, slots, (bf16*)k_pages, (bf16*)v_pages, nh, nkv, hd, page_size, rotate,
+                       v_rows, n * rope_y, rope_y, q_start, q_len, pos0, seq_base, groups);
+    return launched("rope_store (with the portions' values)");
+  }
   if (tiles) {
     const dim3 grid((max_q_len + 15) / 16 + 1, nkv, n_seqs);
     GB_REQUIRE(nkv <= 65535 && n_seqs <= 65535, "rope_store: too many kv heads or requests for one launch");
@@ -451,10 +501,6 @@ extern "C" int gb_rope_store(void* qkv, int dtype, int row_stride, const float* 
       return fail("rope_store: unknown dtype %d", dtype);
     if (int rc = launched("rope_store (values)")) return rc;
   }
-  const bool pairs_of_two = hd % 4 == 0 && row_stride % 2 == 0 && (uintptr_t)qkv % 8 == 0 && (uintptr_t)k_pages % 8 == 0 &&
-                            (!rotate || ((uintptr_t)cosv % 8 == 0 && (uintptr_t)sinv % 8 == 0));
-  const bool pieces = dtype == kBF16 && hd % 16 == 0 && row_stride % 8 == 0 && (uintptr_t)qkv % 16 == 0 &&
-                      (uintptr_t)k_pages % 16 == 0 && (!rotate || ((uintptr_t)cosv % 16 == 0 && (uintptr_t)sinv % 16 == 0));
   if (pieces) {
     const int units = nh + nkv + (slots ? nkv : 0), lanes = units * (hd / 16);
     const int threads = lanes >= 256 ? 256 : 64;
