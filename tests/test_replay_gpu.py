@@ -358,3 +358,37 @@ def test_random_configurations(tmp_path, seed):
                                  f"max abs error {bad[1]:.3e}, allowed {tol:.3e}")
         eng.cache.check_invariants()
         assert eng.cache.used_pages() == 0
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("name,count", [("B", 12), ("E", 20), ("D", 40)])
+def test_many_requests_decode_together(model_dirs, bf16_bound, name, count, dtype):
+    """Twelve, twenty and forty requests whose last 24 tokens are decoded in the same steps: steps of that many single
+    tokens (in bfloat16 replayed from graphs, with filler rows up to the graph's size; the products of 9 to 64 rows
+    prepare each other's norms), every position against the plain implementation.  Requests end at different steps, so
+    the batch shrinks through every size on the way."""
+    from glassbox_amd.engine import Engine
+    folder = model_dirs.get(name)
+    vocab = helpers.TINY[name]["vocab_size"]
+    requests = {f"r{i}": helpers.random_tokens(vocab, 30 + (7 * i) % 41, seed=500 + i) for i in range(count)}
+    tail = 24
+    steps = [{"entries": [(r, t[:len(t) - tail], list(range(len(t) - tail)))], "end": []} for r, t in requests.items()]
+    longest = max(len(t) for t in requests.values())
+    for k in range(tail + longest):
+        entries, end = [], []
+        for i, (r, t) in enumerate(requests.items()):
+            at = len(t) - tail + k - i % 5          # requests start decoding up to four steps apart
+            if len(t) - tail <= at < len(t) and k >= i % 5:
+                entries.append((r, [t[at]], [0]))
+                if at == len(t) - 1:
+                    end.append(r)
+        if entries:
+            steps.append({"entries": entries, "end": end})
+    eng = Engine(folder, dtype=dtype, max_tokens=count * 128, max_seqs=count)
+    got = helpers.replay(eng, steps)
+    assert max(len(s["entries"]) for s in steps) == count
+    if eng.decode_graphs is not None:
+        assert eng.decode_graphs.replays > 0
+    check(folder, requests, got, dtype, f"{count} requests decoding together", tolerance(bf16_bound, folder, requests, dtype))
+    eng.cache.check_invariants()
+    assert eng.cache.used_pages() == 0
