@@ -139,3 +139,26 @@ def test_a_layers_tensors_come_in_one_order_and_include_cache_and_the_next_norm(
                                                                     cache.state.data_ptr()]
     gamma = torch.ones(32)
     assert layer_tape.tensors_of((gamma, 1e-5))[0] is gamma and layer_tape.tensors_of(None) == []
+
+
+def test_every_launch_a_layer_can_make_has_a_taped_form():
+    """The libraries a layer's parts launch from (all but the sampler's) give each entry point that takes a stream a
+    second form that takes its arguments in slots; the bindings pack a launch of it into an entry of the size the
+    native runner reads."""
+    from glassbox_amd import build
+    host = build.load("host")
+    assert host.gbh_tape_entry_bytes() == 24 + 8 * host.gbh_tape_max_args()
+    for libname, sigs in ops._SIGS.items():
+        if libname == "sampling":
+            continue
+        lib = build.load(libname)
+        for fn, argtypes in sigs.items():
+            if argtypes[-1] is not C.c_void_p or len(argtypes) < 4:     # a question about sizes, not a launch
+                continue
+            entry = getattr(lib, fn)
+            entry.argtypes = argtypes
+            how = ops._tape_entry(lib, entry)
+            assert how is not False, f"{libname}: {fn} has no taped form"
+            st, address, mask, n = how
+            assert st.size == host.gbh_tape_entry_bytes() and address and n == len(argtypes)
+            assert all(bool(mask >> i & 1) == (t is C.c_void_p) for i, t in enumerate(argtypes))
