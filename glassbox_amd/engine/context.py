@@ -25,6 +25,9 @@ class Workspace:
         self._views: Dict[tuple, torch.Tensor] = {}
         #: counts the times a buffer was replaced by a larger one: a captured graph holds the old addresses
         self.epoch = 0
+        #: what ``parts.tape`` keeps from step to step of each entry of the model's schedule (the layer's tensors as
+        #: address ranges): it lives here, with the engine's buffers and pages, and goes when they go
+        self.tape_sites: dict = {}
 
     def buffer(self, name: str, shape: Sequence[int], dtype: torch.dtype) -> torch.Tensor:
         vkey = (name, dtype, tuple(shape))

@@ -43,8 +43,8 @@ class DecoderModel(Part):
         self.vocab_size = embedding.vocab
         self.width = embedding.width
         self._check_schedule()
-        self._tape_sites: dict = {}                    # what parts.tape keeps of each schedule entry
-        self._taped: Optional[List[bool]] = None       # which blocks allow it
+        self._taped: Optional[List[bool]] = None       # which blocks let their launches be recorded (parts.tape)
+        self._loads = 0                                # times the weights were loaded: recorded tensors are theirs
 
     # structure ------------------------------------------------------------------
     def children(self) -> Dict[str, Part]:
@@ -89,7 +89,9 @@ class DecoderModel(Part):
         pre = None   # what the block before prepared of this block's first norm
         if self._taped is None:
             self._taped = [b.all_taped() for b in self.blocks]
-        tapes = LayerTapes(ctx, self._tape_sites) if getattr(ctx, "layer_tapes", False) and any(self._taped) else None
+        tapes = None
+        if getattr(ctx, "layer_tapes", False) and any(self._taped):
+            tapes = LayerTapes(ctx, ctx.workspace.tape_sites, self._loads)
         for i, call in enumerate(self.schedule):
             if call.cache is not None:
                 cache = caches[call.cache]
@@ -117,7 +119,7 @@ class DecoderModel(Part):
 
     def load_tree(self, tensors, prefix: str = "") -> None:
         super().load_tree(tensors, prefix)
-        self._tape_sites.clear()   # they hold the tensors that were loaded before
+        self._loads += 1   # what engines keep of the layers' tensors (parts.tape) is of the weights before
 
     def streamed_matrices(self) -> List[torch.Tensor]:
         """Every tensor a step reads whole, once each: those of the scheduled blocks (a block named twice, or a

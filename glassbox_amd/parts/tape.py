@@ -54,7 +54,7 @@ def signature(part: Part, _seen: Optional[set] = None) -> tuple:
         return ("again", type(part).__qualname__)
     seen.add(id(part))
     items: list = [type(part).__module__, type(part).__qualname__]
-    for name, v in vars(part).items():
+    for name, v in getattr(part, "__dict__", {}).items():
         if v is None or name.startswith("_"):
             continue   # nothing set, or the part's own working state (a tensor made on first use)
         if isinstance(v, Part):
@@ -83,7 +83,7 @@ def tensors_of(obj, _seen: Optional[set] = None) -> List[torch.Tensor]:
         if id(obj) in seen:
             return out
         seen.add(id(obj))
-        for v in vars(obj).values():
+        for v in getattr(obj, "__dict__", {}).values():
             if isinstance(v, (torch.Tensor, Part, LayerCache, tuple, list)):
                 out.extend(tensors_of(v, seen))
     return out
@@ -129,8 +129,8 @@ class _Site:
     """What stays of a schedule entry from step to step: its block's signature and, while the block is called with
     the same cache layer and the same norm to prepare, the layer's tensors and the part of the key they make."""
 
-    def __init__(self, block: Part):
-        self.block = block
+    def __init__(self, block: Part, loads: int):
+        self.block, self.loads = block, loads
         sig = signature(block)
         self.kind = _signature_numbers.setdefault(sig, len(_signature_numbers))   # a number hashes faster than the tuple
         self.cache: Optional[LayerCache] = None
@@ -163,10 +163,11 @@ class _Record:
 
 
 class LayerTapes:
-    """The recorded layers of one step.  ``sites`` lives with the model (one entry per schedule entry)."""
+    """The recorded layers of one step.  ``sites`` lives with the engine's workspace (one entry per schedule entry);
+    ``loads`` counts the times the model's weights were loaded: a site of another count holds tensors that are gone."""
 
-    def __init__(self, ctx, sites: Dict[int, _Site]):
-        self.ctx, self.sites = ctx, sites
+    def __init__(self, ctx, sites: Dict[int, _Site], loads: int = 0):
+        self.ctx, self.sites, self.loads = ctx, sites, loads
         self.records: Dict[tuple, _Record] = {}
         self._x = self._x_key = None
         self._pre = self._pre_key = None
@@ -175,8 +176,8 @@ class LayerTapes:
         """``block.forward(ctx, x, cache, **kwargs)``, by replay if a layer of its kind has been recorded in this step."""
         ctx = self.ctx
         site = self.sites.get(index)
-        if site is None or site.block is not block:
-            site = self.sites[index] = _Site(block)
+        if site is None or site.block is not block or site.loads != self.loads:
+            site = self.sites[index] = _Site(block, self.loads)
         site.bind(cache, kwargs.get("emit"))
         pre = kwargs.get("pre")
         if x is not self._x:

@@ -139,3 +139,22 @@ def test_what_is_done_once_a_step_is_not_replayed(model_dirs, monkeypatch, dtype
     assert len(replayed) >= 3 * 3, "layers were not replayed"
     assert all("gb_rope_table" not in names for names in replayed)
     assert all(any(n.startswith("gb_gemm") for n in names) for names in replayed)
+
+
+def test_weights_loaded_again_under_a_live_engine_are_the_ones_replayed(model_dirs):
+    """What the engine keeps of each layer's tensors between steps is of one loading of the weights: after another
+    checkpoint has been loaded into the same model, replayed layers must run on the new tensors."""
+    import os
+    from glassbox_amd.engine import Engine
+    from glassbox_amd.weights import load_weights
+    first, second = model_dirs.get("E", seed=0), model_dirs.get("E", seed=7)
+    toks = helpers.random_tokens(helpers.TINY["E"]["vocab_size"], 50, seed=3)
+    eng = Engine(first, dtype="float32", max_tokens=256, max_seqs=2, graph_decode=False)
+    got = eng.step([("a", toks, [49])]).cpu().numpy()[0]
+    assert np.abs(got - helpers.oracle(first, toks, "float32")[49]).max() <= helpers.TOL_F32
+    eng.end_request("a")
+    load_weights(eng.model, os.path.join(second, "model.safetensors"), torch.float32, eng.device)
+    got = eng.step([("b", toks, [49])]).cpu().numpy()[0]
+    want = helpers.oracle(second, toks, "float32")[49]
+    assert np.abs(got - want).max() <= helpers.TOL_F32
+    assert np.abs(want - helpers.oracle(first, toks, "float32")[49]).max() > 1e-2, "the two checkpoints must differ"
