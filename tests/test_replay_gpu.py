@@ -392,3 +392,23 @@ def test_many_requests_decode_together(model_dirs, bf16_bound, name, count, dtyp
     check(folder, requests, got, dtype, f"{count} requests decoding together", tolerance(bf16_bound, folder, requests, dtype))
     eng.cache.check_invariants()
     assert eng.cache.used_pages() == 0
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("name", ["B", "D"])
+def test_a_context_of_nine_thousand_tokens(model_dirs, bf16_bound, name, dtype):
+    """One request of 9,000 tokens: its prompt in portions of 2,048 (each attending to all the pages before it), a
+    portion of 100 tokens behind 7,844 (workgroups share a block pair's keys and a second pass adds their sums),
+    then 56 tokens one by one over 560 pages (the context in chunks, a pass that merges them; in bfloat16 from graphs):
+    every position against the plain implementation."""
+    from glassbox_amd.engine import Engine
+    folder = model_dirs.get(name)
+    toks = helpers.random_tokens(helpers.TINY[name]["vocab_size"], 9000, seed=77)
+    requests = {"long": toks}
+    cuts = [0, 2048, 4096, 6144, 7844, 7944, 8944]
+    steps = [{"entries": [("long", toks[a:b], list(range(b - a)))], "end": []} for a, b in zip(cuts, cuts[1:])]
+    steps += [{"entries": [("long", [toks[i]], [0])], "end": ["long"] if i == 8999 else []} for i in range(8944, 9000)]
+    eng = Engine(folder, dtype=dtype, max_tokens=9024, max_seqs=1)
+    got = helpers.replay(eng, steps)
+    check(folder, requests, got, dtype, "nine thousand tokens", tolerance(bf16_bound, folder, requests, dtype))
+    assert eng.cache.used_pages() == 0
