@@ -3,17 +3,22 @@
 // (crates/glassbox-core/src/kernels.rs:381,586).  Both operands are contiguous along k, which
 // is the layout MFMA operands want: every lane loads 8 consecutive k as one 16-byte word.
 //
-// Four kernels:
+// Five kernels:
 //  * tiled  (M > 64, prompt portions): a workgroup of 2x2 waves, each wave a block of 2x2 or 2x1
-//    v_mfma_f32_32x32x16_bf16 tiles (workgroup tile 128x128 or 128x64), operands staged through LDS in
-//    k-steps of 64 with two buffers; the SiLU-multiply of stacked gate/up rows can be its epilogue.
+//    v_mfma_f32_32x32x16_bf16 tiles (workgroup tile 128x128 or 128x64; 64 rows high where the taller tiles would be
+//    few), operands staged through LDS in k-steps of 64 with two buffers; the SiLU-multiply of stacked gate/up rows
+//    can be its epilogue.  Its workgroups can also divide k (split k: a second pass adds their sums in order).
+//  * stream (65 to 128 rows, the mixed steps of serving): 128 x 32 or 128 x 64 tiles, both operands through deep
+//    rings in LDS, W asked for by a wave of its own.
 //  * ring   (a thousand rows and more, enough 256x256 tiles to fill the chip): 2x4 waves, a wave 4x2 such
 //    tiles; operands go from memory straight into a ring of LDS buffers in k-steps of 32.
-//  * skinny (M <= 64, decoding): bound by reading W once.  A workgroup owns 16 or 32 rows of W; its
+//  * skinny (M <= 64, decoding): bound by reading W once.  A workgroup owns 16 or 32 rows of W (8 where the
+//    rows of W are few); its
 //    waves take interleaved 64-wide k blocks, stream W straight from memory into MFMA operands
 //    (v_mfma_f32_16x16x32_bf16, W as the A operand so that the 16 rows fill the tile) and combine
 //    through LDS in a fixed order; it can norm float32 rows on the way, apply the SiLU-multiply, or
-//    (the QKV product) rotate the heads and write the key/value cache.
+//    (the QKV product) rotate the heads and write the key/value cache, or prepare the next norm where it adds
+//    into the residual.
 //  * folded (M <= 8 and few rows of W): the skinny kernel with two k ranges side by side in a tile,
 //    so that a workgroup owns 8 rows of W and there are twice as many workgroups.
 // In all, every output cell is summed in an order fixed by (K, kernel) alone, not by M or by
