@@ -73,7 +73,18 @@ struct RopeExtras {
   bf16* k_pages;
   bf16* v_pages;
   int nh, nkv, hd, page_size;
+  int three_halves;  // the launch gives a workgroup a tile and a half (see three_halves_tile), not two tiles
 };
+
+// Tiles of the skinny kernel's rotating product, 8 pairs each, dealt a tile and a half to a workgroup: workgroup g
+// takes tile 3g/2 whole and the first four pairs of the next (g even), or the last four pairs of tile (3g - 1)/2 and
+// the next whole (g odd).  384 tiles (the 6,144 rows of a QKV product) then make 256 workgroups of equal work, one for
+// every compute unit, where two tiles each would make 192.  [lo, hi): the pairs of tile rt that are the workgroup's.
+__device__ __forceinline__ int three_halves_tile(int g, int rt, int* lo, int* hi) {
+  *lo = (g & 1) && rt == 0 ? 4 : 0;
+  *hi = !(g & 1) && rt == 1 ? 4 : 8;
+  return ((g & 1) ? (3 * g - 1) / 2 : 3 * g / 2) + rt;
+}
 
 template <typename CT> __device__ __forceinline__ void store_c(CT* c, float v, int accumulate);
 template <> __device__ __forceinline__ void store_c<float>(float* c, float v, int accumulate) { *c = accumulate ? *c + v : v; }
@@ -1131,7 +1142,8 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_skinny_kernel(const void* __r
   bool row_ok[RT];
 #pragma unroll
   for (int rt = 0; rt < RT; ++rt) {
-    const int tile = blockIdx.x * RT + rt;
+    int tile = blockIdx.x * RT + rt, pair_lo = 0, pair_hi = 8;
+    if (EPI == EPI_ROPE && RT == 2 && rope.three_halves) tile = three_halves_tile(blockIdx.x, rt, &pair_lo, &pair_hi);
     int row;
     if (EPI == EPI_SILU_MUL) {
       row = r < 8 ? tile * 8 + r : N / 2 + tile * 8 + (r - 8);
@@ -1145,6 +1157,7 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_skinny_kernel(const void* __r
       row = tile * 16 + r;
     }
     row_ok[rt] = EPI == EPI_SILU_MUL ? (tile * 8 + (r & 7) < N / 2) : HALF ? (r < 8 && row < N) : row < N;
+    if (EPI == EPI_ROPE) row_ok[rt] = row_ok[rt] && (r & 7) >= pair_lo && (r & 7) < pair_hi;
     wrow[rt] = w + (size_t)(row_ok[rt] ? row : 0) * ldw;
   }
 
@@ -1288,7 +1301,9 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_skinny_kernel(const void* __r
     const bool upper = nrow >= 8;
 #pragma unroll
     for (int rt = 0; rt < RT; ++rt) {
-      const int tile = blockIdx.x * RT + rt;
+      int tile = blockIdx.x * RT + rt, pair_lo = 0, pair_hi = 8;
+      if (RT == 2 && rope.three_halves) tile = three_halves_tile(blockIdx.x, rt, &pair_lo, &pair_hi);
+      if ((nrow & 7) < pair_lo || (nrow & 7) >= pair_hi) continue;
       const int head = tile / per_head, pair = (tile % per_head) * 8 + (nrow & 7);
       const int dim = upper ? half + pair : pair;
       if (head * rope.hd + dim >= N) continue;
@@ -1539,10 +1554,14 @@ int launch_skinny_mt(int tiles, const void* a, int lda, const bf16* w, int ldw, 
       return launched("gemm_bf16 (skinny, half tiles)");
     }
   }
+  // the rotating product with two tiles a workgroup: a tile and a half each where that divides evenly (three_halves_tile)
+  RopeExtras rp = rope;
+  rp.three_halves = (EPI == EPI_ROPE && rt == 2 && tiles % 3 == 0) ? 1 : 0;
+  const int groups = rp.three_halves ? 2 * tiles / 3 : (tiles + rt - 1) / rt;
 #define GB_CFG(WV, IT, RT)                                                                                                 \
   if (waves == WV && iters == (IT) && rt == RT)                                                                            \
-    hipLaunchKernelGGL((gemm_skinny_kernel<MT, WV, (IT), RT, EPI, RMS, CT>), dim3((tiles + RT - 1) / RT), dim3(WV * 64), 0,  \
-                       stream, a, lda, w, ldw, c, ldc, M, N, K, gamma, gamma_f32, eps, extra, rope);
+    hipLaunchKernelGGL((gemm_skinny_kernel<MT, WV, (IT), RT, EPI, RMS, CT>), dim3(groups), dim3(WV * 64), 0, stream, a, lda, \
+                       w, ldw, c, ldc, M, N, K, gamma, gamma_f32, eps, extra, rp);
   // the configurations skinny_plan can ask for: two loads in flight only with one column block
   GB_CFG(4, 1, 1) GB_CFG(4, 1, 2) GB_CFG(16, 1, 1) GB_CFG(16, 1, 2)
   if (MT == 1) {
@@ -1707,7 +1726,7 @@ extern "C" int gb_gemm_bf16_rope(const void* a, int lda, const void* w, int ldw,
              "gemm_bf16_rope: gamma must be aligned float32 or bfloat16, and not given together with parts");
   GB_REQUIRE(!parts || n_parts > 0, "gemm_bf16_rope: partial sums of a norm without a count");
   const NormExtras extra{nullptr, 0, nullptr, 0, nullptr, parts, n_parts};
-  const RopeExtras rope{cosv, sinv, slots, (bf16*)k_pages, (bf16*)v_pages, nh, nkv, hd, page_size};
+  const RopeExtras rope{cosv, sinv, slots, (bf16*)k_pages, (bf16*)v_pages, nh, nkv, hd, page_size, 0};
   if (gamma)
     return launch_skinny<EPI_ROPE, true, bf16>(a, lda, (const bf16*)w, ldw, (bf16*)c, ldc, M, N, K, gamma, gamma_dtype == kF32,
                                                eps, extra, stream, rope);

@@ -413,7 +413,9 @@ def test_rope_table_and_rotation(hd, theta):
 
 
 ROPE_PRODUCTS = [(1, 4, 2, 16, 64), (8, 3, 1, 32, 96), (5, 6, 2, 48, 80), (8, 32, 32, 64, 2048), (33, 8, 2, 128, 264),
-                 (64, 15, 5, 64, 960), (7, 4, 0, 32, 64)]
+                 (64, 15, 5, 64, 960), (7, 4, 0, 32, 64),
+                 # 432 and 400 tiles of 8 pairs: a tile and a half to a workgroup, and two tiles each
+                 (40, 50, 2, 128, 128), (20, 48, 1, 128, 192)]
 
 
 @pytest.mark.parametrize("nh,nkv,hd,page", [(4, 2, 16, 16), (32, 32, 64, 16), (5, 1, 48, 32), (8, 2, 128, 16), (3, 3, 80, 64)])
