@@ -1216,6 +1216,48 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_skinny_kernel(const void* __r
       }
     }
   }
+  // D[n, m]: lane l holds column m = l%16 and rows n = 4*(l/16) + e.  The first 256 threads own the
+  // cells of the tiles: thread tid owns cell (l = tid/4, e = tid%4) of every row tile and column block.
+  const int l = (tid % 256) / 4, e = tid % 4;
+  const int nrow = 4 * (l / 16) + e;  // row of the tile, 0..15
+  // What the owners will need from memory at the end (a cell's old value and the gamma of a norm to prepare; a
+  // row's cosine, sine and cache slot) is asked for here, before the waves meet, so that it arrives while they do.
+  constexpr int ROWS = HALF ? 8 : 16;  // rows of W a tile owns
+  const bool emits = EPI == EPI_ACCUMULATE && extra.emit_h != nullptr;
+  const bool empty = HALF && nrow >= 8;  // the lower half of a half tile
+  float old[RT][MT], emit_g[RT], cs[RT][MT], sn[RT][MT];
+  int slot[MT];
+  if (EPI == EPI_ACCUMULATE && tid < 256) {
+#pragma unroll
+    for (int rt = 0; rt < RT; ++rt) {
+      const int n = (blockIdx.x * RT + rt) * ROWS + nrow;
+      emit_g[rt] = 0.f;
+      if (emits && !empty && n < N)
+        emit_g[rt] = extra.emit_gamma_f32 ? ((const float*)extra.emit_gamma)[n] : (float)((const bf16*)extra.emit_gamma)[n];
+#pragma unroll
+      for (int t = 0; t < MT; ++t) {
+        const int m = t * 16 + l % 16;
+        old[rt][t] = (!empty && m < M && n < N) ? (float)c[(size_t)m * ldc + n] : 0.f;
+      }
+    }
+  }
+  constexpr bool ROPE_EARLY = MT * RT <= 4;  // beyond that the registers would not hold what is asked for early
+  if (EPI == EPI_ROPE && ROPE_EARLY && tid < 256) {
+#pragma unroll
+    for (int t = 0; t < MT; ++t) {
+      const int m = t * 16 + l % 16;
+      slot[t] = (rope.slots != nullptr && m < M) ? rope.slots[m] : 0;
+#pragma unroll
+      for (int rt = 0; rt < RT; ++rt) {
+        int tile = blockIdx.x * RT + rt, pair_lo = 0, pair_hi = 8;
+        if (RT == 2 && rope.three_halves) tile = three_halves_tile(blockIdx.x, rt, &pair_lo, &pair_hi);
+        const int pair = (tile % (rope.hd / 16)) * 8 + (nrow & 7);
+        const bool rotated = rope.cosv != nullptr && m < M && tile / (rope.hd / 16) < rope.nh + rope.nkv;
+        cs[rt][t] = rotated ? rope.cosv[(size_t)m * (rope.hd / 2) + pair] : 1.f;
+        sn[rt][t] = rotated ? rope.sinv[(size_t)m * (rope.hd / 2) + pair] : 0.f;
+      }
+    }
+  }
 #pragma unroll
   for (int rt = 0; rt < RT; ++rt)
 #pragma unroll
@@ -1229,9 +1271,6 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_skinny_kernel(const void* __r
   __syncthreads();
   if (tid >= 256) return;
 
-  // D[n, m]: lane l holds column m = l%16 and rows n = 4*(l/16) + e.  The first 256 threads own the
-  // cells of the tiles: thread tid owns cell (l = tid/4, e = tid%4) of every row tile and column block.
-  const int l = tid / 4, e = tid % 4;
   float v[RT][MT];
 #pragma unroll
   for (int t = 0; t < MT; ++t) {
@@ -1265,7 +1304,6 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_skinny_kernel(const void* __r
       v[rt][t] = s * scale;
     }
   }
-  const int nrow = 4 * (l / 16) + e;  // row of the tile, 0..15
   if (EPI == EPI_SILU_MUL) {
     // rows 0..7 are gate, 8..15 the matching up rows: the up values travel through LDS.  Only the
     // first four waves are here; the slice of the last wave is free once every sum above is done.
@@ -1315,13 +1353,14 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_skinny_kernel(const void* __r
         float y = v[rt][t];
         if (!is_value && rope.cosv != nullptr) {
           const float p = other[(rt * MT + t) * 256 + (tid ^ 128)];
-          const float cs = rope.cosv[(size_t)m * half + pair], sn = rope.sinv[(size_t)m * half + pair];
-          y = upper ? y * cs + p * sn : y * cs - p * sn;
+          const float co = ROPE_EARLY ? cs[rt][t] : rope.cosv[(size_t)m * half + pair];
+          const float si = ROPE_EARLY ? sn[rt][t] : rope.sinv[(size_t)m * half + pair];
+          y = upper ? y * co + p * si : y * co - p * si;
         }
         const bf16 yb = (bf16)y;
         c[(size_t)m * ldc + head * rope.hd + dim] = (CT)yb;
         if (rope.slots != nullptr && head >= rope.nh) {
-          const int slot = rope.slots[m], page = slot / rope.page_size, off = slot % rope.page_size;
+          const int sl = ROPE_EARLY ? slot[t] : rope.slots[m], page = sl / rope.page_size, off = sl % rope.page_size;
           if (is_key)
             rope.k_pages[((size_t)page * rope.nkv + (head - rope.nh)) * rope.page_size * rope.hd +
                          key_offset(off, dim, rope.page_size, 8)] = yb;  // hd is a multiple of 16: pieces of 8
@@ -1331,24 +1370,8 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_skinny_kernel(const void* __r
       }
     }
   } else {
-    // accumulating: all of a thread's old values are asked for before any is added to (behind the checks one
-    // by one, every read would wait for the one before it)
-    float old[RT][MT];
-    const bool emits = EPI == EPI_ACCUMULATE && extra.emit_h != nullptr;
-    const bool empty = HALF && nrow >= 8;  // the lower half of a half tile
+    // accumulating onto the old values asked for above
     if (empty && !emits) return;
-    constexpr int ROWS = HALF ? 8 : 16;  // rows of W a tile owns
-    if (EPI == EPI_ACCUMULATE) {
-#pragma unroll
-      for (int rt = 0; rt < RT; ++rt) {
-        const int n = (blockIdx.x * RT + rt) * ROWS + nrow;
-#pragma unroll
-        for (int t = 0; t < MT; ++t) {
-          const int m = t * 16 + l % 16;
-          old[rt][t] = (!empty && m < M && n < N) ? (float)c[(size_t)m * ldc + n] : 0.f;
-        }
-      }
-    }
     float sq[RT][MT];
 #pragma unroll
     for (int rt = 0; rt < RT; ++rt) {
@@ -1361,8 +1384,7 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_skinny_kernel(const void* __r
           const float now = EPI == EPI_ACCUMULATE ? old[rt][t] + v[rt][t] : v[rt][t];
           c[(size_t)m * ldc + n] = (CT)now;
           if (emits) {
-            const float g = extra.emit_gamma_f32 ? ((const float*)extra.emit_gamma)[n] : (float)((const bf16*)extra.emit_gamma)[n];
-            extra.emit_h[(size_t)m * extra.emit_ldh + n] = (bf16)(g * now);
+            extra.emit_h[(size_t)m * extra.emit_ldh + n] = (bf16)(emit_g[rt] * now);
             sq[rt][t] = now * now;
           }
         }
@@ -1426,6 +1448,24 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_fold_kernel(const void* __res
 #pragma unroll
     for (int e = 0; e < 4; ++e) acc[rt][e] = 0.f;
 
+  // D[n, m]: lane l holds column m = l%16 and rows n = 4*(l/16) + e; thread tid of the first four waves owns cell
+  // (l = tid/4, e = tid%4) at the end.  What it will need from memory then (the cell's old value, the gamma of a norm
+  // to prepare) is asked for now, so that it arrives under the stream of W and not after it.
+  const int l = (tid % 256) / 4, e = tid % 4;
+  const int nrow = 4 * (l / 16) + e, m = l % 16;
+  const bool emits = EPI == EPI_ACCUMULATE && extra.emit_h != nullptr;
+  const bool mine = tid < 256 && nrow < 8 && m < 8;
+  float old[RT], emit_g[RT];
+#pragma unroll
+  for (int rt = 0; rt < RT; ++rt) {
+    const int n = (blockIdx.x * RT + rt) * 8 + nrow;
+    old[rt] = emit_g[rt] = 0.f;
+    if (mine && m < M && n < N) {
+      if (EPI == EPI_ACCUMULATE) old[rt] = (float)c[(size_t)m * ldc + n];
+      if (emits) emit_g[rt] = extra.emit_gamma_f32 ? ((const float*)extra.emit_gamma)[n] : (float)((const bf16*)extra.emit_gamma)[n];
+    }
+  }
+
   for (int kbeg = 0; kbeg < K; kbeg += ITERS * WAVES * 128) {
     bf16x8 wf[RT][ITERS][2], xf[ITERS][2];
 #pragma unroll
@@ -1457,11 +1497,6 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_fold_kernel(const void* __res
   if (RMS) sspart[wave][lane] = ss;
   __syncthreads();
   if (tid >= 256) return;
-  // D[n, m]: lane l holds column m = l%16 and rows n = 4*(l/16) + e; thread tid owns cell (l = tid/4, e = tid%4)
-  const int l = tid / 4, e = tid % 4;
-  const int nrow = 4 * (l / 16) + e, m = l % 16;
-  const bool emits = EPI == EPI_ACCUMULATE && extra.emit_h != nullptr;
-  const bool mine = nrow < 8 && m < 8;
   if (!mine && !emits) return;
   float scale = 1.f;
   if (RMS && mine) {
@@ -1481,13 +1516,9 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_fold_kernel(const void* __res
       float sum = 0.f;
 #pragma unroll
       for (int wv = 0; wv < WAVES; ++wv) sum += part[wv][rt][l][e] + part[wv][rt][l + 40][e];  // cell (n + 8, m + 8)
-      CT* cell = c + (size_t)m * ldc + n;
-      now = EPI == EPI_ACCUMULATE ? (float)*cell + sum * scale : sum * scale;
-      *cell = (CT)now;
-      if (emits) {
-        const float g = extra.emit_gamma_f32 ? ((const float*)extra.emit_gamma)[n] : (float)((const bf16*)extra.emit_gamma)[n];
-        extra.emit_h[(size_t)m * extra.emit_ldh + n] = (bf16)(g * now);
-      }
+      now = EPI == EPI_ACCUMULATE ? old[rt] + sum * scale : sum * scale;
+      c[(size_t)m * ldc + n] = (CT)now;
+      if (emits) extra.emit_h[(size_t)m * extra.emit_ldh + n] = (bf16)(emit_g[rt] * now);
     }
     if (emits && mine) squares[rt][m][nrow] = now * now;
   }
