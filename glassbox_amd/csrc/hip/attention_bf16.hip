@@ -222,49 +222,64 @@ __global__ __launch_bounds__(WAVES * 64) void decode_kernel(const bf16* __restri
 }
 
 // One block of 256 threads per (request, head): the chunks' partial results, combined in a fixed order.
-// The chunks are dealt to 256 / hd groups of threads, each thread of a group taking one dimension, so
-// that few loads depend on each other; the groups' sums meet in LDS.
+// The chunks are dealt to 256 / hd groups of threads, each thread of a group taking one dimension; the groups' sums
+// meet in LDS.  Everything a thread reads from memory depends on nothing but the request's position, so it is all
+// asked for at once (a chunk's maximum and sum by thread k, the first partial results of the thread's dimension),
+// and the maximum over the chunks and the sum of their weights are taken wave by wave, not by one thread in turn:
+// the kernel is short, and round trips and serial loops are what it consists of.
 __global__ __launch_bounds__(256) void decode_reduce_kernel(const float* __restrict__ ws_acc, const float* __restrict__ ws_ml,
                                                             bf16* __restrict__ out, int out_stride,
                                                             const int32_t* __restrict__ positions, int nh, int hd, int window,
                                                             int chunk, int splits) {
-  __shared__ float sm_f[256];        // chunk k's weight exp(m_k - M), then times nothing: l_k is kept beside
-  __shared__ float sm_l[256];
+  constexpr int EARLY = 4;           // partial results a thread asks for before it knows their weights
+  __shared__ float sm_f[256];        // chunk k's weight exp(m_k - M)
   __shared__ float sm_part[256];     // [group][dimension]
-  __shared__ float sm_top;
-  const int s = blockIdx.x / nh, head = blockIdx.x % nh, tid = threadIdx.x;
+  __shared__ float sm_top[4], sm_sum[4];
+  const int s = blockIdx.x / nh, head = blockIdx.x % nh, tid = threadIdx.x, lane = tid % 64, wave = tid / 64;
   const int pos = positions[s];
   const int lo = window > 0 ? max(0, pos - window + 1) : 0;
   const int first = lo / chunk, last = pos / chunk, count = last - first + 1;  // at most 256 chunks hold keys
   const size_t base = ((size_t)s * nh + head) * splits + first;
-  float mine = -INFINITY;
-  if (tid < count) {
-    mine = ws_ml[(base + tid) * 2];
-    sm_l[tid] = ws_ml[(base + tid) * 2 + 1];
-  }
-  sm_f[tid] = mine;
-  __syncthreads();
-  if (tid == 0) {
-    float top = -INFINITY;
-    for (int k = 0; k < count; ++k) top = fmaxf(top, sm_f[k]);
-    sm_top = top;
-  }
-  __syncthreads();
-  const float top = sm_top;
-  __syncthreads();
-  if (tid < count) sm_f[tid] = __expf(mine - top);
-  __syncthreads();
   const int groups = 256 / hd;  // hd <= 128: at least two
   const int d = tid % hd, group = tid / hd;
+  float mine = -INFINITY, mine_l = 0.f, early[EARLY];
+  if (tid < count) {
+    mine = ws_ml[(base + tid) * 2];
+    mine_l = ws_ml[(base + tid) * 2 + 1];
+  }
+#pragma unroll
+  for (int i = 0; i < EARLY; ++i) {
+    const int k = group + i * groups;
+    early[i] = (group < groups && k < count) ? ws_acc[(base + k) * hd + d] : 0.f;
+  }
+  float top = mine;
+#pragma unroll
+  for (int off = 32; off >= 1; off >>= 1) top = fmaxf(top, __shfl_xor(top, off, kWave));
+  if (lane == 0) sm_top[wave] = top;
+  __syncthreads();
+  top = fmaxf(fmaxf(sm_top[0], sm_top[1]), fmaxf(sm_top[2], sm_top[3]));
+  const float f = tid < count ? __expf(mine - top) : 0.f;
+  sm_f[tid] = f;
+  float sum = f * mine_l;  // the chunks' sums, weighted: added lane pairs first, then the waves in order
+#pragma unroll
+  for (int off = 1; off <= 32; off <<= 1) sum += __shfl_xor(sum, off, kWave);
+  if (lane == 0) sm_sum[wave] = sum;
+  __syncthreads();
   float val = 0.f;
-  if (group < groups)
-    for (int k = group; k < count; k += groups) val += ws_acc[(base + k) * hd + d] * sm_f[k];
+  if (group < groups) {
+#pragma unroll
+    for (int i = 0; i < EARLY; ++i) {
+      const int k = group + i * groups;
+      if (k < count) val += early[i] * sm_f[k];
+    }
+    for (int k = group + EARLY * groups; k < count; k += groups) val += ws_acc[(base + k) * hd + d] * sm_f[k];
+  }
   sm_part[tid] = val;
   __syncthreads();
   if (tid < hd) {
-    float total = 0.f, l = 0.f;
+    float total = 0.f;
     for (int g = 0; g < groups; ++g) total += sm_part[g * hd + tid];
-    for (int k = 0; k < count; ++k) l += sm_l[k] * sm_f[k];
+    const float l = ((sm_sum[0] + sm_sum[1]) + sm_sum[2]) + sm_sum[3];
     out[(size_t)s * out_stride + (size_t)head * hd + tid] = (bf16)(total / l);
   }
 }
