@@ -249,6 +249,11 @@ void gbh_sched_row_params(void* h, int j, float* temperature, int* top_k, float*
 }
 // Tokens (prompt and generated) of the request behind wanted row j: the penalty's context.
 int gbh_sched_row_context(void* h, int j, int32_t* out, int cap) { return ((gb::Scheduler*)h)->row_context(j, out, cap); }
+// The repetition penalty's work for the wanted rows: (row, token, occurrences, penalty) for every distinct token of
+// a row with a penalty; returns their number (ask with cap 0, then fill).
+int gbh_sched_penalty_pairs(void* h, int32_t* rows, int32_t* tokens, int32_t* counts, float* penalties, int cap) {
+  return ((gb::Scheduler*)h)->penalty_pairs(rows, tokens, counts, penalties, cap);
+}
 // Finishes the planned step: commits, appends sampled tokens (one per wanted row, with how many
 // candidates the draw had), finishes requests.
 void gbh_sched_finish(void* h, const int32_t* sampled, const int32_t* n_candidates, int n_rows) {

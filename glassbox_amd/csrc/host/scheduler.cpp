@@ -193,6 +193,25 @@ int Scheduler::row_context(int j, int32_t* out, int cap) const {
   return n;
 }
 
+int Scheduler::penalty_pairs(int32_t* rows, int32_t* tokens, int32_t* counts, float* penalties, int cap) {
+  int n = 0;
+  for (int j = 0; j < (int)wants_for_.size(); ++j) {
+    Seq& s = running_[wants_for_[j]];
+    if (s.sampler.repetition_penalty == 1.0f) continue;
+    for (; s.counted < s.tokens.size(); ++s.counted) ++s.occurrences[s.tokens[s.counted]];
+    for (const auto& kv : s.occurrences) {
+      if (n < cap) {
+        rows[n] = j;
+        tokens[n] = kv.first;
+        counts[n] = kv.second;
+        penalties[n] = s.sampler.repetition_penalty;
+      }
+      ++n;
+    }
+  }
+  return n;
+}
+
 void Scheduler::finish(const int32_t* sampled, const int32_t* n_candidates, int n_rows) {
   if (plan_.empty()) return;
   // commit what the step wrote (scheduler.rs:356-368)

@@ -9,6 +9,7 @@
 #pragma once
 #include <cstdint>
 #include <deque>
+#include <unordered_map>
 #include <vector>
 
 #include "cache_manager.h"
@@ -47,6 +48,9 @@ class Scheduler {
   int row_context(int j, int32_t* out, int cap) const;
   void finish(const int32_t* sampled, const int32_t* n_candidates, int n_rows);
 
+  // The repetition penalty of the wanted rows as (row, token, occurrences, penalty), one for every distinct token of
+  // a row whose request has a penalty other than 1.  Returns how many there are; fills at most `cap`.
+  int penalty_pairs(int32_t* rows, int32_t* tokens, int32_t* counts, float* penalties, int cap);
   int take_events(int64_t* ids, int32_t* kinds, int32_t* values, int cap);
   bool request_counts(int64_t id, int* prompt_tokens, int* completion_tokens) const;
   void metrics(int64_t* out7) const;
@@ -62,6 +66,10 @@ class Scheduler {
     SamplerConfig sampler;
     Rng rng;
     std::vector<int32_t> stop;
+    // how often each token occurs among the first `counted` tokens: kept for requests with a repetition penalty,
+    // brought up to date when their penalty is asked for, so that a step costs what it adds and not the context
+    std::unordered_map<int32_t, int32_t> occurrences;
+    size_t counted = 0;
     int generated() const { return (int)tokens.size() - prompt_len; }
   };
   struct Event { int64_t id; int32_t kind; int32_t value; };

@@ -45,6 +45,7 @@ def _host():
             "rows_params": (None, [vp, C.c_int] + [vp] * 7),
             "row_params": (None, [vp, C.c_int, fp, ip, fp, fp, fp, fp, ip]),
             "row_context": (C.c_int, [vp, C.c_int, i32p, C.c_int]),
+            "penalty_pairs": (C.c_int, [vp] + [vp] * 4 + [C.c_int]),
             "finish": (None, [vp, i32p, i32p, C.c_int]),
             "take_events": (C.c_int, [vp, i64p, i32p, i32p, C.c_int]),
             "request_counts": (C.c_int, [vp, i64, ip, ip]),
@@ -181,19 +182,29 @@ class Scheduler:
         temp, top_p, min_p, penalty, uniforms = (a[:rows] for a in fl.tolist())
         top_k = it[0].tolist()[:rows]
         if self.sample_fn is sample_rows and rows and max(temp) <= 0.0 and all(p == 1.0 for p in penalty):
-            configs, contexts = self._greedy[:rows] if rows <= len(self._greedy) else [SamplerConfig()] * rows, None
+            configs, more = self._greedy[:rows] if rows <= len(self._greedy) else [SamplerConfig()] * rows, ()
         else:
             configs = [SamplerConfig(temp[j], top_k[j], top_p[j], min_p[j], penalty[j]) for j in range(rows)]
-            contexts = []
-            for j in range(rows):
-                if penalty[j] != 1.0:
-                    m = lib.gbh_sched_row_context(h, j, None, 0)
-                    cb = (C.c_int32 * max(1, m))()
-                    lib.gbh_sched_row_context(h, j, cb, m)
-                    contexts.append(list(cb[:m]))
-                else:
-                    contexts.append([])
-        tokens, cands = self.sample_fn(logits, configs, uniforms, contexts) if rows else ([], [])
+            if self.sample_fn is sample_rows:
+                # the native scheduler keeps count of every such request's tokens: (row, token, occurrences, penalty)
+                m = lib.gbh_sched_penalty_pairs(h, None, None, None, None, 0) if any(p != 1.0 for p in penalty) else 0
+                pairs = np.empty((4, m), np.int32)
+                if m:
+                    lib.gbh_sched_penalty_pairs(h, pairs[0].ctypes.data, pairs[1].ctypes.data, pairs[2].ctypes.data,
+                                                pairs[3].ctypes.data, m)
+                more = (None, pairs)
+            else:
+                contexts = []
+                for j in range(rows):
+                    if penalty[j] != 1.0:
+                        m = lib.gbh_sched_row_context(h, j, None, 0)
+                        cb = (C.c_int32 * max(1, m))()
+                        lib.gbh_sched_row_context(h, j, cb, m)
+                        contexts.append(list(cb[:m]))
+                    else:
+                        contexts.append([])
+                more = (contexts,)
+        tokens, cands = self.sample_fn(logits, configs, uniforms, *more) if rows else ([], [])
         lib.gbh_sched_finish(h, (C.c_int32 * max(1, rows))(*tokens), (C.c_int32 * max(1, rows))(*cands), rows)
         finished = self._drain_events()
         self._steps += 1

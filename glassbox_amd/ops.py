@@ -717,7 +717,8 @@ def penalize(logits: torch.Tensor, rows: torch.Tensor, tokens: torch.Tensor, cou
 def sample(logits: torch.Tensor, temperature: torch.Tensor, top_k: torch.Tensor, top_p: torch.Tensor,
            min_p: torch.Tensor, uniform: torch.Tensor, out_token: torch.Tensor, out_candidates: torch.Tensor) -> None:
     """The reference's sampler per row: temperature, top-k, min-p, top-p, then an inverse-CDF draw in
-    descending order of probability with the given uniform number; temperature <= 0 is greedy."""
+    descending order of probability with the given uniform number; temperature <= 0 is greedy.  A row that is not
+    greedy is left divided by its temperature."""
     rows, vocab = _logit_rows(logits)
     for t, what in ((temperature, "temperature"), (top_p, "top_p"), (min_p, "min_p"), (uniform, "uniform")):
         if t.dtype != torch.float32 or t.numel() < rows or not t.is_cuda:

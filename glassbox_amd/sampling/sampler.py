@@ -14,6 +14,7 @@ from collections import Counter
 from dataclasses import dataclass
 from typing import List, Optional, Sequence, Tuple
 
+import numpy as np
 import torch
 
 from .. import build, ops
@@ -53,9 +54,34 @@ class Rng:
         return v
 
 
+def penalty_pairs(configs: Sequence[SamplerConfig], contexts: Optional[Sequence[Sequence[int]]]) -> Optional[np.ndarray]:
+    """The repetition penalty's work as one int32 array [4, pairs]: row, token, occurrences of the token in the row's
+    context, and the penalty's bits, for every distinct token of a row whose penalty is not 1 (sampler.rs:100-108
+    applies it once per occurrence).  None if there is nothing to do."""
+    if contexts is None:
+        return None
+    parts = []
+    for r, cfg in enumerate(configs):
+        if cfg.repetition_penalty != 1.0 and len(contexts[r]):
+            counts = contexts[r] if isinstance(contexts[r], Counter) else Counter(contexts[r])
+            part = np.empty((4, len(counts)), np.int32)
+            part[0] = r
+            part[1] = np.fromiter(counts.keys(), np.int32, len(counts))
+            part[2] = np.fromiter(counts.values(), np.int32, len(counts))
+            part[3] = np.float32(cfg.repetition_penalty).view(np.int32)
+            parts.append(part)
+    if not parts:
+        return None
+    return parts[0] if len(parts) == 1 else np.concatenate(parts, axis=1)
+
+
 def sample_rows(logits: torch.Tensor, configs: Sequence[SamplerConfig], uniforms: Sequence[float],
-                contexts: Optional[Sequence[Sequence[int]]] = None) -> Tuple[List[int], List[int]]:
-    """Samples one token per row of ``logits`` (float32 on the GPU; penalties are applied in place).
+                contexts: Optional[Sequence[Sequence[int]]] = None,
+                pairs: Optional[np.ndarray] = None) -> Tuple[List[int], List[int]]:
+    """Samples one token per row of ``logits`` (float32 on the GPU; penalties and temperatures are applied in place).
+
+    ``contexts[r]`` is the context of row r for the repetition penalty: its tokens, or a ``Counter`` of them; a
+    caller that keeps count itself passes ``pairs`` (the array of ``penalty_pairs``) in their place.
 
     Returns (tokens, candidates): ``candidates[r]`` is how many tokens the draw of row r chose
     among; the caller advances the row's generator only if that is more than one, as the
@@ -65,22 +91,23 @@ def sample_rows(logits: torch.Tensor, configs: Sequence[SamplerConfig], uniforms
     if rows == 0:
         return [], []
     # the repetition penalty, once per occurrence of a token in the row's context
-    pr, pt, pc, pp = [], [], [], []
-    for r, cfg in enumerate(configs):
-        if cfg.repetition_penalty != 1.0 and contexts is not None and contexts[r]:
-            for tok, cnt in Counter(contexts[r]).items():
-                pr.append(r); pt.append(tok); pc.append(cnt); pp.append(cfg.repetition_penalty)
-    if pr:
-        ops.penalize(logits, torch.tensor(pr, dtype=torch.int32, device=dev), torch.tensor(pt, dtype=torch.int32, device=dev),
-                     torch.tensor(pc, dtype=torch.int32, device=dev), torch.tensor(pp, dtype=torch.float32, device=dev))
+    if pairs is None:
+        pairs = penalty_pairs(configs, contexts)
+    if pairs is not None and pairs.shape[1]:
+        p = torch.from_numpy(np.ascontiguousarray(pairs, np.int32)).to(dev)      # one copy for the four columns
+        ops.penalize(logits, p[0], p[1], p[2], p[3].view(torch.float32))
     out = torch.empty(2, rows, dtype=torch.int32, device=dev)
     if all(cfg.temperature <= 0.0 for cfg in configs):
         ops.argmax(logits, out[0])
         return out[0].tolist(), [1] * rows
-    fl = torch.tensor([[c.temperature for c in configs], [c.top_p for c in configs], [c.min_p for c in configs],
-                       list(uniforms)], dtype=torch.float32, device=dev)
-    tk = torch.tensor([c.top_k for c in configs], dtype=torch.int32, device=dev)
-    ops.sample(logits, fl[0], tk, fl[1], fl[2], fl[3], out[0], out[1])
+    # temperature, top_p, min_p, the uniform number and top_k of every row: one copy, the numbers as their bits
+    host = np.empty((5, rows), np.int32)
+    host[:4].view(np.float32)[:] = ([c.temperature for c in configs], [c.top_p for c in configs],
+                                    [c.min_p for c in configs], list(uniforms))
+    host[4] = [c.top_k for c in configs]
+    par = torch.from_numpy(host).to(dev)
+    fl = par[:4].view(torch.float32)
+    ops.sample(logits, fl[0], par[4], fl[1], fl[2], fl[3], out[0], out[1])
     both = out.tolist()
     return both[0], both[1]
 
@@ -91,11 +118,25 @@ class Sampler:
     def __init__(self, config: SamplerConfig):
         self.config = config
         self.rng = Rng(config.seed)
+        self._seen: List[int] = []          # the context of the last call, counted in _counts
+        self._counts: Counter = Counter()
+
+    def _count(self, context: Sequence[int]) -> Counter:
+        """How often each token occurs in ``context``.  A request's context grows by a token a call: what the last
+        call counted is kept, and only what follows it is added."""
+        context = list(context)
+        n = len(self._seen)
+        if len(context) < n or context[:n] != self._seen:
+            self._counts, n = Counter(), 0
+        self._counts.update(context[n:])
+        self._seen = context
+        return self._counts
 
     def sample(self, logits_row: torch.Tensor, context: Sequence[int] = ()) -> int:
         """logits_row: float32 [vocab] or [1, vocab] on the GPU."""
         row = logits_row.reshape(1, -1)
-        toks, cands = sample_rows(row, [self.config], [self.rng.peek_f32()], [list(context)])
+        ctx = [self._count(context)] if self.config.repetition_penalty != 1.0 else None
+        toks, cands = sample_rows(row, [self.config], [self.rng.peek_f32()], ctx)
         if self.config.temperature > 0.0 and cands[0] > 1:
             self.rng.next_f32()
         return toks[0]

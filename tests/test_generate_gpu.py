@@ -49,13 +49,15 @@ def test_sampler_vectors_of_the_reference_on_the_device():
     assert toks == [2]
 
 
-@pytest.mark.parametrize("vocab", [97, 331, 49152])
-def test_sampling_kernel_agrees_with_the_plain_sampler(vocab):
+@pytest.mark.parametrize("vocab,spread", [(97, 3.0), (331, 3.0), (49152, 3.0), (2500, 0.05), (49152, 0.2), (128256, 2.0)])
+def test_sampling_kernel_agrees_with_the_plain_sampler(vocab, spread):
+    """Rows of peaked and of nearly flat logits (random weights give the latter: the draw then falls among thousands
+    of tokens of almost one probability), with every filter on and off, against the plain sampler."""
     from glassbox_amd.sampling import SamplerConfig, sample_rows
-    g = torch.Generator().manual_seed(vocab)
-    rng = random.Random(vocab)
+    g = torch.Generator().manual_seed(vocab + int(spread * 100))
+    rng = random.Random(vocab + int(spread * 100))
     rows = 24 if vocab < 1000 else 6
-    logits = torch.randn(rows, vocab, generator=g) * 3
+    logits = torch.randn(rows, vocab, generator=g) * spread
     logits[0, 5] = logits[0, 9] = logits[0].max() + 1         # ties at the top go by token id
     logits[1, :] = 0.25                                        # every logit equal
     cfgs, ctxs, us = [], [], []
@@ -68,20 +70,39 @@ def test_sampling_kernel_agrees_with_the_plain_sampler(vocab):
     toks, cands = sample_rows(logits.to(DEV), cfgs, us, ctxs)
     for r in range(rows):
         c = cfgs[r]
-        dist = psampler.distribution(logits[r].tolist(), ctxs[r], c.temperature, c.top_k, c.top_p, c.min_p,
-                                     c.repetition_penalty)
-        assert cands[r] == len(dist), (r, c)
-        acc, want = np.float32(0), dist[-1][0]
-        near_edge = False
-        for t, p in dist:
-            acc = np.float32(acc + np.float32(p))
-            near_edge |= abs(float(acc) - us[r]) < 1e-5       # a draw this close to a boundary may round either way
-            if us[r] < acc:
-                want = t
-                break
-        if len(dist) == 1:
-            want = dist[0][0]
-        assert toks[r] == want or near_edge, (r, c, toks[r], want)
+        row = logits[r].tolist()
+        dist = psampler.distribution(row, ctxs[r], c.temperature, c.top_k, c.top_p, c.min_p, c.repetition_penalty)
+        if len(dist) == 1 and c.top_p >= 1.0:
+            assert (toks[r], cands[r]) == (dist[0][0], 1), (r, c)
+            continue
+        # The plain sampler adds its n probabilities in 32-bit one after the other, as the reference does: its running
+        # sum is off by some sqrt(n) roundings, and a boundary that lies within that of the target may fall either side.
+        if c.top_p < 1.0 and c.temperature > 0.0:
+            # the candidates that top-p chooses among, with the probabilities it adds up: the softmax over the top k,
+            # of which min-p keeps a prefix
+            kept = len(psampler.distribution(row, ctxs[r], c.temperature, c.top_k, 1.0, c.min_p, c.repetition_penalty))
+            full = psampler.distribution(row, ctxs[r], c.temperature, c.top_k, 1.0, 0.0, c.repetition_penalty)[:kept]
+            run = np.cumsum(np.array([p for _, p in full], dtype=np.float64))
+            eps = max(1e-5, 4 * math.sqrt(len(full)) * 2.0 ** -24)
+            n = cands[r]
+            assert 1 <= n <= len(full), (r, c, n)
+            assert run[n - 1] >= c.top_p - eps or n == len(full), (r, c, n, len(dist))      # the prefix reaches top_p
+            assert n == 1 or run[n - 2] < c.top_p + eps, (r, c, n, len(dist))               # and is the shortest that does
+            order = [t for t, _ in full[:n]]
+            probs = np.array([p for _, p in full[:n]], dtype=np.float64)
+            probs /= probs.sum()
+        else:
+            assert cands[r] == len(dist), (r, c)
+            order = [t for t, _ in dist]
+            probs = np.array([p for _, p in dist], dtype=np.float64)
+        if len(order) == 1:
+            assert toks[r] == order[0], (r, c)
+            continue
+        # the token drawn is the one whose stretch of the running probability holds the uniform number
+        run = np.cumsum(probs)
+        eps = max(1e-5, 4 * math.sqrt(len(order)) * 2.0 ** -24)
+        at = order.index(toks[r])
+        assert (run[at - 1] if at else 0.0) <= us[r] + eps and run[at] >= us[r] - eps, (r, c, toks[r], at, us[r])
 
 
 def test_temperature_draws_follow_the_softmax():

@@ -231,3 +231,43 @@ def test_nothing_to_do():
         s.submit([], 3)
     with pytest.raises(ValueError):
         s.submit([V], 3)
+
+
+def test_the_penalty_pairs_count_each_requests_tokens():
+    """The native scheduler's (row, token, occurrences, penalty) for the wanted rows of a step are what counting
+    each request's context gives (sampler.rs:100-108 walks the context token by token), in steps with portions,
+    under preemption, for requests with and without a penalty."""
+    import numpy as np
+    from collections import Counter
+    rng = random.Random(5)
+    eng = ToyEngine(14, 6)
+    s = None
+    seen = {"steps": 0, "pairs": 0}
+
+    def checked(logits, configs, uniforms, contexts):
+        lib, h = s._lib, s._h
+        m = lib.gbh_sched_penalty_pairs(h, None, None, None, None, 0)
+        pairs = np.zeros((4, m), np.int32)
+        if m:
+            assert lib.gbh_sched_penalty_pairs(h, pairs[0].ctypes.data, pairs[1].ctypes.data, pairs[2].ctypes.data,
+                                               pairs[3].ctypes.data, m) == m
+        got = {}
+        for r, t, c, p in zip(pairs[0].tolist(), pairs[1].tolist(), pairs[2].tolist(), pairs[3].view(np.float32).tolist()):
+            assert (r, t) not in got
+            got[(r, t)] = (c, p)
+        want = {}
+        for r, (cfg, ctx) in enumerate(zip(configs, contexts)):
+            if cfg.repetition_penalty != 1.0:
+                for t, c in Counter(ctx).items():
+                    want[(r, t)] = (c, np.float32(cfg.repetition_penalty).item())
+        assert got == want
+        seen["steps"] += 1
+        seen["pairs"] += m
+        return cpu_sample_rows(logits, configs, uniforms, contexts)
+
+    s = Scheduler(eng, SchedulerConfig(32, 6), sample_fn=checked)
+    for i in range(10):
+        cfg = SamplerConfig(temperature=0.8, repetition_penalty=[1.0, 1.3, 2.0][i % 3], seed=i)
+        s.submit(random_prompt(rng), 12, cfg)
+    s.run()
+    assert s.is_idle() and seen["steps"] > 20 and seen["pairs"] > 100

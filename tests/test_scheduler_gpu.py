@@ -113,7 +113,10 @@ def test_seeded_temperature_replies_are_the_plain_samplers(model_dirs):
     folder = model_dirs.get("B")
     cfg, w = plain.load_folder(folder)
     prompts = [helpers.random_tokens(384, n, seed=n) for n in (1, 9, 40, 70)]
-    samplers = [SamplerConfig(temperature=0.8, seed=s) for s in (1, 2, 3, 4)]
+    # (two of them with a repetition penalty, which the native scheduler counts tokens for, one with every filter)
+    samplers = [SamplerConfig(temperature=0.8, seed=1), SamplerConfig(temperature=0.8, repetition_penalty=1.3, seed=2),
+                SamplerConfig(temperature=0.8, top_k=40, top_p=0.9, min_p=0.002, repetition_penalty=1.2, seed=3),
+                SamplerConfig(temperature=0.8, seed=4)]
     eng = Engine(folder, dtype="float32", max_tokens=2048, max_seqs=8)
     replies, sched, records = serve(eng, prompts, max_tokens=24, samplers=samplers, budget=16, max_seqs=8)
     compared = 0
