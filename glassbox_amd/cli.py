@@ -82,6 +82,7 @@ def cmd_generate(a) -> int:
         return 2
     # as the reference: a cache of exactly prompt + n + 1 tokens for the one request (main.rs:147)
     eng = _engine(a, blocks=-(-(len(prompt) + a.n + 1) // 16))
+    eng.warm_up(len(prompt))     # code loaded, buffers sized, the decode graph captured: the times below are the steps' own
     gen, sampler, stop = Generator(eng), Sampler(_sampler(a)), set(_ids(a.stop))
     torch.cuda.synchronize()
     t0 = time.time()
@@ -109,6 +110,7 @@ def cmd_batch(a) -> int:
     with open(a.prompts) as fh:
         prompts = [_ids(line) for line in fh if line.strip()]
     eng = _engine(a)
+    eng.warm_up(min(a.budget, 64))
     t0 = time.time()
     outs, sched = generate(eng, prompts, a.n, _sampler(a), _ids(a.stop), a.budget, a.max_seqs, return_scheduler=True)
     secs = time.time() - t0

@@ -158,6 +158,22 @@ class Engine:
     def free_tokens(self) -> int:
         return self.cache.min_free_pages() * self.page_size
 
+    def warm_up(self, tokens: int = 32, decode_steps: int = 3) -> None:
+        """Runs a throwaway request (a prompt of ``tokens`` tokens, then single tokens) and gives back what it held.
+        The first step of a shape loads the kernels' code and sizes the buffers, and the second single-token step
+        of a length captures its graph: some 20 ms each that the first real request would otherwise wait for."""
+        name = ("warm-up", self._next_id)
+        tokens = max(1, min(tokens, self.free_tokens() - decode_steps - 1))
+        if self.free_tokens() < tokens + decode_steps + 1:
+            return
+        try:
+            self.step([(name, [0] * tokens, [tokens - 1])])
+            for _ in range(decode_steps):
+                self.step([(name, [0], [0])])
+        finally:
+            self.end_request(name)
+        torch.cuda.synchronize()
+
     # -------------------------------------------------------------------- the step
     def reserve(self, entries: Sequence[Entry]) -> None:
         """Makes room for every entry's tokens; raises OutOfPages when the pool is too small

@@ -239,6 +239,25 @@ def test_seeded_temperature_generation_repeats(model_dirs):
     assert a == b and a != c and all(len(o) == 24 for o in a)
 
 
+def test_a_warm_up_leaves_nothing_behind(model_dirs):
+    """``Engine.warm_up`` runs a throwaway request: afterwards no page is held, no request is live, the decode graph of
+    that length is there, and a request's logits are what they are without it; a pool too small for it is left alone."""
+    from glassbox_amd.engine import Engine
+    folder = model_dirs.get("B")
+    prompt = helpers.random_tokens(384, 21, seed=2)
+    plain_engine = Engine(folder, dtype="float32", max_tokens=128, max_seqs=2)
+    want = plain_engine.step([("a", prompt, [20])]).clone()
+    eng = Engine(folder, dtype="float32", max_tokens=128, max_seqs=2)
+    eng.warm_up(len(prompt))
+    assert eng.cache.used_pages() == 0 and not eng._ids
+    assert eng.decode_graphs is None or eng.decode_graphs.shapes
+    assert torch.equal(eng.step([("a", prompt, [20])]), want)
+    eng.end_request("a")
+    tiny = Engine(folder, dtype="float32", max_tokens=16, max_seqs=1)   # one page
+    tiny.warm_up(64)
+    assert tiny.cache.used_pages() == 0
+
+
 def _glassbox(*args, stdin=None):
     import os
     import subprocess
