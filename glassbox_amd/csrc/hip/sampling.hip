@@ -21,7 +21,7 @@ namespace {
 constexpr int IDX_BITS = 20;   // vocabulary up to 2^20
 
 __device__ __forceinline__ uint32_t ordered_bits(float v) {
-  const uint32_t u = __float_as_uint(v);
+  const uint32_t u = v == 0.f ? 0u : __float_as_uint(v);  // -0 and +0 are one value: they go by token id
   return (u & 0x80000000u) ? ~u : (u | 0x80000000u);  // larger float -> larger unsigned
 }
 // larger composite = earlier in the reference's order (larger logit first, then smaller id)

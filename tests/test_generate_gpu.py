@@ -24,10 +24,12 @@ def test_argmax_first_maximum_wins():
         logits[2, vocab - 1] = 10.0
         logits[3, :] = -1.5                                  # all equal: token 0
         logits[4, 0] = 11.0
+        logits[5] = -logits[5].abs()                         # zeros of both signs are one value: the first of them
+        logits[5, 2], logits[5, 4] = -0.0, 0.0
         out = torch.empty(6, dtype=torch.int32, device=DEV)
         ops.argmax(logits.to(DEV), out)
         assert out.tolist() == [psampler.argmax(r) for r in logits.tolist()]
-        assert out.tolist()[1:5] == [3, vocab - 1, 0, 0]
+        assert out.tolist()[1:] == [3, vocab - 1, 0, 0, 2]
 
 
 def test_sampler_vectors_of_the_reference_on_the_device():
@@ -49,6 +51,51 @@ def test_sampler_vectors_of_the_reference_on_the_device():
     assert toks == [2]
 
 
+def check_sampled(row, context, c, u, token, candidates):
+    """One row's token and number of candidates against the plain sampler.  The reference adds its probabilities in
+    32-bit, one after the other (sampler.rs:118-146,155-163); the kernel adds whole numbers, which is exact.  Where the
+    two differ, the 32-bit sums' rounding decides (a cut or a draw that falls within it of a boundary), so the kernel
+    must give either the plain sampler's answer or the one of the same formulas in 64-bit, within 2e-6 of a boundary."""
+    dist = psampler.distribution(row, context, c.temperature, c.top_k, c.top_p, c.min_p, c.repetition_penalty)
+    if c.temperature <= 0.0:
+        assert (token, candidates) == (dist[0][0], 1), c
+        return
+    delta = 2e-6
+    # the candidates before top-p, most likely first (min-p keeps a prefix of the top k), and exp(l - max) in 64-bit
+    kept = len(psampler.distribution(row, context, c.temperature, c.top_k, 1.0, c.min_p, c.repetition_penalty))
+    top = psampler.distribution(row, context, c.temperature, c.top_k, 1.0, 0.0, c.repetition_penalty)
+    l = np.array(row, dtype=np.float32)
+    if c.repetition_penalty != 1.0:
+        for t in context:
+            l[t] = l[t] / np.float32(c.repetition_penalty) if l[t] > 0 else l[t] * np.float32(c.repetition_penalty)
+    l = (l / np.float32(c.temperature)).astype(np.float32)
+    order = [t for t, _ in top]
+    e = np.exp(l[order].astype(np.float64) - float(l[order[0]]))
+    if c.top_p < 1.0:
+        run = np.cumsum(e[:kept]) / e.sum()                 # the softmax over the top k, min-p's prefix of it
+        n = candidates
+        exact = 1 <= n <= kept and (run[n - 1] >= c.top_p - delta or n == kept) and (n == 1 or run[n - 2] < c.top_p + delta)
+        assert exact or n == len(dist), (c, n, len(dist))
+    else:
+        n = candidates
+        assert n == len(dist), (c, n, len(dist))
+    if n == 1:
+        assert token == order[0], (c, token)
+        return
+    run = np.cumsum(e[:n]) / e[:n].sum()
+    at = order.index(token)
+    assert at < n, (c, token, at, n)
+    exact = (run[at - 1] if at else 0.0) <= u + delta and (run[at] >= u - delta or at == n - 1)
+    # the plain sampler's own draw, from its 32-bit running sum
+    acc, plain_draw = np.float32(0), dist[-1][0]
+    for t, p in dist:
+        acc = np.float32(acc + np.float32(p))
+        if u < acc:
+            plain_draw = t
+            break
+    assert exact or token == plain_draw, (c, token, at, plain_draw, u)
+
+
 @pytest.mark.parametrize("vocab,spread", [(97, 3.0), (331, 3.0), (49152, 3.0), (2500, 0.05), (49152, 0.2), (128256, 2.0)])
 def test_sampling_kernel_agrees_with_the_plain_sampler(vocab, spread):
     """Rows of peaked and of nearly flat logits (random weights give the latter: the draw then falls among thousands
@@ -60,6 +107,8 @@ def test_sampling_kernel_agrees_with_the_plain_sampler(vocab, spread):
     logits = torch.randn(rows, vocab, generator=g) * spread
     logits[0, 5] = logits[0, 9] = logits[0].max() + 1         # ties at the top go by token id
     logits[1, :] = 0.25                                        # every logit equal
+    if rows > 2:
+        logits[2] = (logits[2] * 2).round() / 2                # few values, many ties, zeros of both signs
     cfgs, ctxs, us = [], [], []
     for r in range(rows):
         cfgs.append(SamplerConfig(temperature=rng.choice([0.0, 0.6, 1.0, 2.0]), top_k=rng.choice([0, 0, 1, 7, 50]),
@@ -69,40 +118,40 @@ def test_sampling_kernel_agrees_with_the_plain_sampler(vocab, spread):
         us.append(rng.random())
     toks, cands = sample_rows(logits.to(DEV), cfgs, us, ctxs)
     for r in range(rows):
-        c = cfgs[r]
-        row = logits[r].tolist()
-        dist = psampler.distribution(row, ctxs[r], c.temperature, c.top_k, c.top_p, c.min_p, c.repetition_penalty)
-        if len(dist) == 1 and c.top_p >= 1.0:
-            assert (toks[r], cands[r]) == (dist[0][0], 1), (r, c)
-            continue
-        # The plain sampler adds its n probabilities in 32-bit one after the other, as the reference does: its running
-        # sum is off by some sqrt(n) roundings, and a boundary that lies within that of the target may fall either side.
-        if c.top_p < 1.0 and c.temperature > 0.0:
-            # the candidates that top-p chooses among, with the probabilities it adds up: the softmax over the top k,
-            # of which min-p keeps a prefix
-            kept = len(psampler.distribution(row, ctxs[r], c.temperature, c.top_k, 1.0, c.min_p, c.repetition_penalty))
-            full = psampler.distribution(row, ctxs[r], c.temperature, c.top_k, 1.0, 0.0, c.repetition_penalty)[:kept]
-            run = np.cumsum(np.array([p for _, p in full], dtype=np.float64))
-            eps = max(1e-5, 4 * math.sqrt(len(full)) * 2.0 ** -24)
-            n = cands[r]
-            assert 1 <= n <= len(full), (r, c, n)
-            assert run[n - 1] >= c.top_p - eps or n == len(full), (r, c, n, len(dist))      # the prefix reaches top_p
-            assert n == 1 or run[n - 2] < c.top_p + eps, (r, c, n, len(dist))               # and is the shortest that does
-            order = [t for t, _ in full[:n]]
-            probs = np.array([p for _, p in full[:n]], dtype=np.float64)
-            probs /= probs.sum()
+        check_sampled(logits[r].tolist(), ctxs[r], cfgs[r], us[r], toks[r], cands[r])
+
+
+def test_sampling_kernel_on_rows_of_ties_and_edge_settings():
+    """Rows that are all one value, two values, or a few (with zeros of both signs, which are one value and go by
+    token id), with filters at their edges: top-k of 1 and beyond the vocabulary, top-p of 0 and just below 1, min-p
+    of 1, uniform numbers of 0 and just below 1."""
+    from glassbox_amd.sampling import SamplerConfig, sample_rows
+    checked = 0
+    for seed in range(12):
+        rng = random.Random(seed)
+        g = torch.Generator().manual_seed(seed)
+        vocab = rng.choice([17, 150, 1025, 2500, 4099])
+        spread = rng.choice([0.02, 0.3, 1.0, 8.0])
+        logits = torch.randn(16, vocab, generator=g) * spread
+        mode = seed % 3
+        if mode == 0:
+            logits = (logits * 2).round() / 2
+        elif mode == 1:
+            logits = logits.sign() * spread
         else:
-            assert cands[r] == len(dist), (r, c)
-            order = [t for t, _ in dist]
-            probs = np.array([p for _, p in dist], dtype=np.float64)
-        if len(order) == 1:
-            assert toks[r] == order[0], (r, c)
-            continue
-        # the token drawn is the one whose stretch of the running probability holds the uniform number
-        run = np.cumsum(probs)
-        eps = max(1e-5, 4 * math.sqrt(len(order)) * 2.0 ** -24)
-        at = order.index(toks[r])
-        assert (run[at - 1] if at else 0.0) <= us[r] + eps and run[at] >= us[r] - eps, (r, c, toks[r], at, us[r])
+            logits[:] = rng.choice([0.0, -3.5, 7.25])
+        cfgs, ctxs, us = [], [], []
+        for r in range(16):
+            cfgs.append(SamplerConfig(temperature=rng.choice([0.0, 0.05, 0.6, 2.0, 5.0]), top_k=rng.choice([0, 1, 2, 50, vocab, vocab + 5]),
+                                      top_p=rng.choice([1.0, 0.95, 0.1, 0.0, 0.999]), min_p=rng.choice([0.0, 0.02, 0.9, 1.0]),
+                                      repetition_penalty=rng.choice([1.0, 1.2, 3.0])))
+            ctxs.append([rng.randrange(vocab) for _ in range(rng.randrange(0, 30))])
+            us.append(rng.choice([rng.random(), 0.0, 0.999999]))
+        toks, cands = sample_rows(logits.clone().to(DEV), cfgs, us, ctxs)
+        for r in range(16):
+            check_sampled(logits[r].tolist(), ctxs[r], cfgs[r], us[r], toks[r], cands[r])
+            checked += 1
+    assert checked == 192
 
 
 def test_temperature_draws_follow_the_softmax():
