@@ -1060,6 +1060,15 @@ int launch_split(const bf16* a, int lda, const bf16* w, int ldw, CT* c, int ldc,
 // rows are the float32 residual; the operand is bf16(gamma[k] * x[k]) and sum(x^2) is gathered on
 // the way, so that the caller can scale the finished product by 1/sqrt(mean(x^2) + eps): the RMS
 // norm (crates/glassbox-core/src/model.rs:94-100) without a pass of its own.
+// The 16 bytes that lane `lane` of the wave holds in v.
+__device__ __forceinline__ bf16x8 from_lane(bf16x8 v, int lane) {
+  typedef int i32x4 __attribute__((ext_vector_type(4)));
+  i32x4 w = __builtin_bit_cast(i32x4, v);
+#pragma unroll
+  for (int i = 0; i < 4; ++i) w[i] = __builtin_amdgcn_ds_bpermute(lane * 4, w[i]);
+  return __builtin_bit_cast(bf16x8, w);
+}
+
 template <bool RMS>
 __device__ __forceinline__ bf16x8 load_a(const void* a, int lda, int m, int k, bool ok, const void* gamma, int gamma_f32,
                                          float& ss) {
@@ -1204,9 +1213,22 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_skinny_kernel(const void* __r
         const int k = kbeg + (wave + WAVES * it) * 64 + q * 8;
 #pragma unroll
         for (int t = 0; t < MT; ++t) {
-          const int m = t * 16 + r;
-          const bf16x8 x0 = load_a<RMS>(a, lda, m, k, m < M && k < K, gamma, gamma_f32, ss[t]);
-          const bf16x8 x1 = load_a<RMS>(a, lda, m, k + 32, m < M && k + 32 < K, gamma, gamma_f32, ss[t]);
+          bf16x8 x0, x1;
+          if (RMS) {
+            const int m = t * 16 + r;
+            x0 = load_a<RMS>(a, lda, m, k, m < M && k < K, gamma, gamma_f32, ss[t]);
+            x1 = load_a<RMS>(a, lda, m, k + 32, m < M && k + 32 < K, gamma, gamma_f32, ss[t]);
+          } else {
+            // With several column blocks the rows of A are as much traffic from the cache as W is from memory, and the
+            // cache serves a wave's load faster when neighbouring lanes share a piece of 64 bytes than when each asks
+            // for 16 bytes of another row: lane 4R + Q loads piece Q of row R, and the operand's lane (row lane%16,
+            // piece lane/16) takes it from there through the LDS crossbar.
+            const int m = t * 16 + (lane >> 2), ka = k - q * 8 + (lane & 3) * 8;
+            const bf16x8 y0 = load_a<false>(a, lda, m, ka, m < M && ka < K, gamma, gamma_f32, ss[t]);
+            const bf16x8 y1 = load_a<false>(a, lda, m, ka + 32, m < M && ka + 32 < K, gamma, gamma_f32, ss[t]);
+            x0 = from_lane(y0, 4 * r + q);
+            x1 = from_lane(y1, 4 * r + q);
+          }
 #pragma unroll
           for (int rt = 0; rt < RT; ++rt) {
             acc[rt][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wf[rt][it][0], x0, acc[rt][t], 0, 0, 0);
