@@ -757,7 +757,9 @@ extern "C" int gb_attention_decode_bf16(const void* q, int q_stride, void* out, 
   // one workgroup per request and kv head (no chunks to combine afterwards) gets 16 waves, so that as
   // many loads are in flight as with four workgroups of four
   const int G = nh / nkv;
-  const int waves = (splits == 1 && 16 * (32 + (size_t)hd * G) * sizeof(float) <= 65536) ? 16 : 4;
+  // (not for contexts of up to 512 keys: half of the sixteen waves would find none, and four waves a workgroup put
+  // more workgroups on a compute unit: 32 requests of 512 tokens, SmolLM2-1.7B shapes, 32 -> 23 us a layer)
+  const int waves = (splits == 1 && max_context > 512 && 16 * (32 + (size_t)hd * G) * sizeof(float) <= 65536) ? 16 : 4;
   const size_t lds = (size_t)waves * (32 + (size_t)hd * G) * sizeof(float);
   const dim3 grid(splits, nkv, n_decode), block(waves * 64);
 #define GB_CASE(HD)                                                                                                         \

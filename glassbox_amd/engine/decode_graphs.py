@@ -11,7 +11,8 @@ A shape is (rows, context bucket).  The number of requests is rounded up to a fe
 the rows beyond the live requests are fillers: token 0 at position 0 of a request whose only page
 is the engine's spare page (never handed to a request) and whose state slot is the spare slot, so
 they cost almost nothing and touch nothing that a request holds.  The bucket is the longest
-context rounded up to 1,024 tokens: the attention kernel's split of the context is fixed at launch.
+context rounded up to 1,024 tokens (512 for the shortest: the attention kernel takes contexts that
+short with smaller workgroups): the attention kernel's split of the context is fixed at launch.
 
 The first step of a shape runs without a graph (kernels are loaded and buffers reach their sizes),
 the second is captured, later ones replay.  The model decides whether it can be replayed at all:
@@ -30,6 +31,11 @@ import torch
 from .context import StepContext, Workspace
 
 BUCKET = 1024
+SHORT = 512       # contexts up to here are a bucket of their own
+
+
+def context_bucket(longest: int) -> int:
+    return SHORT if longest <= SHORT else -(-longest // BUCKET) * BUCKET
 MAX_SHAPES = 64   # shapes kept (buffers and a graph each); the least recently used one goes first
 
 
@@ -131,7 +137,7 @@ class DecodeGraphs:
         n = len(entries)
         sids = [e[0] for e in entries]
         longest = cache.max_len(sids) + 1
-        key = (padded_rows(n), -(-longest // BUCKET) * BUCKET)
+        key = (padded_rows(n), context_bucket(longest))
         shape = self.shapes.get(key)
         if shape is None:
             if len(self.shapes) >= MAX_SHAPES:
