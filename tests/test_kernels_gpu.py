@@ -30,7 +30,9 @@ GEMM_SHAPES_BF16 = [(1, 32, 1), (8, 64, 2), (17, 64, 3), (33, 96, 9), (50, 160, 
                     # the tiled kernel over many k-steps, k a multiple of its step and not, one and two
                     # k-steps of prefetch (few and many tiles), fewer k-steps than the prefetch reaches
                     (512, 1024, 200), (2048, 2048, 130), (96, 8192, 70), (1536, 1088, 520), (200, 128, 66), (3000, 192, 300),
-                    (640, 1032, 257)]
+                    (640, 1032, 257),
+                    # a k of twelve to fifteen 64-wide blocks on sixteen waves (some of which find no block, or a part of one)
+                    (960, 960, 12), (2560, 960, 33), (1600, 776, 20), (5120, 1016, 64)]
 
 
 @pytest.mark.parametrize("N,K,M", GEMM_SHAPES_F32)
@@ -152,6 +154,7 @@ def test_gemm_bf16_fused_rms_norm(N, K, M, silu, gamma_dtype):
                                            # few, of 16 beyond), and takes the partial sums of up to 64 rows
                                            (12, 960, 2560, 2880, False), (40, 24704, 128, 512, False), (64, 352, 64, 176, True),
                                            (20, 4096, 1024, 1024, True), (9, 72, 264, 48, False), (17, 2048, 1024, 16384, True),
+                                           (20, 960, 960, 5120, True), (33, 960, 776, 1600, False),
                                            # at most 8 rows by so many rows of W that the folded kernel does not pay
                                            (5, 4096, 512, 256, False)])
 @pytest.mark.parametrize("gamma_dtype", [torch.float32, torch.bfloat16])
