@@ -361,12 +361,13 @@ def test_random_configurations(tmp_path, seed):
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
-@pytest.mark.parametrize("name,count", [("B", 12), ("E", 20), ("D", 40)])
+@pytest.mark.parametrize("name,count", [("B", 12), ("E", 20), ("D", 40), ("M", 33)])
 def test_many_requests_decode_together(model_dirs, bf16_bound, name, count, dtype):
     """Twelve, twenty and forty requests whose last 24 tokens are decoded in the same steps: steps of that many single
     tokens (in bfloat16 replayed from graphs, with filler rows up to the graph's size; the products of 9 to 64 rows
     prepare each other's norms), every position against the plain implementation.  Requests end at different steps, so
-    the batch shrinks through every size on the way."""
+    the batch shrinks through every size on the way.  Thirty-three requests on SmolLM2-360M's widths: a k of 960 on
+    sixteen waves, workgroups of 8 rows of W, short contexts that attention takes whole with four waves."""
     from glassbox_amd.engine import Engine
     folder = model_dirs.get(name)
     vocab = helpers.TINY[name]["vocab_size"]
