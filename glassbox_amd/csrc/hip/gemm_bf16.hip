@@ -319,8 +319,10 @@ int launch_tiled(const bf16* a, int lda, const bf16* w, int ldw, CT* c, int ldc,
   const int cols = EPI == EPI_SILU_MUL ? N / 2 : N, bn = EPI == EPI_SILU_MUL ? 64 : 64 * wn;
   // Tiles of 64 rows where those of 128 would leave a third of the compute units without a workgroup (the
   // products of a narrow model at some hundred rows): a workgroup's time is its k-steps' arithmetic, and half the
-  // rows halve it.
-  const bool low = M > 64 && ((cols + bn - 1) / bn) * ((M + 127) / 128) < 168;
+  // rows halve it.  A SiLU-multiply product, whose workgroups take 128 rows of W each, gains up to 300 workgroups
+  // (two of the smaller ones share a compute unit: gate/up of 256 rows on SmolLM2-1.7B shapes 34 -> 30 us, of 640 to
+  // 896 rows on SmolLM2-360M shapes 17 -> 14 and 24 -> 20 us; the other products lose from 168 on).
+  const bool low = M > 64 && ((cols + bn - 1) / bn) * ((M + 127) / 128) < (EPI == EPI_SILU_MUL ? 300 : 168);
   const int bm = low ? 64 : 128;
   const dim3 grid((cols + bn - 1) / bn, (M + bm - 1) / bm), block(256);
   GB_REQUIRE(grid.y <= 65535, "gemm_bf16: M=%d needs more than 65535 row tiles", M);
