@@ -632,7 +632,20 @@ constexpr int SBK = 64, SBM = 128, SA_STAGES = 6;
 // Measured on SmolLM2-1.7B shapes (each product alone, replayed from a graph): up to 64 rows the skinny kernel is as
 // fast or faster (it keeps A in registers); from about 200 rows on the wide tiles that divide k are (a workgroup here
 // reads two LDS operands for every MFMA); between, this kernel gains 10 to 25 %.
-constexpr int STREAM_MIN_ROWS = 64, STREAM_MAX_ROWS = 128;
+constexpr int STREAM_MAX_ROWS = 128;
+// Narrow tiles enough to fill the chip without dividing k.  (128 were taken for enough once: the 4,096 rows of W of a
+// Llama-3-8B projection then made 128 workgroups that walk all of k, and its O and down projections of 65 to 128 rows
+// took 29 and 81 us where the wide tiles with slices take 14 and 30.)
+constexpr int STREAM_FILLS = 192;
+// The fewest rows minus one that go to the stream kernel: 48 where it takes the product whole (gate/up of 64 rows:
+// SmolLM2-1.7B shapes 23.3 -> 22.0 us, Llama-3-8B shapes 82 -> 73; at 40 rows the wide tiles with slices are as fast or
+// faster), 32 where it divides k (the O projection of the 1.7B shapes at 40 to 64 rows 11.4 -> 9.6 us, the down projection
+// of the 360M shapes 11.1 -> 9.1).
+inline int stream_min_rows(int M, int N, int K, bool silu) {
+  const int tiles = ((N + 31) / 32) * ((M + 127) / 128);
+  const bool divides = tiles < STREAM_FILLS && K >= 1024 && K < 4096;  // as split_plan decides for the stream kernel's range
+  return divides ? 32 : silu ? 48 : 64;  // (other products it would take whole stay with the skinny kernel up to 64 rows)
+}
 constexpr int SLA = SBM / 8 / 4;  // a computing wave's load instructions per stage of A (an instruction moves 8 rows x 8 pieces)
 template <int TN> struct StreamShape {
   static constexpr int BN = 32 * TN, W_STAGES = TN == 1 ? 14 : 7, LW = BN / 8;  // LW: the loading wave's instructions per stage
@@ -841,7 +854,7 @@ struct SplitPlan {
   bool stream;    // the stream kernel's 128 x 32 tiles, if the operands allow (else the tiled kernel's, same slices)
 };
 
-inline SplitPlan split_plan(int M, int N, int K) {
+inline SplitPlan split_plan(int M, int N, int K, bool silu = false) {
   SplitPlan p{M <= 64 ? 64 : 128, 1, 0, 0, false, false};
   // many rows, a long k and few 256 x 256 tiles (the down projection of a prompt portion): slices of k fill the
   // chip with the ring kernel's tiles once; a slice keeps 1,024 of k or more
@@ -860,11 +873,11 @@ inline SplitPlan split_plan(int M, int N, int K) {
       p.slices = 1, p.k_slice = 0;
     }
   }
-  if (M > STREAM_MIN_ROWS && M <= STREAM_MAX_ROWS && K % SBK == 0 && N % 8 == 0) {
+  if (M > stream_min_rows(M, N, K, silu) && M <= STREAM_MAX_ROWS && K % SBK == 0 && N % 8 == 0) {
     // the stream kernel's range: its tiles are narrow, so only products with few rows of W divide k at all
     // (the O and down projections); a slice keeps 512 of k or more
     const int tiles = ((N + 31) / 32) * ((M + SBM - 1) / SBM);
-    if (tiles >= 128) return p;  // enough narrow tiles: no slices at all
+    if (tiles >= STREAM_FILLS) return p;  // enough narrow tiles: no slices at all
     if (K < 4096) {              // a long k (the down projection) is left to the wide tiles' slices below: measured faster
       int want = (256 + tiles - 1) / tiles;
       if (want > K / 512) want = K / 512;
@@ -1690,7 +1703,7 @@ extern "C" int gb_gemm_bf16(const void* a, int lda, const void* w, int ldw, void
   if (M == 0) return 0;
   const bf16* W = (const bf16*)w;
   if (split_ws != nullptr && M > 16 && !gamma && (!emit_h || emits == 2) && !parts) {  // more than the skinny kernels' best range
-    const SplitPlan plan = split_plan(M, N, K);
+    const SplitPlan plan = split_plan(M, N, K, epilogue == EPI_SILU_MUL);
     if (plan.slices > 1 && (epilogue != EPI_SILU_MUL || N % 16 == 0) && (uintptr_t)split_ws % 16 == 0) {
       GB_REQUIRE((long long)plan.floats <= split_ws_floats, "gemm_bf16: the split-k workspace holds %lld floats, %zu are needed",
                  split_ws_floats, plan.floats);
@@ -1711,7 +1724,7 @@ extern "C" int gb_gemm_bf16(const void* a, int lda, const void* w, int ldw, void
   const int narrow_tiles = ((ncols + 31) / 32) * ((M + SBM - 1) / SBM), wide_tiles = ((N + 127) / 128) * ((M + 127) / 128);
   const bool narrow_pays = M <= STREAM_MAX_ROWS ? narrow_tiles >= 64
                                                : (M <= 2 * STREAM_MAX_ROWS && epilogue == EPI_SILU_MUL && narrow_tiles >= 64 && wide_tiles < 128 && K < 2048);
-  if (M > STREAM_MIN_ROWS && narrow_pays && !gamma && !parts && !emit_h && stream_takes(a, lda, w, ldw, K) &&
+  if (M > stream_min_rows(M, N, K, epilogue == EPI_SILU_MUL) && narrow_pays && !gamma && !parts && !emit_h && stream_takes(a, lda, w, ldw, K) &&
       (epilogue != EPI_SILU_MUL || N % 16 == 0) && N < 32768) {
     const bf16* A = (const bf16*)a;
 #define GB_ST(EPI, CT) return launch_stream<EPI, CT>(A, lda, W, ldw, (CT*)c, ldc, M, N, K, 0, 1, stream)

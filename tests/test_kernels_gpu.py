@@ -227,6 +227,8 @@ def test_gemm_bf16_that_divides_k_does_the_next_norm(M, N, K, gamma_dtype):
 
 
 @pytest.mark.parametrize("M,N,K", [(17, 96, 4096), (33, 2048, 2048), (64, 2048, 8192), (100, 2048, 4160),
+                                   # 128 narrow tiles are not enough to go without slices (Llama-3-8B's O and down projections)
+                                   (96, 4096, 8192), (128, 4096, 4096),
                                    # a k that is no multiple of 64: the tiled kernel's slices
                                    (200, 528, 8200), (40, 1008, 4104),
                                    # a thousand rows and more: slices of k through the 256 x 256 tiles
@@ -264,9 +266,9 @@ def test_gemm_bf16_divides_k_over_workgroups(M, N, K, mode):
         ops.gemm(to_dev(a), to_dev(w), outs[0], accumulate=(mode == "f32+"), silu_mul=(mode == "silu"), workspace=ws[:8])
 
 
-@pytest.mark.parametrize("M,N,K", [(65, 6144, 2048), (128, 16384, 2048), (96, 4096, 8192),
+@pytest.mark.parametrize("M,N,K", [(65, 6144, 2048), (128, 16384, 2048), (96, 6144, 8192),
                                    # one, two, three k-steps: fewer than either ring is deep; and more than both
-                                   (100, 4096, 64), (128, 4128, 128), (100, 5000, 192), (70, 4100, 1024), (128, 8200, 1088),
+                                   (100, 4096, 64), (128, 4128, 128), (100, 5000, 192), (70, 6200, 1024), (128, 8200, 1088),
                                    # so many narrow tiles that a workgroup takes 64 columns
                                    (128, 24600, 320), (96, 32760, 512),
                                    # 33 to 64 rows by very many rows of W: the wide tiles, not the skinny kernel
