@@ -644,7 +644,9 @@ constexpr int STREAM_FILLS = 192;
 inline int stream_min_rows(int M, int N, int K, bool silu) {
   const int tiles = ((N + 31) / 32) * ((M + 127) / 128);
   const bool divides = tiles < STREAM_FILLS && K >= 1024 && K < 4096;  // as split_plan decides for the stream kernel's range
-  return divides ? 32 : silu ? 48 : 64;  // (other products it would take whole stay with the skinny kernel up to 64 rows)
+  // (other products it would take whole stay with the skinny kernel up to 64 rows, and so does a SiLU-multiply product
+  // whose narrow tiles do not fill the chip: SmolLM2-360M's gate/up of 49 to 64 rows 8.7 us there, 10.3 here)
+  return divides ? 32 : (silu && tiles >= 2 * STREAM_FILLS) ? 48 : 64;
 }
 constexpr int SLA = SBM / 8 / 4;  // a computing wave's load instructions per stage of A (an instruction moves 8 rows x 8 pieces)
 template <int TN> struct StreamShape {
@@ -1009,7 +1011,7 @@ inline bool fold_pays(int M, int N) { return M <= 8 && (N + 15) / 16 < 256; }
 inline int emit_mode(int M, int N, int K) {
   if (fold_pays(M, N)) return 1;
   if (M > 16 && N % 4 == 0 && N <= SPLIT_NORM_MAX && split_plan(M, N, K).slices > 1) return 2;
-  if (M <= 64 && !(M > 32 && N >= 32768)) return 1;  // the skinny kernel
+  if (M <= 64 && !(M > 16 && N >= 32768)) return 1;  // the skinny kernel
   return 0;
 }
 // Tiles of columns for which an emitting product of these sizes writes partial sums.
@@ -1735,9 +1737,10 @@ extern "C" int gb_gemm_bf16(const void* a, int lda, const void* w, int ldw, void
     GB_ST(EPI_STORE, bf16);
 #undef GB_ST
   }
-  // 33 to 64 rows by very many rows of W (the vocabulary product of a large decode batch): measured twice as fast
-  // through the tiles below as through the skinny kernel with four column blocks (49,152 x 2,048: 102 -> about 50 us)
-  const bool wide_head = M > 32 && N >= 32768 && !gamma && !parts;
+  // 17 to 64 rows by very many rows of W (the vocabulary product of a large decode batch): measured twice as fast
+  // through the tiles below as through the skinny kernel with four column blocks (49,152 x 2,048: 102 -> about 50 us),
+  // and with two column blocks as fast or faster (49,152 x 960 at 17 to 32 rows: 30 -> 25 us)
+  const bool wide_head = M > 16 && N >= 32768 && !gamma && !parts;
   if (M <= 64 && !wide_head) {
     const int gf = gamma_dtype == kF32;
     if (fold_pays(M, N) && epilogue != EPI_SILU_MUL && !parts) {
