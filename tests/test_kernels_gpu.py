@@ -271,8 +271,8 @@ def test_gemm_bf16_divides_k_over_workgroups(M, N, K, mode):
                                    (100, 4096, 64), (128, 4128, 128), (100, 5000, 192), (70, 6200, 1024), (128, 8200, 1088),
                                    # so many narrow tiles that a workgroup takes 64 columns
                                    (128, 24600, 320), (96, 32760, 512),
-                                   # 33 to 64 rows by very many rows of W: the wide tiles, not the skinny kernel
-                                   (64, 49152, 256), (40, 33000, 192),
+                                   # 17 to 64 rows by very many rows of W: the wide tiles, not the skinny kernel
+                                   (64, 49152, 256), (40, 33000, 192), (20, 40000, 192),
                                    # a narrow model's products: few narrow tiles and a k too short to divide; and up to
                                    # 256 rows (two row tiles) where the wide tiles would be fewer still
                                    (96, 2560, 960), (200, 5120, 960), (256, 2500, 448), (129, 2100, 128)])
