@@ -898,9 +898,13 @@ inline SplitPlan split_plan(int M, int N, int K, bool silu = false) {
   // skinny kernel is at its weakest (33 to 64 rows: every workgroup reads all of A) and where the tiles are
   // very few (the O projection of a portion of some hundred rows: 16 to 64 tiles)
   if (K < 4096 && !(M > 32 && M <= 64) && !(M > 64 && K >= 2048 && tiles <= 128)) return p;
-  // a slice keeps at least 8 k-steps (shorter ones cost more in partial sums than they gain)
+  // a slice keeps at least 8 k-steps (shorter ones cost more in partial sums than they gain), and of a long k, beyond
+  // 64 rows, 16 k-steps: a workgroup of 128 rows has more to do in a k-step, and the pass that adds the slices reads
+  // half as much (same box: the down projection of 256 rows on SmolLM2-1.7B shapes 26.7 -> 24.2 us, of 384 rows
+  // 36.0 -> 30.6; Llama-3-8B's QKV of 192 to 256 rows 36-38 -> 31, its O projection 25-26 -> 23-24)
   int want = (512 + tiles - 1) / tiles;
   want = want > 16 ? 16 : want;
+  if (M > 64 && K >= 4096 && want > K / (16 * TBK)) want = K / (16 * TBK);
   if (want > K / (8 * TBK)) want = K / (8 * TBK);
   if (want < 2) return p;
   p.k_slice = ((K + want - 1) / want + TBK - 1) / TBK * TBK;
