@@ -229,6 +229,8 @@ def test_gemm_bf16_that_divides_k_does_the_next_norm(M, N, K, gamma_dtype):
 @pytest.mark.parametrize("M,N,K", [(17, 96, 4096), (33, 2048, 2048), (64, 2048, 8192), (100, 2048, 4160),
                                    # 128 narrow tiles are not enough to go without slices (Llama-3-8B's O and down projections)
                                    (96, 4096, 8192), (128, 4096, 4096),
+                                   # beyond 64 rows a slice of a long k keeps 1,024 of it
+                                   (192, 2048, 4096), (256, 1024, 8192),
                                    # a k that is no multiple of 64: the tiled kernel's slices
                                    (200, 528, 8200), (40, 1008, 4104),
                                    # a thousand rows and more: slices of k through the 256 x 256 tiles
