@@ -86,7 +86,9 @@ def test_gemm_bf16_fused_silu_mul(I, K, M):
 
 
 @pytest.mark.parametrize("M,N,K", [(2100, 14000, 160), (1024, 28672, 128), (2048, 16384, 2048), (4000, 7200, 352),
-                                   (2049, 14080, 128 + 32), (2048, 6144, 128)])
+                                   (2049, 14080, 128 + 32), (2048, 6144, 128),
+                                   # 192 and 384 tiles, the last column tile partly outside
+                                   (2048, 6000, 192), (4096, 6096, 160)])
 @pytest.mark.parametrize("mode", ["bf16", "f32", "f32+", "silu"])
 def test_gemm_bf16_large_products_through_the_lds_ring(M, N, K, mode):
     """Products of a thousand rows and more with some hundred 256 x 256 tiles take the kernel whose operands go
