@@ -362,7 +362,12 @@ __global__ void rope_store_pieces_kernel(bf16* __restrict__ qkv, int row_stride,
                                          const float* __restrict__ sinv, const int32_t* __restrict__ slots,
                                          bf16* __restrict__ k_pages, bf16* __restrict__ v_pages, int nh, int nkv, int hd,
                                          int page_size, int rotate, int v_rows) {
-  rope_store_pieces(blockIdx.x, blockIdx.y * blockDim.x + threadIdx.x, qkv, row_stride, cosv, sinv, slots, k_pages, v_pages, nh,
+  // The chip deals workgroups round its 8 dies by their number, and each die has a second-level cache of its own: a
+  // die takes a run of neighbouring tokens, whose 16-byte pieces lie side by side in a key page, so that the cache
+  // writes back whole lines
+  int t = blockIdx.x;
+  if (gridDim.x % 8 == 0) t = (t % 8) * (gridDim.x / 8) + t / 8;
+  rope_store_pieces(t, blockIdx.y * blockDim.x + threadIdx.x, qkv, row_stride, cosv, sinv, slots, k_pages, v_pages, nh,
                     nkv, hd, page_size, rotate, v_rows);
 }
 
@@ -444,7 +449,9 @@ __global__ void rope_and_values_kernel(bf16* __restrict__ qkv, int row_stride, c
   extern __shared__ unsigned char tile_bytes[];
   const int b = blockIdx.x;
   if (b < rope_blocks) {
-    rope_store_pieces(b / rope_y, (b % rope_y) * blockDim.x + threadIdx.x, qkv, row_stride, cosv, sinv, slots, k_pages, v_pages,
+    // a die (workgroups b, b + 8, ...) takes a run of neighbouring tokens, as in the kernel above
+    const int r = rope_blocks % 8 == 0 ? (b % 8) * (rope_blocks / 8) + b / 8 : b;
+    rope_store_pieces(r / rope_y, (r % rope_y) * blockDim.x + threadIdx.x, qkv, row_stride, cosv, sinv, slots, k_pages, v_pages,
                       nh, nkv, hd, page_size, rotate, v_rows);
     return;
   }
