@@ -97,7 +97,7 @@ class _Shape:
         d_tables = [self.dev[t0 + g * rows * stride:t0 + (g + 1) * rows * stride].view(rows, stride) for g in range(G)]
         # what never changes between the steps of this shape.  First positions and state slots do change: they are
         # ``ctx.pos0`` and ``ctx.state_slots`` on the device, which is where a replayable part reads them
-        host = {"q_start": list(range(rows)), "q_len": [1] * rows, "n_decode": rows, "max_q_len": 1,
+        host = {"q_start": list(range(rows)), "q_len": [1] * rows, "n_decode": rows, "max_q_len": 1, "want_all": True,
                 "max_context": bucket, "graph": True, "pos0": None, "state_slots": None}
         self.ctx = StepContext(device=engine.device, dtype=engine.dtype, page_size=P, workspace=workspace, n=rows,
                                num_seqs=rows, token_ids=d[0], positions=d[1], tok_seq=d[2], slots=d_slots,

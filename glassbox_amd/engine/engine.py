@@ -317,7 +317,8 @@ class Engine:
         tables = [cut(o_rows + G * n + g * S * stride, S * stride).view(S, stride) for g in range(G)]
         n_decode = sum(1 for l in q_len if l == 1)
         host = {"q_start": q_start, "q_len": q_len, "pos0": pos0, "state_slots": state_slots, "n_decode": n_decode,
-                "max_q_len": max(q_len), "max_context": max(p + l for p, l in zip(pos0, q_len))}
+                "max_q_len": max(q_len), "max_context": max(p + l for p, l in zip(pos0, q_len)),
+                "want_all": want_rows == list(range(n))}
         return StepContext(device=self.device, dtype=self.dtype, page_size=P, workspace=self.workspace, n=n,
                            num_seqs=S, token_ids=cut(0, n), positions=cut(n, n), tok_seq=cut(2 * n, n), slots=slots,
                            tables=tables, q_start=cut(3 * n, S), q_len=cut(3 * n + S, S), pos0=cut(3 * n + 2 * S, S),

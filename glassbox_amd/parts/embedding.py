@@ -52,7 +52,10 @@ class LMHead(Part):
     def problems(self, dtype, page_size):
         return needs_multiple_of_8(dtype, "width", self.width)
 
-    def forward(self, ctx, rows):
+    accepts_prepared = True
+
+    def forward(self, ctx, rows, prepared=None):
+        """``prepared``: a PreNormed whose rows these are: the product scales its result by the norm's factor."""
         logits = ctx.buffer("logits", (rows.shape[0], self.vocab), torch.float32)
-        ops.gemm(rows, self.matrix(), logits)
+        ops.gemm(rows, self.matrix(), logits, rms_parts=prepared.as_gemm_arg() if prepared is not None else None)
         return logits

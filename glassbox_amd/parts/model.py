@@ -15,7 +15,7 @@ from typing import Dict, List, Optional, Sequence
 
 import torch
 
-from .base import CacheSpec, LayerCache, Norm, Part, StateSpec
+from .base import CacheSpec, LayerCache, Norm, Normed, Part, PreNormed, StateSpec
 from .embedding import Embedding, LMHead
 from .tape import LayerTapes
 
@@ -106,6 +106,9 @@ class DecoderModel(Part):
             if handover:
                 after = self.blocks[self.schedule[i + 1].block] if i + 1 < len(self.schedule) else None
                 more = {"pre": pre, "emit": after.entry_norm(ctx, ctx.n) if hasattr(after, "entry_norm") else None}
+                if after is None and self._head_takes_prepared(ctx):
+                    # the last block prepares the final norm as it would the next block's first
+                    more["emit"] = self.final_norm.emit_spec(ctx, ctx.n)
             if tapes is not None and self._taped[call.block]:
                 # the first layer of a kind walks through its parts and is recorded; the others are replayed
                 out = tapes.forward(i, block, x, cache, more)
@@ -114,8 +117,18 @@ class DecoderModel(Part):
             pre = out if handover else None
         if ctx.want.numel() == 0:
             return ctx.buffer("logits", (0, self.vocab_size), torch.float32)
+        if self._head_takes_prepared(ctx) and isinstance(pre, (PreNormed, Normed)):
+            return self.head.forward(ctx, pre.rows, prepared=pre if isinstance(pre, PreNormed) else None)
         rows = self.final_norm.forward(ctx, x, rows=ctx.want, out_name="h_out")
         return self.head.forward(ctx, rows)
+
+    HEAD_PREPARED_MAX_ROWS = 16   # beyond, the vocabulary product goes through tiles that take whole rows only
+
+    def _head_takes_prepared(self, ctx) -> bool:
+        """Whether the product that ends the last block may prepare the final norm for the vocabulary product: every
+        row's logits are wanted, in the rows' order (a step of single tokens), and the rows are few."""
+        return (bool(ctx.host.get("want_all")) and ctx.n <= self.HEAD_PREPARED_MAX_ROWS
+                and hasattr(self.final_norm, "emit_spec") and getattr(self.head, "accepts_prepared", False))
 
     def load_tree(self, tensors, prefix: str = "") -> None:
         super().load_tree(tensors, prefix)

@@ -439,6 +439,40 @@ def test_steps_of_single_tokens_replay_graphs_like_plain_steps(model_dirs, name,
         assert e.cache.used_pages() == 0
 
 
+@pytest.mark.parametrize("name", ["B", "M"])
+def test_single_token_steps_leave_the_final_norm_to_the_products(model_dirs, name, monkeypatch):
+    """In a bfloat16 step of a few single tokens, each wanting its logits, no norm runs as a kernel of its own: the
+    first is computed by the first product, the others are prepared by the product that makes the residual before
+    them, the final norm (crates/glassbox-core/src/model.rs:350-361) by the last block's, and the vocabulary
+    product scales by its factor.  A step that wants other rows, or more than sixteen, norms the wanted rows as
+    before; the logits are those of the plain kernels either way."""
+    from glassbox_amd import ops
+    from glassbox_amd.engine import Engine
+    folder = model_dirs.get(name)
+    vocab = helpers.TINY[name]["vocab_size"]
+    fused, plain_eng = (Engine(folder, dtype="bfloat16", max_tokens=2048, max_seqs=24, graph_decode=False, kernels=k)
+                        for k in ("auto", "plain"))
+    calls = []
+    real = ops.rmsnorm
+    monkeypatch.setattr(ops, "rmsnorm", lambda *a, **k: (calls.append(a[0].shape[0]), real(*a, **k))[1])
+
+    def step(entries):
+        calls.clear()
+        got = fused.step(entries).float().cpu()
+        n = len(calls)
+        want = plain_eng.step(entries).float().cpu()
+        assert (got - want).abs().max().item() <= 8e-3 * max(1.0, want.abs().max().item())
+        return n
+
+    prompts = {r: helpers.random_tokens(vocab, 20 + 3 * i, seed=80 + i) for i, r in enumerate("abcdefghijklmnopqr")}
+    assert step([(r, p, [len(p) - 1]) for r, p in prompts.items()]) >= 1          # portions: the wanted rows are normed
+    few = list(prompts)[:5]
+    assert step([(r, [9], [0]) for r in few]) == 0                                # five single tokens: no norm kernel
+    assert step([(r, [11], [0] if i else []) for i, r in enumerate(few)]) >= 1    # one of them wants nothing
+    assert step([(r, [12], [0]) for r in prompts]) >= 1                           # eighteen rows: beyond the limit
+    assert step([(few[0], [13], [0])]) == 0
+
+
 def test_decode_graph_shapes_are_kept_up_to_a_limit(model_dirs, monkeypatch):
     """Only so many shapes keep their buffers and graph; the least recently used one makes room, and a shape that
     comes back is warmed and captured again.  The logits stay those of an engine without graphs."""
