@@ -32,7 +32,10 @@ GB_DEFINE_LAST_ERROR
 namespace {
 
 __device__ __forceinline__ bf16x8 load8(const bf16* p) { return *reinterpret_cast<const bf16x8*>(p); }
+// read once and not again in this kernel: the caches need not keep it
+__device__ __forceinline__ bf16x8 load8_once(const bf16* p) { return __builtin_nontemporal_load(reinterpret_cast<const bf16x8*>(p)); }
 __device__ __forceinline__ bf16x4 load4(const bf16* p) { return *reinterpret_cast<const bf16x4*>(p); }
+__device__ __forceinline__ bf16x4 load4_once(const bf16* p) { return __builtin_nontemporal_load(reinterpret_cast<const bf16x4*>(p)); }
 __device__ __forceinline__ bf16x8 zero8() {
   bf16x8 z;
 #pragma unroll
@@ -81,11 +84,11 @@ __device__ __forceinline__ void attend64(Running<HD>& st, const bf16x8* qf, cons
 #pragma unroll
     for (int ks = 0; ks < KS; ++ks) {
       const int d0 = ks * 32 + c * 8;
-      kf[t][ks] = d0 < HD ? load8(kb + (size_t)(ks * 4 + c) * P * 8) : zero8();
+      kf[t][ks] = d0 < HD ? load8_once(kb + (size_t)(ks * 4 + c) * P * 8) : zero8();
     }
     const bf16* vb = vp + ((size_t)page * nkv + kvh) * HD * P + slot0 + 4 * c;
 #pragma unroll
-    for (int b = 0; b < DB; ++b) vf[b][t] = load4(vb + (size_t)(16 * b + j) * P);
+    for (int b = 0; b < DB; ++b) vf[b][t] = load4_once(vb + (size_t)(16 * b + j) * P);
   }
   float s[4][4];
   float mx = -INFINITY;
