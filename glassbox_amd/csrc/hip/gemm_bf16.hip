@@ -704,7 +704,7 @@ __global__ __launch_bounds__(320, 1) void gemm_stream_kernel(const bf16* __restr
     auto load_w = [&](int step) {
 #pragma unroll
       for (int t = 0; t < LW; ++t)
-        __builtin_amdgcn_global_load_lds((glb_void*)(wsrc[t] + k_of(step)), (lds_void*)&Ws[step % SW][t * 8 * SBK], 16, 0, 0);
+        __builtin_amdgcn_global_load_lds((glb_void*)(wsrc[t] + k_of(step)), (lds_void*)&Ws[step % SW][t * 8 * SBK], 16, 0, 2);  // nontemporal: W is read once, in whole 128-byte lines
     };
     for (int t = 0; t < DW && t < steps; ++t) load_w(t);
     // stage 0 has landed once at most the loads asked for after it are on their way
