@@ -60,6 +60,8 @@ def _host():
                                              [C.c_void_p, C.c_int, C.c_void_p, C.c_int]
         lib.gbh_cache_max_len.restype = C.c_int
         lib.gbh_cache_max_len.argtypes = [C.c_void_p, C.POINTER(C.c_int64), C.c_int]
+        lib.gbh_cache_max_pages.restype = C.c_int
+        lib.gbh_cache_max_pages.argtypes = [C.c_void_p, C.POINTER(C.c_int64), C.c_int]
         lib.gbh_cache_step_rows.restype = C.c_int
         lib.gbh_cache_step_rows.argtypes = [C.c_void_p, C.POINTER(C.c_int64), C.POINTER(C.c_int32), C.c_int, C.c_int] + \
                                            [C.c_void_p] * 5 + [C.c_void_p, C.c_int, C.c_void_p, C.c_int]
@@ -173,6 +175,15 @@ class CacheManager:
         """The longest of the requests' lengths."""
         ids = (C.c_int64 * max(1, len(seq_ids)))(*seq_ids)
         n = self._lib.gbh_cache_max_len(self._h, ids, len(seq_ids))
+        if n < 0:
+            raise CacheError("unknown request")
+        return n
+
+    def max_pages(self, seq_ids: Sequence[int]) -> int:
+        """The longest of the requests' block tables, in pages.  It can exceed what the lengths need: pages of a
+        reservation that was never committed stay with the request."""
+        ids = (C.c_int64 * max(1, len(seq_ids)))(*seq_ids)
+        n = self._lib.gbh_cache_max_pages(self._h, ids, len(seq_ids))
         if n < 0:
             raise CacheError("unknown request")
         return n

@@ -125,6 +125,8 @@ template <class T> inline T from_slot(unsigned long long v) {
   if constexpr (std::is_pointer_v<T>) {
     return reinterpret_cast<T>(static_cast<uintptr_t>(v));
   } else if constexpr (std::is_floating_point_v<T>) {
+    // a slot carries the 32 bits of a float: a parameter of more precision would be cut to float without a word
+    static_assert(std::is_same_v<T, float>, "a taped entry point takes its floating-point parameters as float");
     const uint32_t bits = static_cast<uint32_t>(v);
     float f;
     std::memcpy(&f, &bits, sizeof f);

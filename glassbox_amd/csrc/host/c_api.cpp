@@ -241,6 +241,17 @@ int gbh_cache_max_len(void* h, const int64_t* ids, int n) {
   }
   return longest;
 }
+// The longest block table among the requests, in pages, over all groups (-1 for an unknown request).  A request
+// may hold more pages than its length needs: a reservation that was never committed keeps them.
+int gbh_cache_max_pages(void* h, const int64_t* ids, int n) {
+  auto* cm = (CacheManager*)h;
+  int longest = 0;
+  for (int i = 0; i < n; ++i) {
+    if (cm->seq_len(ids[i]) < 0) return -1;
+    for (int g = 0; g < cm->num_groups(); ++g) longest = std::max(longest, (int)cm->table(ids[i], g)->size());
+  }
+  return longest;
+}
 // Sampling parameters of the j-th wanted row, with a uniform number drawn ahead from a copy of
 // the request's generator (the draw is kept only if the device reports more than one candidate).
 void gbh_sched_row_params(void* h, int j, float* temperature, int* top_k, float* top_p, float* min_p,

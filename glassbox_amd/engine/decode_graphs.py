@@ -118,6 +118,7 @@ class DecodeGraphs:
         self.workspace = Workspace(engine.device)
         self.shapes: "OrderedDict[Tuple[int, int], _Shape]" = OrderedDict()
         self.epoch = 0
+        self.loads = getattr(engine.model, "loads", 0)
         self.replays = 0
 
     def applies(self, entries: Sequence[Tuple[int, List[int], List[int]]]) -> bool:
@@ -136,7 +137,9 @@ class DecodeGraphs:
         cache = eng.cache
         n = len(entries)
         sids = [e[0] for e in entries]
-        longest = cache.max_len(sids) + 1
+        # the shape's tables must hold the longest table, which pages of an uncommitted reservation (a step that
+        # found no room for a later entry) can make longer than the lengths need
+        longest = max(cache.max_len(sids) + 1, cache.max_pages(sids) * eng.page_size)
         key = (padded_rows(n), context_bucket(longest))
         shape = self.shapes.get(key)
         if shape is None:
@@ -154,11 +157,15 @@ class DecodeGraphs:
                           shape.tables_ptr, shape.tables_gap)
         shape.dev.copy_(shape.host, non_blocking=True)
         shape.copied.record()
-        if self.workspace.epoch != self.epoch:
-            # a buffer was replaced by a larger one since graphs were captured: they hold the old address
+        loads = getattr(eng.model, "loads", 0)
+        if self.workspace.epoch != self.epoch or loads != self.loads:
+            # a buffer was replaced by a larger one, or the weights by another loading of them, since graphs were
+            # captured: they hold the old addresses
+            if any(s.graph is not None for s in self.shapes.values()):
+                torch.cuda.synchronize()     # a replay may still be running on what the dropped graphs hold
             for s in self.shapes.values():
                 s.graph, s.logits, s.runs = None, None, min(s.runs, 1)
-            self.epoch = self.workspace.epoch
+            self.epoch, self.loads = self.workspace.epoch, loads
         if shape.graph is not None:
             shape.graph.replay()
             self.replays += 1

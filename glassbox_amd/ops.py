@@ -208,6 +208,18 @@ class TapeOperands:
         self.bytes = (C.c_uint64 * max(1, n))(*sizes)
         self.count = n
         self.keep = list(tensors)
+        # pairs of ranges that overlap or coincide (a tensor that the layer holds in two places): a pointer into such a
+        # place has two ranges to be moved by
+        order = sorted((i for i in range(n) if sizes[i]), key=lambda i: ptrs[i])
+        self.overlaps = [(a, b) for k, a in enumerate(order) for b in order[k + 1:] if ptrs[b] < ptrs[a] + sizes[a]]
+
+    def maps_onto(self, target: "TapeOperands") -> bool:
+        """Whether every pointer into these tensors has one place in ``target``'s: ranges that overlap here must be
+        moved by the same distance (the runner takes the first range that holds a pointer)."""
+        for a, b in self.overlaps:
+            if target.ptrs[a] - self.ptrs[a] != target.ptrs[b] - self.ptrs[b]:
+                return False
+        return True
 
 
 def start_tape() -> LaunchTape:
@@ -226,7 +238,7 @@ def stop_tape() -> None:
 
 def run_tape(tape: LaunchTape, recorded: TapeOperands, target: TapeOperands) -> None:
     """Makes the recorded launches again with the tensors of ``recorded`` replaced, one for one, by those of ``target``."""
-    if not tape.usable or recorded.sizes != target.sizes:
+    if not tape.usable or recorded.sizes != target.sizes or not recorded.maps_onto(target):
         raise KernelError("run_tape: the layer's tensors do not match those of the recorded layer")
     rc = _host_lib().gbh_tape_run(tape.pointer(), len(tape), C.addressof(recorded.ptrs), C.addressof(recorded.bytes),
                                   C.addressof(target.ptrs), recorded.count)
@@ -424,6 +436,13 @@ def copy_rows(base: torch.Tensor, src: torch.Tensor, dst: torch.Tensor) -> None:
 
 # ------------------------------------------------------------------------ products
 FUSED_NORM_MAX_ROWS = 16   # measured: beyond one 16-row block the re-reading of float32 rows costs more than a norm pass
+HEAD_PREPARED_MAX_ROWS = 16   # beyond, the vocabulary product goes through tiles that take whole rows only
+
+
+def head_takes_parts(rows: int) -> bool:
+    """Whether a vocabulary product of ``rows`` rows can scale by the partial sums that the product before it left
+    (``gemm(..., rms_parts=)``) instead of reading rows that a norm kernel wrote."""
+    return rows <= HEAD_PREPARED_MAX_ROWS
 
 
 def parts_stride(rows: int) -> int:

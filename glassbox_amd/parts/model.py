@@ -15,6 +15,7 @@ from typing import Dict, List, Optional, Sequence
 
 import torch
 
+from .. import ops
 from .base import CacheSpec, LayerCache, Norm, Normed, Part, PreNormed, StateSpec
 from .embedding import Embedding, LMHead
 from .tape import LayerTapes
@@ -44,7 +45,7 @@ class DecoderModel(Part):
         self.width = embedding.width
         self._check_schedule()
         self._taped: Optional[List[bool]] = None       # which blocks let their launches be recorded (parts.tape)
-        self._loads = 0                                # times the weights were loaded: recorded tensors are theirs
+        self.loads = 0                                # times the weights were loaded: recorded tensors are theirs
 
     # structure ------------------------------------------------------------------
     def children(self) -> Dict[str, Part]:
@@ -91,7 +92,7 @@ class DecoderModel(Part):
             self._taped = [b.all_taped() for b in self.blocks]
         tapes = None
         if getattr(ctx, "layer_tapes", False) and any(self._taped):
-            tapes = LayerTapes(ctx, ctx.workspace.tape_sites, self._loads)
+            tapes = LayerTapes(ctx, ctx.workspace.tape_sites, self.loads)
         for i, call in enumerate(self.schedule):
             if call.cache is not None:
                 cache = caches[call.cache]
@@ -122,17 +123,15 @@ class DecoderModel(Part):
         rows = self.final_norm.forward(ctx, x, rows=ctx.want, out_name="h_out")
         return self.head.forward(ctx, rows)
 
-    HEAD_PREPARED_MAX_ROWS = 16   # beyond, the vocabulary product goes through tiles that take whole rows only
-
     def _head_takes_prepared(self, ctx) -> bool:
         """Whether the product that ends the last block may prepare the final norm for the vocabulary product: every
         row's logits are wanted, in the rows' order (a step of single tokens), and the rows are few."""
-        return (bool(ctx.host.get("want_all")) and ctx.n <= self.HEAD_PREPARED_MAX_ROWS
+        return (bool(ctx.host.get("want_all")) and ops.head_takes_parts(ctx.n)
                 and hasattr(self.final_norm, "emit_spec") and getattr(self.head, "accepts_prepared", False))
 
     def load_tree(self, tensors, prefix: str = "") -> None:
         super().load_tree(tensors, prefix)
-        self._loads += 1   # what engines keep of the layers' tensors (parts.tape) is of the weights before
+        self.loads += 1   # what engines keep of the layers' tensors (parts.tape) is of the weights before
 
     def streamed_matrices(self) -> List[torch.Tensor]:
         """Every tensor a step reads whole, once each: those of the scheduled blocks (a block named twice, or a

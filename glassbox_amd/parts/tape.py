@@ -14,7 +14,8 @@ What makes two layers of a kind is decided here, from the parts themselves, and 
   ``forward`` (``Part.taped``);
 * the blocks have one ``signature``: the same classes, arranged alike, with the same constants (every
   attribute that is a number, a string, a truth value or a tuple or list of such, but for those whose names begin
-  with an underscore);
+  with an underscore; an attribute of any other kind, tensors and parts aside, makes blocks differ unless they hold
+  the same object);
 * the walk of the recorded layer added nothing to the step's memo (``ctx.memo``: what a part computes once a step
   for all layers, like the rotation's table, is not among the launches of the layers after it);
 * they are called alike: what the block before prepared of the first norm, whether the block after asks for its
@@ -28,8 +29,10 @@ tables, sizes) is the same for both by the conditions above.
 """
 from __future__ import annotations
 
+import dataclasses
 from typing import Dict, List, Optional
 
+import numpy as np
 import torch
 
 from .. import ops
@@ -39,11 +42,21 @@ _SCALARS = (int, float, bool, str, type(None))
 
 
 def _constant(v):
-    """``v`` as part of a signature if it is a constant of the kinds that count, else None."""
+    """``v`` as part of a signature if it is a constant of a kind that can be compared by value (numbers, strings,
+    truth values; tuples, lists, mappings and dataclasses of such; arrays on the host), else None."""
     if isinstance(v, _SCALARS):
         return ("v", v)
-    if isinstance(v, (tuple, list)) and all(isinstance(e, _SCALARS) for e in v):
-        return ("l", tuple(v))
+    if isinstance(v, (tuple, list)):
+        inner = tuple(_constant(e) for e in v)
+        return None if any(c is None for c in inner) else ("l", inner)
+    if isinstance(v, dict):
+        inner = tuple((repr(k), _constant(e)) for k, e in v.items())
+        return None if any(c is None for _, c in inner) else ("m", inner)
+    if dataclasses.is_dataclass(v) and not isinstance(v, type):
+        inner = tuple((f.name, _constant(getattr(v, f.name))) for f in dataclasses.fields(v))
+        return None if any(c is None for _, c in inner) else ("d", type(v).__qualname__, inner)
+    if isinstance(v, np.ndarray):
+        return ("a", v.shape, str(v.dtype), v.tobytes())
     return None
 
 
@@ -61,10 +74,13 @@ def signature(part: Part, _seen: Optional[set] = None) -> tuple:
             items.append((name, signature(v, seen)))
         elif isinstance(v, (tuple, list)) and v and all(isinstance(e, Part) for e in v):
             items.append((name, tuple(signature(e, seen) for e in v)))
+        elif isinstance(v, torch.Tensor):
+            continue   # an operand: listed by ``tensors_of``, compared by size before each replay
         else:
             c = _constant(v)
-            if c is not None:
-                items.append((name, c))
+            # anything else (a mapping, a callable, an object of another kind) may decide what the part launches and
+            # cannot be compared here: it counts as a difference unless both blocks hold the very same object
+            items.append((name, c if c is not None else ("other", type(v).__qualname__, id(v))))
     return tuple(items)
 
 
@@ -189,10 +205,11 @@ class LayerTapes:
         rec = self.records.get(key)
         if rec is not None and rec.epoch == epoch:
             target = site.tensors()
-            if target.sizes == rec.operands.sizes:
+            if target.sizes == rec.operands.sizes and rec.operands.maps_onto(target):
                 ops.run_tape(rec.tape, rec.operands, target)
                 return rec.result
-            # a part of this layer has not yet made a tensor that the recorded layer's part made on its walk
+            # a part of this layer has not yet made a tensor that the recorded layer's part made on its walk, or a
+            # tensor that the recorded layer held in two places is two tensors here: the layer is walked
             result = block.forward(ctx, x, cache, **kwargs)
             site.forget()
             return result

@@ -364,3 +364,26 @@ def test_step_rows_fills_the_callers_arrays():
         cm.step_rows([5], [1], stride, *args(stride, tables)[3:])
     with pytest.raises(CacheError):   # two tokens where one is reserved
         cm.step_rows([7], [18], stride + 1, *args(stride, i32(2, S, stride + 1))[3:-1], S * (stride + 1))
+
+
+def test_a_table_can_be_longer_than_the_length_needs_and_max_pages_says_so():
+    """Pages of a reservation that is never committed stay with the request (a step whose later entry found no
+    room): 1,020 tokens hold 64 pages, ten more reserved make 65, and a single token reserved after that needs no
+    further page.  What sizes the tables of a replayed step must go by ``max_pages``, not by the lengths."""
+    cm = full(70, share=False)
+    cm.add_seq(1)
+    cm.reserve(1, 1020)
+    cm.commit(1, [3] * 1020)
+    cm.add_seq(2)
+    cm.reserve(2, 5)
+    assert cm.max_pages([1, 2]) == 64 and cm.max_len([1, 2]) == 1020
+    cm.reserve(1, 10)                       # never committed
+    assert cm.max_pages([1]) == 65 and cm.max_pages([2]) == 1 and cm.max_pages([2, 1]) == 65
+    cm.reserve(1, 1)
+    assert len(cm.table(1)) == 65 and cm.seq_len(1) == 1020
+    with pytest.raises(CacheError):
+        cm.max_pages([1, 99])
+    cm.check_invariants()
+    cm.remove_seq(1)
+    cm.remove_seq(2)
+    assert cm.used_pages() == 0

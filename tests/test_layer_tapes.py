@@ -125,6 +125,44 @@ def test_layers_are_of_a_kind_by_classes_and_constants():
     assert not d.all_taped()
 
 
+def test_an_attribute_that_cannot_be_compared_makes_blocks_differ():
+    """Constants are compared by value, also inside tuples, mappings and dataclasses; an attribute of a kind that
+    cannot be compared (a callable, an object) may decide what a part launches, so blocks holding different ones
+    are not of a kind, and blocks holding the same one are."""
+    a, b = block(), block()
+    a.ffn.table, b.ffn.table = {"k": (1, 2.0)}, {"k": (1, 2.0)}
+    assert layer_tape.signature(a) == layer_tape.signature(b)
+    b.ffn.table = {"k": (1, 2.5)}
+    assert layer_tape.signature(a) != layer_tape.signature(b)
+    b.ffn.table = {"k": (1, 2.0)}
+    a.ffn.rule, b.ffn.rule = (lambda n: n > 8), (lambda n: n > 16)
+    assert layer_tape.signature(a) != layer_tape.signature(b)
+    b.ffn.rule = a.ffn.rule
+    assert layer_tape.signature(a) == layer_tape.signature(b)
+
+
+def test_a_tensor_held_in_two_places_must_go_to_one_tensor():
+    """The runner moves a pointer by the first range that holds it.  A layer that holds one tensor in two places (a
+    block scheduled right after itself: its first norm's gamma is also the gamma it is asked to prepare) may only be
+    replayed for a layer whose two places hold one tensor too."""
+    g1, w1, g2, w2, g3 = (torch.zeros(16) for _ in range(5))
+    recorded = ops.TapeOperands([g1, w1, g1])
+    assert recorded.overlaps == [(0, 2)] or recorded.overlaps == [(2, 0)]
+    assert recorded.maps_onto(ops.TapeOperands([g2, w2, g2]))
+    assert not recorded.maps_onto(ops.TapeOperands([g2, w2, g3]))
+    assert ops.TapeOperands([g1, w1, g2]).overlaps == [] and ops.TapeOperands([g1, w1, g2]).maps_onto(ops.TapeOperands([g3, w2, g3]))
+    seen = []
+    lib, entry = fake_entry("fake_e", [C.c_void_p], seen)
+    tape = ops.LaunchTape()
+    tape.add(lib, entry, (g1.data_ptr(),))
+    with pytest.raises(ops.KernelError, match="do not match"):
+        ops.run_tape(tape, recorded, ops.TapeOperands([g2, w2, g3]))
+    assert not seen
+    # a view into a larger tensor beside the tensor itself overlaps it too
+    big = torch.zeros(64)
+    assert ops.TapeOperands([big, big[8:24]]).overlaps == [(0, 1)]
+
+
 def test_a_layers_tensors_come_in_one_order_and_include_cache_and_the_next_norm():
     a, b = block(), block()
     load_random(a)

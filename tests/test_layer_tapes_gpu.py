@@ -116,8 +116,26 @@ def test_layers_of_two_kinds_are_recorded_apart_and_a_block_named_twice_is_repla
             assert ops.TAPE_COUNTS["replayed_layers"] - before["replayed_layers"] >= 5 * eng.steps
     for r in requests:
         assert np.array_equal(got[True][r], got[False][r]), f"request {r}: replayed layers changed the logits"
-    # and the windowed layers did matter: the same model without windows says something else
     assert len(eng.group_keys) == 2
+    # both against the plain parts wired by the same schedule (a mistake that both runs share would pass the
+    # comparison above), and the windows did matter: the plain model without them says something else
+    from plain import llama as plain
+    cfg, w = plain.load_folder(folder)
+    w = {k: v.double() for k, v in w.items()}
+
+    def plain_two_kinds(tokens, windows=True):
+        positions = list(range(len(tokens)))
+        x = w["model.embed_tokens.weight"][torch.tensor(tokens, dtype=torch.long)]
+        for block in (0, 1, 2, 3, 4, 5, 0, 1):
+            x = plain.decoder_layer(x, w, f"model.layers.{block}.", cfg, positions, window=7 if windows and block % 2 else 0)
+        return (plain.rms_norm(x, w["model.norm.weight"], cfg["rms_norm_eps"]) @ w["model.embed_tokens.weight"].T).numpy()
+
+    for r, toks in requests.items():
+        want = plain_two_kinds(toks)
+        bad = helpers.first_bad(got[True][r], want, helpers.TOL_F32)
+        assert bad is None, f"request {r} ({len(toks)} tokens): first wrong position {bad[0]}, error {bad[1]:.3e}"
+    longest = requests["r2"]
+    assert np.abs(plain_two_kinds(longest) - plain_two_kinds(longest, windows=False))[8:].max() > 1e-3
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])

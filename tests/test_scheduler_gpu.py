@@ -17,9 +17,12 @@ from plain import sampler as psampler
 pytestmark = pytest.mark.gpu
 
 
-def serve(eng, prompts, max_tokens, samplers=None, budget=16, max_seqs=4, abort_every=0):
+def serve(eng, prompts, max_tokens, samplers=None, budget=16, max_seqs=4, abort_every=0, abort_seed=0, max_aborts=7):
     """Runs the prompts through a scheduler and records, for every step, which request brought which positions and
-    the logits that came back.  Returns (replies, scheduler, records); a record is (request index, position, row)."""
+    the logits that came back.  Returns (replies, scheduler, records); a record is (request index, position, row).
+    ``abort_every``: after every so many steps one live request, drawn at random, is aborted (up to ``max_aborts``),
+    the cache's invariants are checked after every step, and ``scheduler.aborted`` counts the aborted requests that
+    were running and that were waiting (crates/glassbox-server/tests/scheduler.rs:142-151)."""
     from glassbox_amd.engine import Scheduler, SchedulerConfig
     from glassbox_amd.sampling import SamplerConfig
     sched = Scheduler(eng, SchedulerConfig(token_budget=budget, max_seqs=max_seqs))
@@ -41,12 +44,22 @@ def serve(eng, prompts, max_tokens, samplers=None, budget=16, max_seqs=4, abort_
         return logits
 
     eng.run_reserved = spy
+    rng = random.Random(abort_seed)
+    sched.aborted = {"running": 0, "waiting": 0}
     try:
         guard = 0
         while not sched.is_idle():
             sched.step()
             guard += 1
             assert guard < 100000
+            if abort_every:
+                eng.cache.check_invariants()
+                live = [rid for rid in ids if sched.outputs[rid].finish is None]
+                if guard % abort_every == 0 and live and sum(sched.aborted.values()) < max_aborts:
+                    before = sched.running()
+                    sched.abort(rng.choice(live))
+                    sched.aborted["running" if sched.running() < before else "waiting"] += 1
+                    eng.cache.check_invariants()
     finally:
         del eng.run_reserved
     return [sched.outputs[i].tokens for i in ids], sched, records
