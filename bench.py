@@ -9,7 +9,8 @@ replays steps of single tokens from HIP graphs) and the device sampler (``sampli
 tokens fed back as the next step's input.  The batch is first prefilled (through the same step function, in
 portions of 2,048 tokens) so that the last timed step reaches the context length.  K steps are timed ``--reps``
 times in a row, each time between synchronisations; ``ms_per_step`` and ``value`` are the mean over the
-repetitions and ``reps`` holds their spread.  ``points.decode_b<batch>_scheduler`` is the same workload as
+repetitions and ``reps`` holds their spread; the batch 1 and 64 points are repeated as often, with their spread
+beside them (``points.decode_b1_sd``).  ``points.decode_b<batch>_scheduler`` is the same workload as
 requests under ``Scheduler.step`` (plan, step, sample, finish).  Prints one JSON line.  One GPU only: for
 --gpus > 1 it says so and exits with 2.
 """
@@ -18,7 +19,6 @@ import datetime
 import json
 import os
 import statistics
-import subprocess
 import sys
 import time
 
@@ -210,16 +210,13 @@ def main() -> int:
                 points[f"decode_b{b}"] = round(value, 1)
                 continue
             k = max(8, min(a.steps, 32))
-            pts, _ = decode_run(b, k, min(a.warmup, 4), 1)
-            points[f"decode_b{b}"] = round(b * k / pts[0], 1)
+            pts, _ = decode_run(b, k, min(a.warmup, 4), a.reps)
+            rates = [b * k / t for t in pts]
+            points[f"decode_b{b}"] = round(statistics.mean(rates), 1)
+            points[f"decode_b{b}_sd"] = round(statistics.stdev(rates), 1) if len(rates) > 1 else 0.0
+            points[f"decode_b{b}_reps"] = len(rates)
 
-    def commit():
-        here = os.path.dirname(os.path.abspath(__file__))
-        try:
-            r = subprocess.run(["git", "-C", here, "rev-parse", "--short", "HEAD"], capture_output=True, text=True, timeout=10)
-            return r.stdout.strip() or None
-        except (OSError, subprocess.SubprocessError):
-            return None
+    from glassbox_amd.build import source_version
     ms = [t / a.steps * 1e3 for t in times]
 
     out = {
@@ -237,7 +234,7 @@ def main() -> int:
                    "graph": eng.decode_graphs is not None},
         "reps": {"n": a.reps, "ms_per_step": [round(m, 4) for m in ms], "mean_ms": round(statistics.mean(ms), 4),
                  "sd_ms": round(statistics.stdev(ms), 4) if len(ms) > 1 else 0.0},
-        "meta": {"gpu": torch.cuda.get_device_name(0), "commit": commit(),
+        "meta": {"gpu": torch.cuda.get_device_name(0), "commit": source_version(),
                  "date": datetime.datetime.now(datetime.timezone.utc).strftime("%Y-%m-%dT%H:%M:%SZ"),
                  "torch": torch.__version__, "path": "Engine.step + sampling.sample_rows"},
         "prefill": prefill,

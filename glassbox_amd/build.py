@@ -181,6 +181,53 @@ def build_all(force: bool = True, names: Optional[List[str]] = None, jobs: int =
         return
     with ThreadPoolExecutor(max_workers=max(1, min(jobs, len(todo)))) as pool:
         list(pool.map(compile_library, todo))
+    _stamp_version()
+
+
+def _git_commit() -> Optional[str]:
+    """The checkout's commit (short, with ``+`` if tracked files differ from it), or None where there is no git."""
+    root = os.path.dirname(_HERE)
+    try:
+        r = subprocess.run(["git", "-C", root, "rev-parse", "--short", "HEAD"], capture_output=True, text=True, timeout=10)
+        if r.returncode != 0 or not r.stdout.strip():
+            return None
+        d = subprocess.run(["git", "-C", root, "status", "--porcelain", "--untracked-files=no"], capture_output=True,
+                           text=True, timeout=10)
+        return r.stdout.strip() + ("+" if d.returncode == 0 and d.stdout.strip() else "")
+    except (OSError, subprocess.SubprocessError):
+        return None
+
+
+def _stamp_version() -> None:
+    """Notes the commit beside the built libraries, which travel to machines where the sources are no checkout."""
+    commit = _git_commit()
+    if commit:
+        try:
+            with open(os.path.join(_lib_dir(), "commit.stamp"), "w") as fh:
+                fh.write(commit)
+        except OSError:
+            pass
+
+
+def source_version() -> str:
+    """What a measurement names as the code it ran: the commit of the checkout; where there is none, ``$GLASSBOX_COMMIT``
+    or the commit noted when the libraries were built (``built@...``: the tree may have moved on since); failing
+    that, a hash of the native sources (``src-...``)."""
+    commit = _git_commit() or os.environ.get("GLASSBOX_COMMIT")
+    if commit:
+        return commit
+    for d in (os.path.join(_HERE, "_lib"), _lib_dir()):
+        try:
+            with open(os.path.join(d, "commit.stamp")) as fh:
+                noted = fh.read().strip()
+            if noted:
+                return "built@" + noted
+        except OSError:
+            pass
+    h = hashlib.sha256()
+    for name in sorted(LIBRARIES):
+        h.update(_digest(name).encode())
+    return "src-" + h.hexdigest()[:12]
 
 
 def load(name: str) -> ctypes.CDLL:

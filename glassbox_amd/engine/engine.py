@@ -42,12 +42,37 @@ def check_supported(model, dtype: torch.dtype, page_size: int) -> None:
         raise EngineError(f"this model cannot run in {name} with pages of {page_size}:\n  " + "\n  ".join(lines))
 
 
+def sharing_obstacles(model) -> List[str]:
+    """Why requests with the same beginning cannot share its pages in this model, one line per reason (empty if they
+    can).  Sharing hands a new request the pages that another wrote and skips those tokens, in every layer at once,
+    so every cache layer must still hold them and must need nothing else to go on from there."""
+    windows: Dict[int, List[int]] = {}
+    stateful: List[int] = []
+    for c, (spec, state) in enumerate(zip(model.cache_specs(), model.state_specs())):
+        if spec is not None and spec.kind != FULL:
+            windows.setdefault(spec.window, []).append(c)
+        if state is not None:
+            stateful.append(c)
+    lines = []
+    several = lambda cs: ("cache layers " if len(cs) > 1 else "cache layer ") + ", ".join(map(str, cs))
+    for window, cs in sorted(windows.items()):
+        lines.append(f"{several(cs)}: a window of {window} positions, whose pages are given back as soon as the window "
+                     f"has passed them, so that a later request does not find them")
+    if stateful:
+        lines.append(f"{several(stateful)}: state of its own for each request, which a request that skips tokens would "
+                     f"need as it was at the edge of the last shared page")
+    return lines
+
+
 class Engine:
     """model: a folder (config.json + model.safetensors) or a built and loaded model.
 
     max_tokens: tokens the cache holds over all live requests (rounded up to whole pages).
     max_seqs: most live requests (= state slots).  page_size: tokens per page (16 as in the
     reference, crates/glassbox-core/src/kv.rs:11).
+    prefix_caching: requests whose prompts begin alike share the pages of the beginning (kv.rs:135-157).  A model
+    with a windowed or stateful layer cannot (``sharing_obstacles``); asking for it there is an error that says why,
+    not a silent "off".
     graph_decode: replay steps of one token per request from HIP graphs (engine.decode_graphs); by
     default where the arithmetic is bfloat16 and every part of the model allows it.
     kernels: "auto", or "plain": every part takes its plain kernels, one per operation and nothing fused, which
@@ -89,8 +114,13 @@ class Engine:
         self.group_keys = keys
         self.has_state = any(s is not None for s in states)
         groups = [GroupSpec(kind, window, num_pages) for kind, window in keys]
-        share = prefix_caching and not self.has_state and all(kind == FULL for kind, _ in keys)
-        self.cache = CacheManager(self.page_size, groups, self.max_seqs, share)
+        if prefix_caching:
+            obstacles = sharing_obstacles(model)
+            if obstacles:
+                raise EngineError("prefix_caching=True: this model's requests cannot share the pages of a common "
+                                  "beginning (build the engine with prefix_caching=False, on the command line "
+                                  "--no-prefix-cache):\n  " + "\n  ".join(obstacles))
+        self.cache = CacheManager(self.page_size, groups, self.max_seqs, bool(prefix_caching))
 
         self.layers: List[LayerCache] = []
         for spec, state in zip(specs, states):

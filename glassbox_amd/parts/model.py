@@ -33,8 +33,12 @@ class DecoderModel(Part):
 
     def __init__(self, config, embedding: Embedding, blocks: Sequence[Part], schedule: Sequence[LayerCall],
                  final_norm: Norm, head: LMHead, names=("model.embed_tokens", "model.layers.{}", "model.norm", "lm_head"),
-                 ignorable: Sequence[str] = (), arg_keys: Optional[Dict[str, str]] = None):
+                 ignorable: Sequence[str] = (), arg_keys: Optional[Dict[str, str]] = None, sources=None):
         self.config = config
+        #: where the checkpoint keeps a tensor that it names or cuts otherwise than the parts do: a mapping, or a
+        #: function, from the model's tensor name to the checkpoint's name or to (name, first row, last row) of a
+        #: tensor that holds several stacked by rows; None for a tensor of the same name (weights.loader)
+        self.sources = sources
         #: constructor argument of a part -> the key of config.json that set it, for messages
         self.arg_keys = dict(arg_keys or {})
         self.embedding, self.blocks, self.schedule = embedding, list(blocks), list(schedule)
@@ -55,6 +59,11 @@ class DecoderModel(Part):
         out[self.names[2]] = self.final_norm
         out[self.names[3]] = self.head
         return out
+
+    def source_of(self, name: str):
+        if self.sources is None:
+            return None
+        return self.sources(name) if callable(self.sources) else self.sources.get(name)
 
     def _check_schedule(self) -> None:
         owners: Dict[int, int] = {}

@@ -6,6 +6,12 @@ missing tensor, every unexpected one and every wrong shape.  Tensor names and
 the single-file layout follow the reference
 (crates/glassbox-core/src/load.rs:34-96), which checks none of this.
 
+A checkpoint need not name or cut its tensors as the parts do: a model may say where each of its
+tensors comes from (``DecoderModel(sources=...)``: another name, or a range of the rows of a tensor
+that holds several stacked), so that the stock parts load a file with fused or renamed projections
+without a subclass.  The reference has neither renaming nor splitting (load.rs:52-67 reads the
+parts' own names); the error still speaks of the file's names.
+
 Types on the device: matrices follow the compute type (bfloat16 stays
 bfloat16; the 32-bit path converts everything to float32); vectors stored in
 32-bit stay 32-bit in the bfloat16 path; integer tables become int32.
@@ -13,7 +19,7 @@ bfloat16; the 32-bit path converts everything to float32); vectors stored in
 from __future__ import annotations
 
 import os
-from typing import Dict, Optional
+from typing import Dict, List, NamedTuple, Optional, Tuple
 
 import torch
 
@@ -63,17 +69,72 @@ def load_model(folder: str, dtype="bfloat16", device="cuda:0"):
     return model
 
 
+class Source(NamedTuple):
+    """Where a tensor of the model lies in the checkpoint: the whole tensor ``name``, or its rows
+    ``first`` .. ``last - 1`` (a tensor that holds several of the model's stacked by rows)."""
+    name: str
+    first: Optional[int] = None
+    last: Optional[int] = None
+
+
+def source_of(model, name: str) -> Source:
+    """The checkpoint's place for the model's tensor ``name``: what the model says (``source_of``), else the
+    tensor of the same name."""
+    ask = getattr(model, "source_of", None)
+    src = ask(name) if ask is not None else None
+    if src is None:
+        return Source(name)
+    if isinstance(src, str):
+        return Source(src)
+    src = Source(*src)
+    if (src.first is None) != (src.last is None) or (src.first is not None and not 0 <= src.first < src.last):
+        raise WeightError(f"{name}: {tuple(src)} is no range of rows")
+    return src
+
+
+def checkpoint_layout(model) -> Tuple[Dict[str, Source], Dict[str, Tuple[int, ...]]]:
+    """(model tensor -> its source, checkpoint tensor -> the shape the model's tensors give it).  A checkpoint tensor
+    that is cut by rows must be covered by its parts exactly: from row 0, without gaps or overlaps."""
+    specs: Dict[str, TensorSpec] = dict(model.named_specs())
+    sources = {name: source_of(model, name) for name in specs}
+    shapes: Dict[str, Tuple[int, ...]] = {}
+    cuts: Dict[str, List[Tuple[int, int, str]]] = {}
+    for name, src in sources.items():
+        shape = tuple(specs[name].shape)
+        if src.first is None:
+            if src.name in shapes or src.name in cuts:
+                raise WeightError(f"{src.name} is the source of more than one tensor of the model")
+            shapes[src.name] = shape
+        else:
+            if src.name in shapes:
+                raise WeightError(f"{src.name} is the source of more than one tensor of the model")
+            if not shape or shape[0] != src.last - src.first:
+                raise WeightError(f"{name} has {shape[0] if shape else 0} rows, its source names rows {src.first} to {src.last}")
+            cuts.setdefault(src.name, []).append((src.first, src.last, name))
+    for ckpt, parts in cuts.items():
+        parts.sort()
+        at, rest = 0, None
+        for first, last, name in parts:
+            r = tuple(specs[name].shape[1:])
+            if first != at or (rest is not None and r != rest):
+                raise WeightError(f"{ckpt}: the model's tensors do not cover its rows one after the other "
+                                  f"({name} takes rows {first} to {last})")
+            at, rest = last, r
+        shapes[ckpt] = (at,) + rest
+    return sources, shapes
+
+
 def load_weights(model, path: str, dtype: torch.dtype, device) -> None:
     try:
         f = SafetensorsFile(path)
     except ValueError as e:
         raise WeightError(str(e)) from None
     expected: Dict[str, TensorSpec] = dict(model.named_specs())
+    sources, shapes = checkpoint_layout(model)
     have = set(f.names())
-    missing = sorted(n for n in expected if n not in have)
-    unexpected = sorted(n for n in have if n not in expected and n not in getattr(model, "ignorable", ()))
-    wrong = sorted((n, f.shape(n), expected[n].shape) for n in expected
-                   if n in have and tuple(f.shape(n)) != tuple(expected[n].shape))
+    missing = sorted(n for n in shapes if n not in have)
+    unexpected = sorted(n for n in have if n not in shapes and n not in getattr(model, "ignorable", ()))
+    wrong = sorted((n, f.shape(n), shapes[n]) for n in shapes if n in have and tuple(f.shape(n)) != shapes[n])
     if missing or unexpected or wrong:
         lines = [f"{path} does not fit the model {type(model.config).__name__}:"]
         if missing:
@@ -86,10 +147,29 @@ def load_weights(model, path: str, dtype: torch.dtype, device) -> None:
         raise WeightError("\n".join(lines))
     tensors = {}
     for name, spec in expected.items():
-        host = f.tensor(name)
+        src = sources[name]
+        host = f.tensor(src.name)
+        if src.first is not None:
+            host = host[src.first:src.last]
         tensors[name] = host.to(device=device, dtype=target_dtype(spec, host.dtype, dtype))
     model.load_tree(tensors)
     f.close()
+
+
+def checkpoint_tensors(model, tensors: Dict[str, torch.Tensor]) -> Dict[str, torch.Tensor]:
+    """The model's tensors, by its own names, as the checkpoint lays them out (renamed, stacked by rows)."""
+    sources, shapes = checkpoint_layout(model)
+    out: Dict[str, torch.Tensor] = {}
+    for name, t in tensors.items():
+        src = sources[name]
+        if src.first is None:
+            out[src.name] = t
+        else:
+            whole = out.get(src.name)
+            if whole is None:
+                whole = out[src.name] = torch.empty(shapes[src.name], dtype=t.dtype, device=t.device)
+            whole[src.first:src.last] = t
+    return out
 
 
 def random_tensors(model, seed: int, std: float = 0.02, norm_init: str = "ones",
@@ -121,7 +201,8 @@ def write_random_model(config: ModelConfig, folder: str, seed: int, std: float =
     os.makedirs(folder, exist_ok=True)
     model = build_model(config)
     config.save(folder)
-    save_file(random_tensors(model, seed, std, norm_init, dtype), os.path.join(folder, "model.safetensors"))
+    save_file(checkpoint_tensors(model, random_tensors(model, seed, std, norm_init, dtype)),
+              os.path.join(folder, "model.safetensors"))
     return folder
 
 

@@ -36,3 +36,14 @@ def bf16_bound():
     """The tolerance of bfloat16 engines with tuned kernels: see helpers.Bf16Bound."""
     import helpers
     return helpers.Bf16Bound()
+
+
+def pytest_terminal_summary(terminalreporter):
+    """The plain kernels' bfloat16 errors that this run measured, beside the recorded figures they are held to."""
+    import helpers
+    if not helpers.MEASURED_PLAIN_BF16_REL:
+        return
+    terminalreporter.write_line("plain kernels in bfloat16, largest error relative to the largest logit (measured / recorded):")
+    for label, rel in sorted(helpers.MEASURED_PLAIN_BF16_REL.items()):
+        rec = helpers.PLAIN_BF16_REL.get(label)
+        terminalreporter.write_line(f"  {label}: {rel:.3e} / {'-' if rec is None else format(rec, '.3e')}")

@@ -239,3 +239,168 @@ def test_the_bytes_of_a_decode_step_are_the_matrices_each_part_names():
         per_layer = d * (cfg.q_dim + 2 * cfg.kv_dim) + cfg.q_dim * d + 3 * I * d
         assert model.weight_bytes() == 4 * (L * per_layer + V * d)
         assert len(model.streamed_matrices()) == 4 * L + 1
+
+
+# --------------------------------------------- a checkpoint that names and cuts its tensors otherwise than the parts do
+def register_fused_toy():
+    """An architecture, defined here, whose checkpoints keep query, key and value rows in one ``qkv_proj`` tensor,
+    gate and up rows in one ``gate_up_proj``, and call the norms otherwise: built from the stock parts, with nothing
+    but a function from the parts' tensor names to the checkpoint's."""
+    import re
+    from glassbox_amd.config import LlamaConfig, register_architecture
+    from glassbox_amd.parts.attention import PagedAttention
+    from glassbox_amd.parts.block import PreNormBlock
+    from glassbox_amd.parts.embedding import Embedding, LMHead
+    from glassbox_amd.parts.mlp import SwiGLU
+    from glassbox_amd.parts.model import DecoderModel, LayerCall
+    from glassbox_amd.parts.norm import RMSNorm
+    from glassbox_amd.parts.rotary import Rotary
+
+    class FusedToyConfig(LlamaConfig):
+        architecture = "FusedToyForCausalLM"
+
+    def build(cfg):
+        d, hd, q, kv, inter = cfg.hidden_size, cfg.head_size, cfg.q_dim, cfg.kv_dim, cfg.intermediate_size
+        rotary = Rotary(hd, cfg.rope_theta)
+        blocks = [PreNormBlock(RMSNorm(d, cfg.rms_norm_eps),
+                               PagedAttention(d, cfg.num_attention_heads, cfg.num_key_value_heads, hd, rotary),
+                               RMSNorm(d, cfg.rms_norm_eps), SwiGLU(d, inter)) for _ in range(cfg.num_hidden_layers)]
+        rows = {"self_attn.q_proj": ("self_attn.qkv_proj", 0, q), "self_attn.k_proj": ("self_attn.qkv_proj", q, q + kv),
+                "self_attn.v_proj": ("self_attn.qkv_proj", q + kv, q + 2 * kv),
+                "mlp.gate_proj": ("mlp.gate_up_proj", 0, inter), "mlp.up_proj": ("mlp.gate_up_proj", inter, 2 * inter)}
+        renamed = {"input_layernorm": "ln_1", "post_attention_layernorm": "ln_2"}
+
+        def sources(name):
+            if name == "model.norm.weight":
+                return "model.final_layernorm.weight"
+            m = re.fullmatch(r"(model\.layers\.\d+\.)(.+)\.weight", name)
+            if m and m.group(2) in rows:
+                fused, first, last = rows[m.group(2)]
+                return (f"{m.group(1)}{fused}.weight", first, last)
+            if m and m.group(2) in renamed:
+                return f"{m.group(1)}{renamed[m.group(2)]}.weight"
+            return None
+
+        emb = Embedding(cfg.vocab_size, d)
+        return DecoderModel(cfg, emb, blocks, [LayerCall(i, cache=i) for i in range(cfg.num_hidden_layers)],
+                            RMSNorm(d, cfg.rms_norm_eps), LMHead(cfg.vocab_size, d, tied_to=None), sources=sources)
+
+    register_architecture("FusedToyForCausalLM", FusedToyConfig, build)
+    return dict(helpers.TINY_B, architectures=["FusedToyForCausalLM"])
+
+
+def plain_names(tensors):
+    """A fused toy's checkpoint under the names and cuts of the plain implementation (sizes of the second tiny
+    configuration: 96 query rows, 32 key and 32 value rows, 256 gate and 256 up rows)."""
+    out = {}
+    for n, t in tensors.items():
+        n = n.replace("ln_1", "input_layernorm").replace("ln_2", "post_attention_layernorm").replace("final_layernorm", "norm")
+        if "qkv_proj" in n:
+            for part, a, b in (("q", 0, 96), ("k", 96, 128), ("v", 128, 160)):
+                out[n.replace("qkv_proj", part + "_proj")] = t[a:b]
+        elif "gate_up_proj" in n:
+            out[n.replace("gate_up_proj", "gate_proj")], out[n.replace("gate_up_proj", "up_proj")] = t[:256], t[256:]
+        else:
+            out[n] = t
+    return out
+
+
+def test_the_stock_parts_load_a_checkpoint_with_fused_and_renamed_tensors(tmp_path):
+    raw = register_fused_toy()
+    cfg = config_from_dict(raw)
+    folder = write_random_model(cfg, str(tmp_path / "fused"), seed=5, norm_init="uniform")
+    f = SafetensorsFile(os.path.join(folder, "model.safetensors"))
+    names = set(f.names())
+    assert "model.layers.0.self_attn.qkv_proj.weight" in names and "model.layers.2.mlp.gate_up_proj.weight" in names
+    assert "model.layers.1.ln_1.weight" in names and "model.final_layernorm.weight" in names
+    assert not any("q_proj" in n or "up_proj.weight" in n.replace("gate_up_proj", "") or "input_layernorm" in n for n in names)
+    assert len(names) == 3 * 6 + 3 and f.shape("model.layers.0.self_attn.qkv_proj.weight") == (96 + 2 * 32, 96)
+    model = build_model(cfg)
+    load_weights(model, os.path.join(folder, "model.safetensors"), torch.float32, "cpu")
+    for i, b in enumerate(model.blocks):
+        assert torch.equal(b.mixer.wqkv, f.tensor(f"model.layers.{i}.self_attn.qkv_proj.weight"))
+        assert torch.equal(b.ffn.w_gate_up, f.tensor(f"model.layers.{i}.mlp.gate_up_proj.weight"))
+        assert torch.equal(b.mixer_norm.weight, f.tensor(f"model.layers.{i}.ln_1.weight"))
+        assert torch.equal(b.ffn_norm.weight, f.tensor(f"model.layers.{i}.ln_2.weight"))
+    assert torch.equal(model.final_norm.weight, f.tensor("model.final_layernorm.weight"))
+    # the same weights under the plain names load into the Llama model as the same tensors
+    tensors = {n: f.tensor(n).clone() for n in f.names()}
+    llama = build_model(config_from_dict(helpers.TINY_B))
+    save_file(plain_names(tensors), str(tmp_path / "plain.safetensors"))
+    load_weights(llama, str(tmp_path / "plain.safetensors"), torch.float32, "cpu")
+    assert torch.equal(llama.blocks[1].mixer.wqkv, model.blocks[1].mixer.wqkv)
+    assert torch.equal(llama.blocks[2].ffn.w_gate_up, model.blocks[2].ffn.w_gate_up)
+
+
+def test_errors_of_a_fused_checkpoint_speak_of_the_files_tensors(tmp_path):
+    raw = register_fused_toy()
+    cfg = config_from_dict(raw)
+    folder = write_random_model(cfg, str(tmp_path / "fused"), seed=5)
+    path = os.path.join(folder, "model.safetensors")
+    f = SafetensorsFile(path)
+    tensors = {n: f.tensor(n).clone() for n in f.names()}
+    del tensors["model.layers.1.self_attn.qkv_proj.weight"]                   # three of the model's tensors, one of the file's
+    tensors["model.layers.0.mlp.gate_up_proj.weight"] = torch.zeros(500, 96)  # rows that the parts do not cover
+    tensors["model.layers.2.self_attn.k_proj.weight"] = torch.zeros(32, 96)   # the parts' own name is not the file's
+    del tensors["model.final_layernorm.weight"]
+    save_file(tensors, path)
+    with pytest.raises(WeightError) as e:
+        load_weights(build_model(cfg), path, torch.float32, "cpu")
+    msg = str(e.value)
+    assert "missing tensors (2): model.final_layernorm.weight, model.layers.1.self_attn.qkv_proj.weight" in msg
+    assert "unexpected tensors (1): model.layers.2.self_attn.k_proj.weight" in msg
+    assert "wrong shapes (1): model.layers.0.mlp.gate_up_proj.weight is [500, 96], expected [512, 96]" in msg
+
+
+def test_sources_that_do_not_cover_a_tensor_are_refused():
+    from glassbox_amd.weights import checkpoint_layout
+    from glassbox_amd.parts.mlp import SwiGLU
+
+    class Model(SwiGLU):
+        def __init__(self, sources):
+            super().__init__(8, 16)
+            self.table = sources
+
+        def source_of(self, name):
+            return self.table.get(name)
+
+    ok = {"gate_proj.weight": ("gu.weight", 0, 16), "up_proj.weight": ("gu.weight", 16, 32), "down_proj.weight": "d.weight"}
+    sources, shapes = checkpoint_layout(Model(ok))
+    assert shapes == {"gu.weight": (32, 8), "d.weight": (8, 16)} and sources["up_proj.weight"] == ("gu.weight", 16, 32)
+    for bad, word in ((dict(ok, **{"up_proj.weight": ("gu.weight", 20, 36)}), "one after the other"),      # a gap
+                      (dict(ok, **{"up_proj.weight": ("gu.weight", 8, 24)}), "one after the other"),       # an overlap
+                      (dict(ok, **{"up_proj.weight": ("gu.weight", 16, 30)}), "16 rows"),                  # a wrong count
+                      (dict(ok, **{"up_proj.weight": ("gu.weight", 16, None)}), "no range"),
+                      (dict(ok, **{"down_proj.weight": "gu.weight"}), "more than one"),
+                      (dict(ok, **{"gate_proj.weight": "d.weight", "up_proj.weight": None}), "more than one")):
+        with pytest.raises(WeightError, match=word):
+            checkpoint_layout(Model(bad))
+
+
+def test_why_a_model_cannot_share_beginnings_is_said_layer_by_layer():
+    """Prefix sharing needs every cache layer to keep every page and nothing beside pages: the engine refuses
+    ``prefix_caching=True`` with these lines instead of switching it off without a word."""
+    from glassbox_amd.engine.engine import sharing_obstacles
+    from glassbox_amd.parts.attention import PagedAttention
+    from glassbox_amd.parts.base import StateSpec
+    from glassbox_amd.parts.block import PreNormBlock
+    from glassbox_amd.parts.embedding import Embedding, LMHead
+    from glassbox_amd.parts.mlp import SwiGLU
+    from glassbox_amd.parts.model import DecoderModel, LayerCall
+    from glassbox_amd.parts.norm import RMSNorm
+    from glassbox_amd.parts.rotary import Rotary
+    assert sharing_obstacles(build_model(config_from_dict(helpers.TINY_A))) == []
+    rotary = Rotary(8, 10000.0)
+
+    class WithState(PagedAttention):
+        state_spec = StateSpec((4,))
+
+    def block(window=0, cls=PagedAttention):
+        return PreNormBlock(RMSNorm(32, 1e-5), cls(32, 4, 2, 8, rotary, window=window), RMSNorm(32, 1e-5), SwiGLU(32, 48))
+    emb = Embedding(50, 32)
+    model = DecoderModel(None, emb, [block(), block(7), block(cls=WithState), block(7), block(9)],
+                         [LayerCall(i, cache=i) for i in range(5)], RMSNorm(32, 1e-5), LMHead(50, 32, tied_to=emb))
+    lines = sharing_obstacles(model)
+    assert len(lines) == 3
+    assert lines[0].startswith("cache layers 1, 3: a window of 7") and lines[1].startswith("cache layer 4: a window of 9")
+    assert lines[2].startswith("cache layer 2: state of its own")

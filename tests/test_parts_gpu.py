@@ -424,3 +424,30 @@ def test_toy_with_routing_and_learned_positions(tmp_path):
             assert bad is None, f"{r}: first wrong position {bad}"
         eng.cache.check_invariants()
         assert eng.cache.used_pages(0) == 0
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_a_checkpoint_with_fused_projections_steps_like_the_same_weights_under_the_parts_names(tmp_path, bf16_bound, dtype):
+    """The stock mixer and feed-forward load a checkpoint that keeps query, key and value rows in one tensor and
+    gate and up rows in another, under other names (a function from names to sources, given to the model): the
+    engine's logits are the plain implementation's on the same weights cut and named the plain way."""
+    import os
+    from test_config_weights import plain_names, register_fused_toy
+    from glassbox_amd.config import config_from_dict
+    from glassbox_amd.engine import Engine
+    from glassbox_amd.weights import SafetensorsFile, save_file, write_random_model
+    raw = register_fused_toy()
+    fused = write_random_model(config_from_dict(raw), str(tmp_path / "fused"), seed=11, norm_init="uniform")
+    f = SafetensorsFile(os.path.join(fused, "model.safetensors"))
+    plain_folder = str(tmp_path / "plain")
+    os.makedirs(plain_folder)
+    config_from_dict(helpers.TINY_B).save(plain_folder)
+    save_file(plain_names({n: f.tensor(n).clone() for n in f.names()}), os.path.join(plain_folder, "model.safetensors"))
+    requests = {"a": helpers.random_tokens(384, 45, seed=1), "b": helpers.random_tokens(384, 20, seed=2)}
+    steps, peak = helpers.schedule_mixed(requests, seed=3, live=2, tail=8)
+    eng = Engine(fused, dtype=dtype, max_tokens=max(peak, 128), max_seqs=2)
+    got = helpers.replay(eng, steps)
+    tol = helpers.TOL_F32 if dtype == "float32" else bf16_bound.get(plain_folder, requests)
+    for r, toks in requests.items():
+        bad = helpers.first_bad(got[r], helpers.oracle(plain_folder, toks, dtype), tol)
+        assert bad is None, f"request {r}: first wrong position {bad[0]}, error {bad[1]:.3e}, allowed {tol:.3e}"

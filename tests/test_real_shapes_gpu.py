@@ -54,7 +54,7 @@ def test_parity_at_the_sizes_of_real_models(name):
     schedules = {"whole": (helpers.schedule_whole(requests), 1024), "tail32": (helpers.schedule_tail(requests), 1024),
                  "chunks": (helpers.schedule_chunks(requests, sizes=(33, 2, 64, 7, 17)), 1024), "mixed": (mixed, peak)}
     plain_engine = engine_of(cfg, tensors, "bfloat16", 1024, kernels="plain")
-    bf16_tol = helpers.Bf16Bound.measure(plain_engine, requests, lambda r: want[r])
+    bf16_tol = helpers.Bf16Bound.measure(plain_engine, requests, lambda r: want[r], label=name)
     del plain_engine
     for dtype in ("float32", "bfloat16"):
         tol = helpers.TOL_F32 if dtype == "float32" else bf16_tol
