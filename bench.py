@@ -79,7 +79,9 @@ def main() -> int:
     from glassbox_amd.weights import build_model, init_random
 
     MODEL = SHAPES[a.shapes]
-    cfg = config_from_dict(dict(MODEL, num_hidden_layers=a.layers or MODEL["num_hidden_layers"]))
+    # (a context beyond the model's own limit is measured all the same: the scheduler would end requests at the limit)
+    cfg = config_from_dict(dict(MODEL, num_hidden_layers=a.layers or MODEL["num_hidden_layers"],
+                                max_position_embeddings=max(MODEL["max_position_embeddings"], a.context + 1)))
     model = build_model(cfg)
     init_random(model, seed=0, dtype=a.dtype, device="cuda:0")
     batches = [a.batch] + ([] if a.no_points else [b for b in (1, 64) if b != a.batch])
@@ -174,7 +176,8 @@ def main() -> int:
 
     # ---- the same workload as requests under the scheduler: plan, step, sample, finish
     def scheduler_run(batch, steps, warmup):
-        slack = 4 * batch + 8          # tokens that the first requests decode while the last ones are still prompts
+        # tokens that the first requests decode while the last ones are still prompts (a step of prompt portions each)
+        slack = batch * -(-a.context // PREFILL_TOKENS) + 8
         budget = warmup + steps + slack
         start = a.context - budget
         sched = Scheduler(eng, SchedulerConfig(token_budget=PREFILL_TOKENS, max_seqs=batch))
