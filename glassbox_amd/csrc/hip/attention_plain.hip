@@ -6,8 +6,20 @@
 // Token t of request s at position p reads keys lo..p of its own request through the block
 // table, lo = 0 or p - window + 1 (crates/glassbox-core/src/model.rs:285-312):
 //   score = dot(q, k) * scale ; prob = softmax(score) ; out = sum prob * v
-// Keys are taken in chunks of 256 in ascending position with a running maximum and sum, so
-// the order of every addition depends on the position alone, not on the batch.
+//
+// The order of every addition depends on the token's position alone, not on the batch and not
+// on how the work is spread over workgroups.  Keys go in chunks of 256 from lo on.  A chunk is
+// computed by itself: a thread a key for the scores (dot products in ascending dimension), the
+// chunk's own maximum m_c, e = exp(score - m_c), their sum l_c, and sum e * v, for which a thread
+// owns (dimension, word of four slots of a page) pairs and walks the chunk's pages in order, so
+// that a page's values are read as whole 16-byte words by neighbouring lanes.  Chunks are then
+// merged in ascending order (merge_chunk), and at the end a dimension's words are added in
+// ascending order and divided by the sum.
+//
+// Two ways to run this, with the same bits: one workgroup walks all chunks of its (token, head)
+// and merges in registers; or, for a few tokens with long contexts (a decode step, whose handful
+// of workgroups would leave most of the chip idle), a workgroup a chunk writes (m_c, l_c, sums) to
+// a workspace and a second kernel merges them, chunk by chunk, by the same function.
 #include "common.h"
 
 using namespace gb;
@@ -17,90 +29,295 @@ GB_DEFINE_LAST_ERROR
 namespace {
 
 constexpr int kChunk = 256;
+constexpr int kMaxOwn = 16;   // (dimension, word) pairs a thread owns at most: head size * page size <= 16,384
 
+struct Running {
+  float m, l;
+};
+
+// (m, l, acc) of the chunks so far, joined by the next chunk's (m_c, l_c, a_c).  The same
+// expressions in both kernels that merge: products and fused multiply-adds are spelled out, so
+// that the compiler has no choice of how to contract them.
+template <int PER>
+__device__ __forceinline__ void merge_chunk(Running& r, float (&acc)[PER], float m_c, float l_c, const float (&a_c)[PER]) {
+  const float m_new = fmaxf(r.m, m_c);
+  const float alpha = expf(r.m - m_new);   // 0 for the first chunk (m = -inf)
+  const float beta = expf(m_c - m_new);
+  r.l = fmaf(l_c, beta, r.l * alpha);
+#pragma unroll
+  for (int u = 0; u < PER; ++u) acc[u] = fmaf(a_c[u], beta, acc[u] * alpha);
+  r.m = m_new;
+}
+
+template <typename T> __device__ __forceinline__ void load_words(const T* p, float (&v)[4]);
+template <> __device__ __forceinline__ void load_words<float>(const float* p, float (&v)[4]) {
+  const f32x4 x = *reinterpret_cast<const f32x4*>(p);
+  v[0] = x[0]; v[1] = x[1]; v[2] = x[2]; v[3] = x[3];
+}
+template <> __device__ __forceinline__ void load_words<bf16>(const bf16* p, float (&v)[4]) {
+  const bf16x4 x = *reinterpret_cast<const bf16x4*>(p);
+  v[0] = (float)x[0]; v[1] = (float)x[1]; v[2] = (float)x[2]; v[3] = (float)x[3];
+}
+
+// dot(q, key) in ascending dimension; the key lies in pieces of `piece` elements (key_offset)
 template <typename T>
+__device__ __forceinline__ float key_dot(const float* qs, const T* kb, int slot, int hd, int page_size, int piece) {
+  float dot = 0.f;
+  if (piece == 8) {
+#pragma unroll 4
+    for (int d0 = 0; d0 < hd; d0 += 8) {
+      const T* kr = kb + ((size_t)(d0 / 8) * page_size + slot) * 8;
+      float lo[4], hi[4];
+      load_words<T>(kr, lo);
+      load_words<T>(kr + 4, hi);
+#pragma unroll
+      for (int e = 0; e < 4; ++e) dot = fmaf(qs[d0 + e], lo[e], dot);
+#pragma unroll
+      for (int e = 0; e < 4; ++e) dot = fmaf(qs[d0 + 4 + e], hi[e], dot);
+    }
+  } else {
+    for (int d0 = 0; d0 < hd; d0 += piece) {
+      const T* kr = kb + key_offset(slot, d0, page_size, piece);
+      for (int e = 0; e < piece; ++e) dot = fmaf(qs[d0 + e], to_f(kr[e]), dot);
+    }
+  }
+  return dot;
+}
+
+struct Shape {
+  int nh, nkv, hd, page_size, window, table_stride;
+  float scale;
+};
+
+// One chunk by itself: keys c0 .. hi of the token's request.  Leaves m_c, l_c and the thread's sums a_c.
+// `qs` holds the query, `es` (kChunk floats) and `scratch` (17) are the block's.
+template <typename T, int PER>
+__device__ __forceinline__ void chunk_alone(const Shape& sh, const float* qs, float* es, float* scratch,
+                                            const int32_t* __restrict__ table, const T* __restrict__ k_pages,
+                                            const T* __restrict__ v_pages, int kvh, int c0, int hi, float& m_c, float& l_c,
+                                            float (&a_c)[PER]) {
+  const int tid = threadIdx.x;
+  const int ps = sh.page_size, hd = sh.hd;
+  const int p = c0 + tid;
+  float s = -INFINITY;
+  if (p <= hi) {
+    const int page = table[p / ps];
+    const T* kb = k_pages + ((size_t)page * sh.nkv + kvh) * ps * hd;
+    s = key_dot<T>(qs, kb, p % ps, hd, ps, key_piece(hd)) * sh.scale;
+  }
+  m_c = block_max(s, scratch);
+  const float e = p <= hi ? expf(s - m_c) : 0.f;
+  es[tid] = e;
+  l_c = block_sum(e, scratch);   // also orders the writes of es before the reads below
+  const int words = ps / 4, pairs = hd * words;
+#pragma unroll
+  for (int u = 0; u < PER; ++u) a_c[u] = 0.f;
+  const int pg_last = hi / ps;
+#pragma unroll 4
+  for (int pg = c0 / ps; pg <= pg_last; ++pg) {
+    const int page = table[pg];
+    const T* vb = v_pages + ((size_t)page * sh.nkv + kvh) * hd * ps;
+#pragma unroll
+    for (int u = 0; u < PER; ++u) {
+      const int idx = tid + kChunk * u;
+      if (idx >= pairs) continue;
+      const int d = idx / words, p0 = pg * ps + 4 * (idx % words);
+      if (p0 + 3 < c0 || p0 > hi) continue;
+      float v[4];
+      load_words<T>(vb + (size_t)d * ps + 4 * (idx % words), v);
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        const int pj = p0 + j;
+        if (pj >= c0 && pj <= hi) a_c[u] = fmaf(es[pj - c0], v[j], a_c[u]);
+      }
+    }
+  }
+  __syncthreads();   // es is written again by the next chunk
+}
+
+// The end: a dimension's words added in ascending order, divided by the sum.
+template <typename T, int PER>
+__device__ __forceinline__ void finish(const Shape& sh, float* comb, const float (&acc)[PER], float l, T* out_row) {
+  const int tid = threadIdx.x;
+  const int words = sh.page_size / 4, pairs = sh.hd * words;
+#pragma unroll
+  for (int u = 0; u < PER; ++u) {
+    const int idx = tid + kChunk * u;
+    if (idx < pairs) comb[idx] = acc[u];
+  }
+  __syncthreads();
+  if (tid < sh.hd) {
+    float sum = 0.f;
+    for (int wd = 0; wd < words; ++wd) sum += comb[tid * words + wd];
+    out_row[tid] = from_f<T>(sum / l);
+  }
+}
+
+__device__ __forceinline__ int ws_stride(int per) { return per * kChunk + 2; }
+
+template <typename T, int PER, bool SPLIT>
 __global__ __launch_bounds__(kChunk) void attention_plain_kernel(
     const T* __restrict__ q, int q_stride, T* __restrict__ out, int out_stride, const int32_t* __restrict__ positions,
-    const int32_t* __restrict__ tok_seq, const int32_t* __restrict__ tables, int table_stride,
-    const T* __restrict__ k_pages, const T* __restrict__ v_pages, int nh, int nkv, int hd, int page_size, float scale,
-    int window) {
+    const int32_t* __restrict__ tok_seq, const int32_t* __restrict__ tables, const T* __restrict__ k_pages,
+    const T* __restrict__ v_pages, Shape sh, float* __restrict__ ws, int max_chunks) {
   extern __shared__ float smem[];
-  float* qs = smem;              // [hd]
-  float* es = smem + hd;         // [kChunk]
-  float* scratch = es + kChunk;  // [17]
-  const int t = blockIdx.x / nh, h = blockIdx.x % nh;
-  const int kvh = h / (nh / nkv);
+  float* qs = smem;                   // [hd]
+  float* es = smem + sh.hd;           // [kChunk]
+  float* scratch = es + kChunk;       // [17]
+  float* comb = scratch + 17;         // [hd * page_size / 4]
+  const int t = blockIdx.x / sh.nh, h = blockIdx.x % sh.nh;
+  const int kvh = h / (sh.nh / sh.nkv);
   const int pos = positions[t];
-  const int32_t* table = tables + (size_t)tok_seq[t] * table_stride;
-  const int lo = window > 0 ? max(0, pos - window + 1) : 0;
+  const int32_t* table = tables + (size_t)tok_seq[t] * sh.table_stride;
+  const int lo = sh.window > 0 ? max(0, pos - sh.window + 1) : 0;
+  const int n_chunks = (pos - lo) / kChunk + 1;
   const int tid = threadIdx.x;
-  const int piece = key_piece(hd);
+  if (SPLIT && (int)blockIdx.y >= n_chunks) return;
 
-  for (int d = tid; d < hd; d += kChunk) qs[d] = to_f(q[(size_t)t * q_stride + (size_t)h * hd + d]);
+  for (int d = tid; d < sh.hd; d += kChunk) qs[d] = to_f(q[(size_t)t * q_stride + (size_t)h * sh.hd + d]);
   __syncthreads();
 
-  float m = -INFINITY, l = 0.f, acc = 0.f;  // acc: output dimension `tid` (tid < hd)
-  for (int c0 = lo; c0 <= pos; c0 += kChunk) {
-    const int p = c0 + tid;
-    float s = -INFINITY;
-    if (p <= pos) {
-      const int page = table[p / page_size];
-      const T* kb = k_pages + ((size_t)page * nkv + kvh) * page_size * hd;  // pieces of the head size, see key_piece()
-      float dot = 0.f;
-      for (int d0 = 0; d0 < hd; d0 += piece) {
-        const T* kr = kb + key_offset(p % page_size, d0, page_size, piece);
-        for (int e = 0; e < piece; ++e) dot = fmaf(qs[d0 + e], to_f(kr[e]), dot);
-      }
-      s = dot * scale;
+  if (SPLIT) {
+    const int c = blockIdx.y, c0 = lo + c * kChunk;
+    float m_c, l_c, a_c[PER];
+    chunk_alone<T, PER>(sh, qs, es, scratch, table, k_pages, v_pages, kvh, c0, min(c0 + kChunk - 1, pos), m_c, l_c, a_c);
+    float* cell = ws + ((size_t)blockIdx.x * max_chunks + c) * ws_stride(PER);
+#pragma unroll
+    for (int u = 0; u < PER; ++u) cell[u * kChunk + tid] = a_c[u];
+    if (tid == 0) {
+      cell[PER * kChunk] = m_c;
+      cell[PER * kChunk + 1] = l_c;
     }
-    const float cm = block_max(s, scratch);
-    const float m_new = fmaxf(m, cm);
-    const float e = p <= pos ? expf(s - m_new) : 0.f;
-    es[tid] = e;
-    const float csum = block_sum(e, scratch);  // also orders the writes of es before the reads below
-    const float rescale = expf(m - m_new);     // 0 on the first chunk (m = -inf)
-    l = l * rescale + csum;
-    acc *= rescale;
-    if (tid < hd) {
-      const int cnt = min(kChunk, pos - c0 + 1);
-      for (int j = 0; j < cnt; ++j) {
-        const int pj = c0 + j;
-        const int page = table[pj / page_size];
-        acc = fmaf(es[j], to_f(v_pages[(((size_t)page * nkv + kvh) * hd + tid) * page_size + pj % page_size]), acc);
-      }
-    }
-    m = m_new;
-    __syncthreads();
+    return;
   }
-  if (tid < hd) out[(size_t)t * out_stride + (size_t)h * hd + tid] = from_f<T>(acc / l);
+  Running r{-INFINITY, 0.f};
+  float acc[PER];
+#pragma unroll
+  for (int u = 0; u < PER; ++u) acc[u] = 0.f;
+  for (int c = 0; c < n_chunks; ++c) {
+    const int c0 = lo + c * kChunk;
+    float m_c, l_c, a_c[PER];
+    chunk_alone<T, PER>(sh, qs, es, scratch, table, k_pages, v_pages, kvh, c0, min(c0 + kChunk - 1, pos), m_c, l_c, a_c);
+    merge_chunk<PER>(r, acc, m_c, l_c, a_c);
+  }
+  finish<T, PER>(sh, comb, acc, r.l, out + (size_t)t * out_stride + (size_t)h * sh.hd);
+}
+
+// Merges what the workgroups of a (token, head) left, chunk by chunk in ascending order.
+template <typename T, int PER>
+__global__ __launch_bounds__(kChunk) void attention_plain_merge_kernel(T* __restrict__ out, int out_stride,
+                                                                       const int32_t* __restrict__ positions, Shape sh,
+                                                                       const float* __restrict__ ws, int max_chunks) {
+  extern __shared__ float smem[];   // [hd * page_size / 4]
+  const int t = blockIdx.x / sh.nh, h = blockIdx.x % sh.nh;
+  const int pos = positions[t];
+  const int lo = sh.window > 0 ? max(0, pos - sh.window + 1) : 0;
+  const int n_chunks = min((pos - lo) / kChunk + 1, max_chunks);   // (never beyond what the workspace holds)
+  const int tid = threadIdx.x;
+  Running r{-INFINITY, 0.f};
+  float acc[PER];
+#pragma unroll
+  for (int u = 0; u < PER; ++u) acc[u] = 0.f;
+  for (int c = 0; c < n_chunks; ++c) {
+    const float* cell = ws + ((size_t)blockIdx.x * max_chunks + c) * ws_stride(PER);
+    float a_c[PER];
+#pragma unroll
+    for (int u = 0; u < PER; ++u) a_c[u] = cell[u * kChunk + tid];
+    merge_chunk<PER>(r, acc, cell[PER * kChunk], cell[PER * kChunk + 1], a_c);
+  }
+  finish<T, PER>(sh, smem, acc, r.l, out + (size_t)t * out_stride + (size_t)h * sh.hd);
+}
+
+inline int own_pairs(int hd, int page_size) {
+  const int per = (hd * (page_size / 4) + kChunk - 1) / kChunk;
+  for (int p = 1; p <= kMaxOwn; p *= 2)
+    if (per <= p) return p;
+  return 0;
+}
+
+template <typename T, int PER>
+void launch(const void* q, int q_stride, void* out, int out_stride, const int32_t* positions, const int32_t* tok_seq,
+            const int32_t* tables, const void* k_pages, const void* v_pages, int n, const Shape& sh, float* ws,
+            int max_chunks, hipStream_t stream) {
+  const size_t comb = sizeof(float) * sh.hd * (sh.page_size / 4);
+  const size_t smem = sizeof(float) * (sh.hd + kChunk + 17) + comb;
+  if (ws != nullptr) {
+    hipLaunchKernelGGL((attention_plain_kernel<T, PER, true>), dim3((unsigned)(n * sh.nh), (unsigned)max_chunks), dim3(kChunk),
+                       smem, stream, (const T*)q, q_stride, (T*)out, out_stride, positions, tok_seq, tables,
+                       (const T*)k_pages, (const T*)v_pages, sh, ws, max_chunks);
+    hipLaunchKernelGGL((attention_plain_merge_kernel<T, PER>), dim3((unsigned)(n * sh.nh)), dim3(kChunk), comb, stream,
+                       (T*)out, out_stride, positions, sh, (const float*)ws, max_chunks);
+  } else {
+    hipLaunchKernelGGL((attention_plain_kernel<T, PER, false>), dim3((unsigned)(n * sh.nh)), dim3(kChunk), smem, stream,
+                       (const T*)q, q_stride, (T*)out, out_stride, positions, tok_seq, tables, (const T*)k_pages,
+                       (const T*)v_pages, sh, nullptr, 0);
+  }
+}
+
+template <typename T>
+int launch_by_pairs(int per, const void* q, int q_stride, void* out, int out_stride, const int32_t* positions,
+                    const int32_t* tok_seq, const int32_t* tables, const void* k_pages, const void* v_pages, int n,
+                    const Shape& sh, float* ws, int max_chunks, hipStream_t stream) {
+#define GB_PLAIN_CASE(P)                                                                                              \
+  case P:                                                                                                             \
+    launch<T, P>(q, q_stride, out, out_stride, positions, tok_seq, tables, k_pages, v_pages, n, sh, ws, max_chunks, stream); \
+    break;
+  switch (per) {
+    GB_PLAIN_CASE(1) GB_PLAIN_CASE(2) GB_PLAIN_CASE(4) GB_PLAIN_CASE(8) GB_PLAIN_CASE(16)
+    default: return fail("attention_plain: no kernel for %d pairs a thread", per);
+  }
+#undef GB_PLAIN_CASE
+  return launched("attention_plain");
 }
 
 }  // namespace
 
+// Floats of workspace that the chunk-by-chunk form needs for n tokens whose longest context (keys a token reads) is
+// max_context, or 0 where the sizes are refused anyway.
+extern "C" long long gb_attention_plain_split_floats(int n, int nh, int hd, int page_size, int max_context) {
+  if (n <= 0 || nh <= 0 || hd <= 0 || page_size <= 0 || page_size % 4 || max_context <= 0) return 0;
+  const int per = own_pairs(hd, page_size);
+  if (per == 0) return 0;
+  const long long chunks = (max_context + kChunk - 1) / kChunk;
+  return (long long)n * nh * chunks * (per * kChunk + 2);
+}
+
+// ws = nullptr: a workgroup a (token, head) walks the whole context.  Otherwise ws holds at least
+// gb_attention_plain_split_floats(n, nh, hd, page_size, max_context) floats, max_context is at least the most keys any
+// of the tokens reads, and a workgroup a chunk of 256 keys leaves its part there for a second kernel to merge: the
+// same bits, for steps of few tokens with long contexts.
 extern "C" int gb_attention_plain(const void* q, int q_stride, void* out, int out_stride, int dtype,
                                   const int32_t* positions, const int32_t* tok_seq, const int32_t* tables,
                                   int table_stride, const void* k_pages, const void* v_pages, int n, int nh, int nkv,
-                                  int hd, int page_size, float scale, int window, hipStream_t stream) {
+                                  int hd, int page_size, float scale, int window, float* ws, long long ws_floats,
+                                  int max_context, hipStream_t stream) {
   GB_REQUIRE(n >= 0 && nh > 0 && nkv > 0 && hd > 0, "attention_plain: bad sizes n=%d nh=%d nkv=%d hd=%d", n, nh, nkv, hd);
   GB_REQUIRE(nh % nkv == 0, "attention_plain: %d query heads are not a multiple of %d key heads", nh, nkv);
   GB_REQUIRE(hd <= kChunk, "attention_plain: head size %d is above the supported 256", hd);
   GB_REQUIRE(q_stride >= nh * hd && out_stride >= nh * hd, "attention_plain: row strides shorter than the heads");
   GB_REQUIRE(page_size > 0 && table_stride > 0 && window >= 0, "attention_plain: bad page size, table stride or window");
+  GB_REQUIRE(page_size % 4 == 0, "attention_plain: a page of %d tokens is not whole words of four slots", page_size);
   GB_REQUIRE((long long)n * nh < (1ll << 31), "attention_plain: too many (token, head) pairs");
+  const int per = own_pairs(hd, page_size);
+  GB_REQUIRE(per != 0, "attention_plain: head size %d times page size %d is above %d", hd, page_size, kMaxOwn * kChunk * 4);
   if (n == 0) return 0;
-  const size_t smem = sizeof(float) * (hd + kChunk + 17);
-  const dim3 grid((unsigned)(n * nh));
+  int max_chunks = 0;
+  if (ws != nullptr) {
+    GB_REQUIRE(max_context > 0, "attention_plain: the chunk-by-chunk form needs the longest context");
+    max_chunks = (max_context + kChunk - 1) / kChunk;
+    GB_REQUIRE(max_chunks <= 65535, "attention_plain: a context of %d keys is more chunks than a launch takes", max_context);
+    GB_REQUIRE(ws_floats >= gb_attention_plain_split_floats(n, nh, hd, page_size, max_context),
+               "attention_plain: the workspace holds %lld floats, %lld are needed", ws_floats,
+               gb_attention_plain_split_floats(n, nh, hd, page_size, max_context));
+  }
+  const Shape sh{nh, nkv, hd, page_size, window, table_stride, scale};
   if (dtype == kF32)
-    hipLaunchKernelGGL(attention_plain_kernel<float>, grid, dim3(kChunk), smem, stream, (const float*)q, q_stride,
-                       (float*)out, out_stride, positions, tok_seq, tables, table_stride, (const float*)k_pages,
-                       (const float*)v_pages, nh, nkv, hd, page_size, scale, window);
-  else if (dtype == kBF16)
-    hipLaunchKernelGGL(attention_plain_kernel<bf16>, grid, dim3(kChunk), smem, stream, (const bf16*)q, q_stride,
-                       (bf16*)out, out_stride, positions, tok_seq, tables, table_stride, (const bf16*)k_pages,
-                       (const bf16*)v_pages, nh, nkv, hd, page_size, scale, window);
-  else
-    return fail("attention_plain: unknown dtype %d", dtype);
-  return launched("attention_plain");
+    return launch_by_pairs<float>(per, q, q_stride, out, out_stride, positions, tok_seq, tables, k_pages, v_pages, n, sh, ws,
+                                  max_chunks, stream);
+  if (dtype == kBF16)
+    return launch_by_pairs<bf16>(per, q, q_stride, out, out_stride, positions, tok_seq, tables, k_pages, v_pages, n, sh, ws,
+                                 max_chunks, stream);
+  return fail("attention_plain: unknown dtype %d", dtype);
 }
 
 // the launches of a layer can be recorded and made again for the layers like it (common.h)

@@ -51,6 +51,7 @@ _SIGS = {
     },
     "gemm_f32": {
         "gb_gemm_f32": [_vp, _i, _vp, _i, _vp, _i, _i, _i, _i, _i, _vp],
+        "gb_gemm_f32_by": [_vp, _i, _vp, _i, _vp, _i, _i, _i, _i, _i, _i, _vp],
     },
     "gemm_bf16": {
         # a, lda, w, ldw, c, ldc, c_dtype, M, N, K, epilogue, gamma, gamma_dtype, eps,
@@ -66,7 +67,11 @@ _SIGS = {
                               _i, _i, _i, _i, _vp],
     },
     "attention_plain": {
-        "gb_attention_plain": [_vp, _i, _vp, _i, _i, _vp, _vp, _vp, _i, _vp, _vp, _i, _i, _i, _i, _i, _f, _i, _vp],
+        # q, q_stride, out, out_stride, dtype, positions, tok_seq, tables, table_stride, k, v, n, nh, nkv, hd, page,
+        # scale, window, workspace, workspace floats, max_context, stream
+        "gb_attention_plain": [_vp, _i, _vp, _i, _i, _vp, _vp, _vp, _i, _vp, _vp, _i, _i, _i, _i, _i, _f, _i, _vp,
+                               C.c_longlong, _i, _vp],
+        "gb_attention_plain_split_floats": [_i, _i, _i, _i, _i],
     },
     "attention_bf16": {
         # q, q_stride, out, out_stride, ws_acc, ws_ml, positions, tables, table_stride, k, v,
@@ -615,10 +620,25 @@ MAX_HEAD_DIM = 256        # attention_plain.hip: a head's dimensions are held by
 MAX_VOCAB = 1 << 20       # sampling.hip: a token id takes 20 bits of the (logit, token) key the sampler searches
 
 
+PLAIN_SPLIT_MAX_PAIRS = 1024   # (token, head) pairs up to which a step of long contexts goes a workgroup a chunk
+
+
+def attention_plain_split_floats(n: int, n_heads: int, head_dim: int, page_size: int, max_context: int) -> int:
+    """Floats of workspace with which ``attention_plain`` spreads the chunks of long contexts over workgroups, or 0
+    where it would not: many (token, head) pairs fill the chip by themselves, and a context of one chunk has
+    nothing to spread.  The bits of the result are the same either way."""
+    if n * n_heads > PLAIN_SPLIT_MAX_PAIRS or max_context <= 256:
+        return 0
+    return int(_lib("attention_plain").gb_attention_plain_split_floats(n, n_heads, head_dim, page_size, max_context))
+
+
 def attention_plain(q: torch.Tensor, out: torch.Tensor, positions: torch.Tensor, tok_seq: torch.Tensor,
                     tables: torch.Tensor, k_pages: torch.Tensor, v_pages: torch.Tensor, n_heads: int,
-                    scale: float, window: int = 0) -> None:
-    """Paged attention, one block per (token, head); q may be a view into the stacked qkv rows."""
+                    scale: float, window: int = 0, workspace: Optional[torch.Tensor] = None, max_context: int = 0) -> None:
+    """Paged attention, one block per (token, head); q may be a view into the stacked qkv rows.
+    ``workspace`` (float32, ``attention_plain_split_floats`` elements) with ``max_context`` (at least the most keys a
+    token of the step reads): a workgroup a chunk of 256 keys and a second kernel that merges them, for steps of few
+    tokens with long contexts; the same bits as without."""
     _dev(q, out, positions, tok_seq, tables, k_pages, v_pages)
     n = q.shape[0]
     if q.dtype != out.dtype:
@@ -630,10 +650,15 @@ def attention_plain(q: torch.Tensor, out: torch.Tensor, positions: torch.Tensor,
     _i32(tok_seq, "tok_seq", n)
     if tables.dtype != torch.int32 or tables.dim() != 2 or tables.stride(1) != 1:
         raise KernelError("attention: block tables must be int32 [requests, pages]")
+    if workspace is not None:
+        _dev(workspace)
+        if workspace.dtype != torch.float32 or not workspace.is_contiguous() or max_context <= 0:
+            raise KernelError("attention: the workspace must be contiguous float32 and come with the longest context")
     lib = _lib("attention_plain")
     _launch(lib, lib.gb_attention_plain, _p(q), _rows(q, "q"), _p(out), _rows(out, "out"), dtype_code(q), _p(positions),
                                        _p(tok_seq), _p(tables), tables.stride(0), _p(k_pages), _p(v_pages), n,
-                                       n_heads, nkv, hd, page_size, float(scale), int(window), _stream())
+                                       n_heads, nkv, hd, page_size, float(scale), int(window), _p(workspace),
+                                       workspace.numel() if workspace is not None else 0, int(max_context), _stream())
 
 
 def tuned_attention_supports(k_pages: torch.Tensor, n_heads: int, window: int) -> bool:

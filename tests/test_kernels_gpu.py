@@ -22,7 +22,11 @@ def to_dev(t, dtype=None):
 # ----------------------------------------------------------------------- products
 # (rows of W, k, tokens): the awkward shapes of the reference's own matmul test
 # (crates/glassbox-core/src/kernels.rs:697) and larger ones that cross tile edges
-GEMM_SHAPES_F32 = [(1, 32, 1), (8, 64, 2), (17, 64, 3), (33, 96, 9), (50, 160, 17), (331, 100, 70), (130, 257, 129)]
+GEMM_SHAPES_F32 = [(1, 32, 1), (8, 64, 2), (17, 64, 3), (33, 96, 9), (50, 160, 17), (331, 100, 70), (130, 257, 129),
+                   # few rows through the skinny kernel: a k of one slice and a part, of many groups of slices, rows of W
+                   # that do not fill the last workgroup, rows of A in several passes
+                   (2048, 2048, 1), (50, 100, 5), (2048, 8192, 8), (331, 2120, 16), (96, 4100, 33), (1000, 72, 64),
+                   (130, 258, 7)]
 GEMM_SHAPES_BF16 = [(1, 32, 1), (8, 64, 2), (17, 64, 3), (33, 96, 9), (50, 160, 17), (331, 104, 64), (331, 104, 65),
                     (130, 264, 129), (16, 2048, 8), (272, 72, 300), (49, 520, 33),
                     # few rows of W and a long k: the skinny kernels split k over the waves of a workgroup
@@ -45,6 +49,49 @@ def test_gemm_f32(N, K, M, accumulate):
     ops.gemm(to_dev(a), to_dev(w), c, accumulate=accumulate)
     err = (c.cpu().double() - want).abs().max().item()
     assert err <= 1e-4 * (1 + want.abs().max().item()), err   # kernels.rs:716 tolerance
+
+
+@pytest.mark.parametrize("N,K", [(1, 32), (50, 160), (17, 64), (331, 100), (96, 4100), (2048, 2048), (512, 8192), (8, 16384)])
+def test_gemm_f32_is_summed_in_one_order_by_both_kernels_and_at_every_number_of_rows(N, K):
+    """A cell's sum is cut into slices of 64 of k, each a chain of fused multiply-adds from zero, added in order
+    (``csrc/hip/gemm_f32.hip``): the skinny kernel (8 rows of W a workgroup, a lane a slice) and the tiled one give the
+    same bits, and a row of A gives the same bits alone, among 8 and among 70 rows, which is what lets batched
+    and unbatched generation agree exactly in 32-bit."""
+    from glassbox_amd import ops
+    lib = ops._lib("gemm_f32")
+    stream = torch.cuda.current_stream().cuda_stream
+    a, w = to_dev(rnd(70, K, seed=5)), to_dev(rnd(N, K, seed=6))
+    c0 = to_dev(rnd(70, N, seed=7))
+
+    def run(rows, which, accumulate):
+        c = c0[:rows].clone()
+        rc = lib.gb_gemm_f32_by(a.data_ptr(), K, w.data_ptr(), K, c.data_ptr(), N, rows, N, K, accumulate, which, stream)
+        assert rc == 0, lib.gb_last_error().decode()
+        return c.cpu()
+
+    for accumulate in (0, 1):
+        tiled = run(70, 1, accumulate)
+        want = a.cpu().double() @ w.cpu().double().T + (c0.cpu().double() if accumulate else 0)
+        assert (tiled.double() - want).abs().max().item() <= 1e-4 * (1 + want.abs().max().item())
+        for rows in (1, 2, 3, 8, 13, 16, 17, 40, 64):
+            skinny = run(rows, 2, accumulate)
+            assert torch.equal(skinny, tiled[:rows]), f"{rows} rows: the skinny kernel's bits differ from the tiled kernel's"
+            assert torch.equal(run(rows, 1, accumulate), tiled[:rows]), f"{rows} rows: the tiled kernel's bits depend on M"
+    # the skinny kernel is refused where it does not apply, not run wrongly
+    assert lib.gb_gemm_f32_by(a.data_ptr(), K, w.data_ptr(), K, c0.data_ptr(), N, 70, N, K, 0, 2, stream) == 1
+    assert "skinny" in lib.gb_last_error().decode()
+
+
+def test_gemm_f32_takes_rows_that_are_no_words_of_16_bytes():
+    """A k that is no multiple of 4, or operands that start in the middle of a word, go through the tiled kernel."""
+    from glassbox_amd import ops
+    for K, off in ((30, 0), (32, 1), (257, 0)):
+        a, w = rnd(5, K + off, seed=8), rnd(20, K + off, seed=9)
+        c = to_dev(torch.zeros(5, 20))
+        da, dw = to_dev(a)[:, off:], to_dev(w)[:, off:]
+        ops.gemm(da, dw, c)
+        want = a[:, off:].double() @ w[:, off:].double().T
+        assert (c.cpu().double() - want).abs().max().item() <= 1e-4 * (1 + want.abs().max().item())
 
 
 @pytest.mark.parametrize("N,K,M", GEMM_SHAPES_BF16)
@@ -614,6 +661,41 @@ def test_attention_plain_kernel(dtype, nh, nkv, hd, window):
     tol = 2e-5 if dtype == torch.float32 else 2 ** -7
     err = (out.cpu().double() - want).abs().max().item()
     assert err < tol, err
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("nh,nkv,hd,window,page", [(4, 2, 16, 0, 16), (8, 8, 64, 0, 16), (3, 1, 32, 0, 48), (8, 2, 128, 0, 32),
+                                                   (2, 1, 256, 0, 64), (4, 2, 32, 300, 16), (5, 5, 80, 0, 64)])
+def test_attention_plain_spread_over_workgroups_gives_the_bits_of_one_workgroup(dtype, nh, nkv, hd, window, page):
+    """With a workspace the plain kernel gives every chunk of 256 keys a workgroup and merges them in a second kernel,
+    by the same steps in the same order as one workgroup that walks them: bit for bit the same rows, and those of the
+    float64 formula.  Contexts of one chunk, of a chunk and a key, of many; a window that starts inside a page."""
+    from glassbox_amd import ops
+    ctx_lens = [1, 256, 257, 1200, 700]
+    k_pages, v_pages, tables, ks, vs = paged_setup(ctx_lens, nkv, hd, page, seed=hd + nh + page, dtype=dtype)
+    tok_seq = [0, 1, 2, 3, 4, 3, 3]
+    positions = [c - 1 for c in ctx_lens] + [600, 255]
+    n = len(tok_seq)
+    q = rnd(n, nh * hd, seed=12).to(dtype)
+    scale = 1 / math.sqrt(hd)
+    args = (torch.tensor(positions, dtype=torch.int32, device=DEV), torch.tensor(tok_seq, dtype=torch.int32, device=DEV),
+            to_dev(tables), to_dev(ops.pack_keys(k_pages)), to_dev(v_pages), nh, scale, window)
+    walked = torch.empty(n, nh * hd, device=DEV, dtype=dtype)
+    ops.attention_plain(to_dev(q), walked, *args)
+    floats = ops.attention_plain_split_floats(n, nh, hd, page, 1280)
+    assert floats > 0
+    ws = torch.full((floats,), float("nan"), device=DEV)
+    spread = torch.empty(n, nh * hd, device=DEV, dtype=dtype)
+    ops.attention_plain(to_dev(q), spread, *args, workspace=ws, max_context=1280)
+    assert torch.equal(spread, walked)
+    want = plain_attention_rows(q, ks, vs, tok_seq, positions, nh, scale, window)
+    tol = 2e-5 if dtype == torch.float32 else 2 ** -7
+    assert (walked.cpu().double() - want).abs().max().item() < tol
+    # many (token, head) pairs, or contexts of one chunk: nothing to spread
+    assert ops.attention_plain_split_floats(2000, nh, hd, page, 1280) == 0
+    assert ops.attention_plain_split_floats(n, nh, hd, page, 256) == 0
+    with pytest.raises(ops.KernelError, match="workspace"):
+        ops.attention_plain(to_dev(q), spread, *args, workspace=ws[:100], max_context=1280)
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
