@@ -203,3 +203,4 @@ extern "C" int gb_gemm_f32(const float* a, int lda, const float* w, int ldw, flo
 
 // the launches of a layer can be recorded and made again for the layers like it (common.h)
 GB_TAPED(gb_gemm_f32)
+GB_TAPED(gb_gemm_f32_by)

@@ -956,3 +956,4 @@ def test_copy_rows():
     want[4], want[0] = want[1].clone(), want[5].clone()
     ops.copy_rows(base, torch.tensor([1, 5], dtype=torch.int32, device=DEV), torch.tensor([4, 0], dtype=torch.int32, device=DEV))
     assert torch.equal(base, want)
+
