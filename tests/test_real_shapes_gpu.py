@@ -68,3 +68,41 @@ def test_parity_at_the_sizes_of_real_models(name):
             eng.cache.check_invariants()
             assert eng.cache.used_pages() == 0
             del eng
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_a_long_context_at_the_benchmark_widths_with_the_full_vocabulary(dtype):
+    """SmolLM2-1.7B's widths (two layers) with all 49,152 tokens and a context of 1,100: a prompt of 1,060 tokens in
+    portions of 512, then 40 tokens one by one across the 1,024th position (where the decode graphs change their
+    bucket and attention its split), the logits wanted at places spread over the context and at every decoded token.
+    The vocabulary product, attention over 69 pages and the 2,048-wide products together, against float64."""
+    from glassbox_amd.config import config_from_dict
+    from glassbox_amd.weights import build_model, random_tensors
+    raw = dict(SHAPES["smollm2-1.7b"], num_hidden_layers=2)
+    cfg = config_from_dict(raw)
+    tensors = random_tensors(build_model(cfg), seed=21, norm_init="uniform", device="cuda:0")
+    tensors = {n: (t.bfloat16().float() if t.dim() == 2 else t) for n, t in tensors.items()}
+    pcfg = dict(raw, head_dim=raw["hidden_size"] // raw["num_attention_heads"])
+    toks = helpers.random_tokens(raw["vocab_size"], 1100, seed=77)
+    want = plain.forward({n: t.cpu().double() for n, t in tensors.items()}, pcfg, toks).numpy()
+    places = {0: [0, 15, 16, 300, 511], 512: [0, 255, 511], 1024: [0, 20, 35]}     # first token of a portion -> wanted places
+    eng = engine_of(cfg, tensors, dtype, 1152)
+    tol = helpers.TOL_F32
+    if dtype == "bfloat16":
+        plain_engine = engine_of(cfg, tensors, "bfloat16", 1152, kernels="plain")
+        tol = helpers.Bf16Bound.measure(plain_engine, {"long": toks}, lambda r: want, label="smollm2-1.7b")
+        del plain_engine
+    for at, wanted in places.items():
+        n = min(512, 1060 - at)
+        got = eng.step([("long", toks[at:at + n], wanted)]).float().cpu().numpy()
+        for row, w in zip(got, wanted):
+            err = float(np.abs(row - want[at + w]).max())
+            assert err <= tol, f"{dtype}: position {at + w}: error {err:.3e}, allowed {tol:.3e}"
+    for p in range(1060, 1100):
+        got = eng.step([("long", [toks[p]], [0])]).float().cpu().numpy()[0]
+        err = float(np.abs(got - want[p]).max())
+        assert err <= tol, f"{dtype}: decoded position {p}: error {err:.3e}, allowed {tol:.3e}"
+    if eng.decode_graphs is not None:
+        assert eng.decode_graphs.replays > 30 and len({bucket for _, bucket in eng.decode_graphs.shapes}) == 1
+    eng.end_request("long")
+    assert eng.cache.used_pages() == 0
