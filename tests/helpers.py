@@ -117,7 +117,7 @@ def max_error(got: Dict[str, np.ndarray], folder: str, requests: Dict[str, List[
 #: tuned kernels' bound along with itself.
 PLAIN_BF16_REL: Dict[str, float] = {
     "A": 1.96e-3, "B": 4.50e-3, "C": 2.49e-3, "D": 4.95e-3, "E": 4.00e-3, "M": 7.41e-3, "W": 7.14e-3,
-    "Bx8": 2.96e-2, "Dx8": 5.01e-2, "smollm2-1.7b": 1.20e-2, "llama-3-8b": 1.29e-2,
+    "Bx8": 2.96e-2, "Dx8": 5.01e-2, "smollm2-1.7b": 1.20e-2, "llama-3-8b": 1.31e-2,
 }
 #: what this run measured, by the same labels (printed at the end of a run: conftest.pytest_terminal_summary)
 MEASURED_PLAIN_BF16_REL: Dict[str, float] = {}
