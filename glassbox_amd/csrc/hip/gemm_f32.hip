@@ -5,11 +5,17 @@
 // Every output cell is summed in one order, whatever kernel computes it and whatever else is
 // in the batch: k is cut into slices of 64; a slice's products are added in ascending k by a
 // chain of fused multiply-adds that starts from zero; the slices' sums are added in ascending
-// order.  So a cell's bits do not depend on M, on the tile it falls in, or on which of the two
+// order.  So a cell's bits do not depend on M, on the tile it falls in, or on which of the three
 // kernels ran:
 //
 //  * tiled (any sizes): a 64 x 64 tile of C a workgroup, k in steps of 16 through LDS, a thread
 //    4 x 4 cells; after every fourth step (a slice) the chain's sum goes into the cell's total.
+//  * wide (prompts; rows of 16 bytes): a 128 x 64 tile a workgroup and 8 x 4 cells a thread, so
+//    that a k-step's 32 multiply-adds of a thread stand against three 16-byte reads from LDS
+//    where the tiled kernel has 16 against two; the next k-step's operands are on their way
+//    from memory while this one is multiplied, and LDS holds two k-steps, one barrier a step.
+//    (Tiles of 128 x 128 with 8 x 8 cells leave one wave a SIMD on square products of 2,048 and
+//    were slower at every size measured.)
 //  * skinny (M <= 64, rows of 16 bytes: a decode step, a short prompt portion): the tiled kernel
 //    would start N / 64 workgroups that walk all of k one step behind the other.  Here a workgroup
 //    owns 8 rows of W and every lane one (slice, row) pair: it asks for its 64 weights at once
@@ -89,6 +95,109 @@ __global__ __launch_bounds__(256) void gemm_f32_kernel(const float* __restrict__
     }
   }
 }
+
+// ---- wide: 128 x 64 of C a workgroup, 8 x 4 cells a thread, two k-steps in LDS ------------------------------
+constexpr int WM = 128, WN = 64, WK = 16;
+static_assert(kSlice % WK == 0, "a slice is whole steps of the wide kernel");
+
+__global__ __launch_bounds__(256) void gemm_f32_wide_kernel(const float* __restrict__ a, int lda, const float* __restrict__ w,
+                                                            int ldw, float* __restrict__ c, int ldc, int M, int N, int K,
+                                                            int accumulate) {
+  constexpr int NB = WN / 64, CN = 4 * NB;   // blocks of 64 columns, columns a thread
+  __shared__ __attribute__((aligned(16))) float As[2][WK][WM + 4];
+  __shared__ __attribute__((aligned(16))) float Ws[2][WK][WN + 4];
+  const int tid = threadIdx.x;
+  const int tx = tid % 16, ty = tid / 16;
+  const int m0 = blockIdx.y * WM, n0 = blockIdx.x * WN;
+  // a thread brings word lc of the k-step's four for rows lr and lr + 64 of the operands
+  const int lr = tid / 4, lc = tid % 4;
+  f32x4 pa[2], pw[NB];
+  const f32x4 zero = {0.f, 0.f, 0.f, 0.f};
+  auto fetch = [&](int k0) {
+    const int gk = k0 + 4 * lc;   // K is whole words: a word is inside k or outside
+#pragma unroll
+    for (int h = 0; h < 2; ++h) {
+      const int gm = m0 + lr + 64 * h;
+      pa[h] = (gm < M && gk < K) ? *reinterpret_cast<const f32x4*>(a + (size_t)gm * lda + gk) : zero;
+    }
+#pragma unroll
+    for (int h = 0; h < NB; ++h) {
+      const int gn = n0 + lr + 64 * h;
+      pw[h] = (gn < N && gk < K) ? *reinterpret_cast<const f32x4*>(w + (size_t)gn * ldw + gk) : zero;
+    }
+  };
+  auto stash = [&](int buf) {
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+#pragma unroll
+      for (int h = 0; h < 2; ++h) As[buf][4 * lc + i][lr + 64 * h] = pa[h][i];
+#pragma unroll
+      for (int h = 0; h < NB; ++h) Ws[buf][4 * lc + i][lr + 64 * h] = pw[h][i];
+    }
+  };
+  // cells (ty*4 + i%4 + 64*(i/4), tx*4 + j%4 + 64*(j/4))
+  float acc[8][CN], total[8][CN];
+#pragma unroll
+  for (int i = 0; i < 8; ++i)
+#pragma unroll
+    for (int j = 0; j < CN; ++j) acc[i][j] = total[i][j] = 0.f;
+
+  const int steps = (K + WK - 1) / WK;
+  fetch(0);
+  stash(0);
+  __syncthreads();
+  for (int s = 0; s < steps; ++s) {
+    const int buf = s & 1;
+    if (s + 1 < steps) fetch((s + 1) * WK);
+#pragma unroll
+    for (int kk = 0; kk < WK; ++kk) {
+      float av[8], wv[CN];
+#pragma unroll
+      for (int h = 0; h < 2; ++h) {
+        const f32x4 x = *reinterpret_cast<const f32x4*>(&As[buf][kk][ty * 4 + 64 * h]);
+#pragma unroll
+        for (int i = 0; i < 4; ++i) av[4 * h + i] = x[i];
+      }
+#pragma unroll
+      for (int h = 0; h < NB; ++h) {
+        const f32x4 x = *reinterpret_cast<const f32x4*>(&Ws[buf][kk][tx * 4 + 64 * h]);
+#pragma unroll
+        for (int i = 0; i < 4; ++i) wv[4 * h + i] = x[i];
+      }
+#pragma unroll
+      for (int i = 0; i < 8; ++i)
+#pragma unroll
+        for (int j = 0; j < CN; ++j) acc[i][j] = fmaf(av[i], wv[j], acc[i][j]);
+    }
+    if (((s + 1) * WK) % kSlice == 0 || s + 1 == steps) {   // a slice ends: its sum joins the total
+#pragma unroll
+      for (int i = 0; i < 8; ++i)
+#pragma unroll
+        for (int j = 0; j < CN; ++j) {
+          total[i][j] += acc[i][j];
+          acc[i][j] = 0.f;
+        }
+    }
+    // the other half of LDS was last read a step ago, before the barrier that every thread has passed since
+    if (s + 1 < steps) stash(buf ^ 1);
+    __syncthreads();
+  }
+#pragma unroll
+  for (int i = 0; i < 8; ++i) {
+    const int gm = m0 + ty * 4 + (i & 3) + 64 * (i >> 2);
+    if (gm >= M) continue;
+#pragma unroll
+    for (int j = 0; j < CN; ++j) {
+      const int gn = n0 + tx * 4 + (j & 3) + 64 * (j >> 2);
+      if (gn >= N) continue;
+      float* dst = c + (size_t)gm * ldc + gn;
+      *dst = accumulate ? *dst + total[i][j] : total[i][j];
+    }
+  }
+}
+
+// the wide kernel from so many of its tiles on; below that the small tiles spread the work further
+constexpr int kWideMinTiles = 64;
 
 // ---- skinny: 8 rows of W a workgroup, a lane a (slice, row) pair ------------------------------------------
 constexpr int SR = 8;             // rows of W a workgroup
@@ -171,15 +280,16 @@ inline bool words_of_16_bytes(const void* p, int ld) { return (reinterpret_cast<
 
 }  // namespace
 
-// which = 0: the kernel the sizes call for; 1: the tiled kernel; 2: the skinny kernel (refused where it does not
-// apply).  Both give the same bits; tests compare them.
+// which = 0: the kernel the sizes call for; 1: the tiled kernel; 2: the skinny kernel; 3: the wide kernel (the last
+// two refused where they do not apply).  All give the same bits; tests compare them.
 extern "C" int gb_gemm_f32_by(const float* a, int lda, const float* w, int ldw, float* c, int ldc, int M, int N, int K,
                               int accumulate, int which, hipStream_t stream) {
   GB_REQUIRE(M >= 0 && N > 0 && K > 0, "gemm_f32: bad sizes M=%d N=%d K=%d", M, N, K);
   GB_REQUIRE(lda >= K && ldw >= K && ldc >= N, "gemm_f32: a leading dimension is shorter than its row (lda=%d ldw=%d ldc=%d)", lda, ldw, ldc);
-  GB_REQUIRE(which >= 0 && which <= 2, "gemm_f32: no kernel %d", which);
+  GB_REQUIRE(which >= 0 && which <= 3, "gemm_f32: no kernel %d", which);
   if (M == 0) return 0;
-  const bool skinny_fits = M <= kSkinnyMaxRows && K % 4 == 0 && words_of_16_bytes(a, lda) && words_of_16_bytes(w, ldw);
+  const bool words = K % 4 == 0 && words_of_16_bytes(a, lda) && words_of_16_bytes(w, ldw);
+  const bool skinny_fits = M <= kSkinnyMaxRows && words;
   GB_REQUIRE(which != 2 || skinny_fits, "gemm_f32: the skinny kernel takes at most %d rows of 16-byte words (M=%d K=%d)",
              kSkinnyMaxRows, M, K);
   if (which == 2 || (which == 0 && skinny_fits)) {
@@ -189,6 +299,13 @@ extern "C" int gb_gemm_f32_by(const float* a, int lda, const float* w, int ldw, 
     else if (M <= 8) launch_skinny<8>(a, lda, w, ldw, c, ldc, M, N, K, accumulate, stream);
     else launch_skinny<16>(a, lda, w, ldw, c, ldc, M, N, K, accumulate, stream);
     return launched("gemm_f32 (skinny)");
+  }
+  GB_REQUIRE(which != 3 || words, "gemm_f32: the wide kernel takes rows of 16-byte words (K=%d lda=%d ldw=%d)", K, lda, ldw);
+  const dim3 wide((N + WN - 1) / WN, (M + WM - 1) / WM);
+  if (which == 3 || (which == 0 && words && (long long)wide.x * wide.y >= kWideMinTiles)) {
+    GB_REQUIRE(wide.y <= 65535, "gemm_f32: M=%d needs more than 65535 row tiles", M);
+    hipLaunchKernelGGL(gemm_f32_wide_kernel, wide, dim3(256), 0, stream, a, lda, w, ldw, c, ldc, M, N, K, accumulate);
+    return launched("gemm_f32 (wide)");
   }
   const dim3 grid((N + BN - 1) / BN, (M + BM - 1) / BM);
   GB_REQUIRE(grid.y <= 65535, "gemm_f32: M=%d needs more than 65535 row tiles", M);

@@ -70,7 +70,7 @@ _SIGS = {
         # q, q_stride, out, out_stride, dtype, positions, tok_seq, tables, table_stride, k, v, n, nh, nkv, hd, page,
         # scale, window, workspace, workspace floats, max_context, stream
         "gb_attention_plain": [_vp, _i, _vp, _i, _i, _vp, _vp, _vp, _i, _vp, _vp, _i, _i, _i, _i, _i, _f, _i, _vp,
-                               C.c_longlong, _i, _vp],
+                               C.c_longlong, _i, _i, _vp],
         "gb_attention_plain_split_floats": [_i, _i, _i, _i, _i],
     },
     "attention_bf16": {
@@ -623,6 +623,10 @@ MAX_VOCAB = 1 << 20       # sampling.hip: a token id takes 20 bits of the (logit
 PLAIN_SPLIT_MAX_PAIRS = 1024   # (token, head) pairs up to which a step of long contexts goes a workgroup a chunk
 
 
+#: from so many rows of prompt portions on, ``attention_plain`` takes them eight rows a workgroup
+PLAIN_GROUP_MIN_ROWS = 64
+
+
 def attention_plain_split_floats(n: int, n_heads: int, head_dim: int, page_size: int, max_context: int) -> int:
     """Floats of workspace with which ``attention_plain`` spreads the chunks of long contexts over workgroups, or 0
     where it would not: many (token, head) pairs fill the chip by themselves, and a context of one chunk has
@@ -634,11 +638,14 @@ def attention_plain_split_floats(n: int, n_heads: int, head_dim: int, page_size:
 
 def attention_plain(q: torch.Tensor, out: torch.Tensor, positions: torch.Tensor, tok_seq: torch.Tensor,
                     tables: torch.Tensor, k_pages: torch.Tensor, v_pages: torch.Tensor, n_heads: int,
-                    scale: float, window: int = 0, workspace: Optional[torch.Tensor] = None, max_context: int = 0) -> None:
+                    scale: float, window: int = 0, workspace: Optional[torch.Tensor] = None, max_context: int = 0,
+                    grouped: bool = False) -> None:
     """Paged attention, one block per (token, head); q may be a view into the stacked qkv rows.
     ``workspace`` (float32, ``attention_plain_split_floats`` elements) with ``max_context`` (at least the most keys a
     token of the step reads): a workgroup a chunk of 256 keys and a second kernel that merges them, for steps of few
-    tokens with long contexts; the same bits as without."""
+    tokens with long contexts; the same bits as without.  ``grouped`` (without a workspace): a workgroup takes eight
+    rows and loads a key once where these are one request's consecutive tokens, for the rows of prompt portions; the
+    same bits again."""
     _dev(q, out, positions, tok_seq, tables, k_pages, v_pages)
     n = q.shape[0]
     if q.dtype != out.dtype:
@@ -658,7 +665,8 @@ def attention_plain(q: torch.Tensor, out: torch.Tensor, positions: torch.Tensor,
     _launch(lib, lib.gb_attention_plain, _p(q), _rows(q, "q"), _p(out), _rows(out, "out"), dtype_code(q), _p(positions),
                                        _p(tok_seq), _p(tables), tables.stride(0), _p(k_pages), _p(v_pages), n,
                                        n_heads, nkv, hd, page_size, float(scale), int(window), _p(workspace),
-                                       workspace.numel() if workspace is not None else 0, int(max_context), _stream())
+                                       workspace.numel() if workspace is not None else 0, int(max_context),
+                                       1 if grouped else 0, _stream())
 
 
 def tuned_attention_supports(k_pages: torch.Tensor, n_heads: int, window: int) -> bool:

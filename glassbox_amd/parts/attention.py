@@ -27,13 +27,25 @@ def paged_attention(ctx, q: torch.Tensor, out: torch.Tensor, cache: LayerCache, 
     one row go to the split-context decode kernel, longer portions to the matrix-core prefill kernel; a step
     with ``ctx.tuned`` off takes the plain kernel throughout."""
     if ctx.dtype == torch.float32 or not ctx.tuned or not ops.tuned_attention_supports(cache.k_pages, n_heads, window):
-        # few tokens with long contexts (a decode step): a workgroup a chunk of the context, merged by a second kernel
         longest = int(ctx.host["max_context"])
         _, _, n_pieces, page_size, piece = cache.k_pages.shape
-        floats = ops.attention_plain_split_floats(q.shape[0], n_heads, n_pieces * piece, page_size, longest)
-        ws = ctx.buffer("attention_plain_parts", (floats,), torch.float32) if floats else None
-        ops.attention_plain(q, out, ctx.positions, ctx.tok_seq, ctx.tables[cache.group], cache.k_pages, cache.v_pages,
-                            n_heads, scale, window, workspace=ws, max_context=longest)
+        tables = ctx.tables[cache.group]
+
+        def rows(a, b, grouped):
+            # few tokens with long contexts (a decode step): a workgroup a chunk of the context, merged by a second kernel
+            floats = 0 if grouped else ops.attention_plain_split_floats(b - a, n_heads, n_pieces * piece, page_size, longest)
+            ws = ctx.buffer("attention_plain_parts", (floats,), torch.float32) if floats else None
+            ops.attention_plain(q[a:b], out[a:b], ctx.positions[a:b], ctx.tok_seq[a:b], tables, cache.k_pages, cache.v_pages,
+                                n_heads, scale, window, workspace=ws, max_context=longest, grouped=grouped)
+
+        # the rows of requests with one token come first; many rows of prompt portions go eight rows a workgroup
+        n, n_decode = q.shape[0], ctx.host["n_decode"]
+        if n - n_decode >= ops.PLAIN_GROUP_MIN_ROWS and window == 0:
+            if n_decode > 0:
+                rows(0, n_decode, False)
+            rows(n_decode, n, True)
+        else:
+            rows(0, n, False)
         return
     n_decode = ctx.host["n_decode"]
     if n_decode > 0:

@@ -82,6 +82,31 @@ def test_gemm_f32_is_summed_in_one_order_by_both_kernels_and_at_every_number_of_
     assert "skinny" in lib.gb_last_error().decode()
 
 
+@pytest.mark.parametrize("N,K,M", [(331, 100, 200), (130, 260, 129), (2048, 2048, 300), (512, 8192, 65), (96, 4100, 331),
+                                   (257, 16, 128), (128, 72, 1)])
+def test_gemm_f32_wide_kernel_gives_the_bits_of_the_tiled_kernel(N, K, M):
+    """The kernel for prompts (128 x 64 of C a workgroup, 8 x 4 cells a thread, two k-steps in LDS) keeps the one
+    summation order: the same bits as the tiled kernel, with and without accumulation, on tiles that hang over
+    every edge; and it is refused where rows are no 16-byte words."""
+    from glassbox_amd import ops
+    lib = ops._lib("gemm_f32")
+    stream = torch.cuda.current_stream().cuda_stream
+    a, w, c0 = to_dev(rnd(M, K, seed=11)), to_dev(rnd(N, K, seed=12)), to_dev(rnd(M, N, seed=13))
+    for accumulate in (0, 1):
+        got = {}
+        for which in (1, 3):
+            c = c0.clone()
+            rc = lib.gb_gemm_f32_by(a.data_ptr(), K, w.data_ptr(), K, c.data_ptr(), N, M, N, K, accumulate, which, stream)
+            assert rc == 0, lib.gb_last_error().decode()
+            got[which] = c.cpu()
+        want = a.cpu().double() @ w.cpu().double().T + (c0.cpu().double() if accumulate else 0)
+        assert (got[1].double() - want).abs().max().item() <= 1e-4 * (1 + want.abs().max().item())
+        assert torch.equal(got[3], got[1]), "the wide kernel's bits differ from the tiled kernel's"
+    if K > 4:
+        assert lib.gb_gemm_f32_by(a.data_ptr() + 4, K, w.data_ptr(), K, c0.data_ptr(), N, M, N, K - 4, 0, 3, stream) == 1
+        assert "wide" in lib.gb_last_error().decode()
+
+
 def test_gemm_f32_takes_rows_that_are_no_words_of_16_bytes():
     """A k that is no multiple of 4, or operands that start in the middle of a word, go through the tiled kernel."""
     from glassbox_amd import ops
@@ -696,6 +721,44 @@ def test_attention_plain_spread_over_workgroups_gives_the_bits_of_one_workgroup(
     assert ops.attention_plain_split_floats(n, nh, hd, page, 256) == 0
     with pytest.raises(ops.KernelError, match="workspace"):
         ops.attention_plain(to_dev(q), spread, *args, workspace=ws[:100], max_context=1280)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("nh,nkv,hd,page", [(4, 2, 16, 16), (8, 8, 64, 16), (3, 1, 32, 48), (2, 1, 128, 32), (2, 2, 256, 16),
+                                            (5, 5, 80, 64)])
+def test_attention_plain_eight_rows_a_workgroup_gives_the_bits_of_one_row_a_workgroup(dtype, nh, nkv, hd, page):
+    """Many rows of prompt portions go eight rows a workgroup, which loads a key once where the eight are one request's
+    consecutive tokens: bit for bit the rows of the one-row form.  Portions that start and end inside a group of
+    eight, a group across the edge of a chunk of 256 keys (its first tokens have no key in the last chunk), single
+    decoded tokens between portions; a head size and page for which the form is not built takes the one-row form."""
+    from glassbox_amd import ops
+    ctx_lens = [120, 263, 701, 531, 40]
+    k_pages, v_pages, tables, ks, vs = paged_setup(ctx_lens, nkv, hd, page, seed=hd + nh + page + 1, dtype=dtype)
+    rows = ([(0, p) for p in range(0, 101)]            # 101 rows: the next portion starts inside a group
+            + [(1, p) for p in range(251, 262)]        # across key 256 in the middle of a group
+            + [(2, 700)]                               # a decoded token
+            + [(3, p) for p in range(509, 531)]        # across key 512
+            + [(4, p) for p in range(0, 40)] + [(1, 262)])
+    tok_seq, positions = [r[0] for r in rows], [r[1] for r in rows]
+    n = len(rows)
+    q = rnd(n, nh * hd, seed=14).to(dtype)
+    scale = 1 / math.sqrt(hd)
+    pos_d, seq_d = torch.tensor(positions, dtype=torch.int32, device=DEV), torch.tensor(tok_seq, dtype=torch.int32, device=DEV)
+    rest = (to_dev(tables), to_dev(ops.pack_keys(k_pages)), to_dev(v_pages), nh, scale, 0)
+    qd = to_dev(q)
+    grouped = torch.empty(n, nh * hd, device=DEV, dtype=dtype)
+    ops.attention_plain(qd, grouped, pos_d, seq_d, *rest, grouped=True)
+    single = torch.empty(n, nh * hd, device=DEV, dtype=dtype)
+    ops.attention_plain(qd, single, pos_d, seq_d, *rest)
+    # the groups of eight fall elsewhere when the step's rows start at another row
+    shifted = torch.empty(n, nh * hd, device=DEV, dtype=dtype)
+    ops.attention_plain(qd[:3], shifted[:3], pos_d[:3], seq_d[:3], *rest, grouped=True)
+    ops.attention_plain(qd[3:], shifted[3:], pos_d[3:], seq_d[3:], *rest, grouped=True)
+    assert torch.equal(shifted, single)
+    assert torch.equal(grouped, single)
+    want = plain_attention_rows(q, ks, vs, tok_seq, positions, nh, scale, 0)
+    tol = 2e-5 if dtype == torch.float32 else 2 ** -7
+    assert (grouped.cpu().double() - want).abs().max().item() < tol
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
