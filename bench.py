@@ -4,9 +4,10 @@
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--batch 8] [--context 4096] [--layers 24]
                     [--shapes smollm2-1.7b|smollm2-360m|llama-3-8b] [--reps 3]
 
-A step is one decode step of the whole batch through the path that generation uses: ``Engine.step`` (which
-replays steps of single tokens from HIP graphs) and the device sampler (``sampling.sample_rows``), the sampled
-tokens fed back as the next step's input.  The batch is first prefilled (through the same step function, in
+A step is one decode step of the whole batch through the path that greedy generation uses: ``Engine.step`` (which
+replays steps of single tokens from HIP graphs) and the device sampler (``sampling.greedy_pending``), the sampled
+tokens fed back as the next step's input: the step takes them from the device and the host reads every one of
+them while it runs (``--read-back-first`` reads them before the next step is launched, as a sampler that draws does).  The batch is first prefilled (through the same step function, in
 portions of 2,048 tokens) so that the last timed step reaches the context length.  K steps are timed ``--reps``
 times in a row, each time between synchronisations; ``ms_per_step`` and ``value`` are the mean over the
 repetitions and ``reps`` holds their spread; the batch 1 and 64 points are repeated as often, with their spread
@@ -61,6 +62,8 @@ def main() -> int:
     ap.add_argument("--page-size", type=int, default=16, help="tokens a page of the cache (16 as in the reference)")
     ap.add_argument("--reps", type=int, default=3, help="times the K timed steps are repeated (mean and spread are reported)")
     ap.add_argument("--no-scheduler", action="store_true", help="skip the figure through Scheduler.step")
+    ap.add_argument("--read-back-first", action="store_true",
+                    help="read a step's sampled tokens back before the next step is launched")
     ap.add_argument("--prefill-tokens", type=int, default=PREFILL_TOKENS,
                     help="with --only prefill, for profiling: a prompt of another length than the 2,048 tokens of the record")
     a = ap.parse_args()
@@ -75,7 +78,7 @@ def main() -> int:
     from glassbox_amd.config import config_from_dict
     from glassbox_amd.engine import Engine
     from glassbox_amd.engine import Scheduler, SchedulerConfig
-    from glassbox_amd.sampling import SamplerConfig, sample_rows
+    from glassbox_amd.sampling import SamplerConfig, greedy_pending, sample_rows
     from glassbox_amd.weights import build_model, init_random
 
     MODEL = SHAPES[a.shapes]
@@ -151,13 +154,17 @@ def main() -> int:
             n = min(PREFILL_TOKENS, start - 1 - at)
             for name, p in zip(names, prompts):
                 eng.step([(name, p[at:at + n], [])])
-        greedy_rows, uniforms = [SamplerConfig()] * batch, [0.0] * batch
         tokens = [p[-1] for p in prompts]
 
         def one_step():
             nonlocal tokens
+            # the sampled tokens stay on the device for the next step, which is launched before the host has their
+            # values; Engine.step waits for them after the launch (the cache manager keeps every request's tokens)
             logits = eng.step([(name, [t], [0]) for name, t in zip(names, tokens)])
-            tokens, _ = sample_rows(logits, greedy_rows, uniforms)     # reads the tokens back: the step has ended
+            if a.read_back_first:
+                tokens, _ = sample_rows(logits, [SamplerConfig()] * batch, [0.0] * batch)
+            else:
+                tokens = greedy_pending(logits)
 
         for _ in range(warmup):
             one_step()
@@ -239,7 +246,7 @@ def main() -> int:
                  "sd_ms": round(statistics.stdev(ms), 4) if len(ms) > 1 else 0.0},
         "meta": {"gpu": torch.cuda.get_device_name(0), "commit": source_version(),
                  "date": datetime.datetime.now(datetime.timezone.utc).strftime("%Y-%m-%dT%H:%M:%SZ"),
-                 "torch": torch.__version__, "path": "Engine.step + sampling.sample_rows"},
+                 "torch": torch.__version__, "path": "Engine.step + sampling." + ("sample_rows" if a.read_back_first else "greedy_pending")},
         "prefill": prefill,
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": PEAK["hbm_gbs"], "unit": "GB/s",
                      "frac": round(achieved / PEAK["hbm_gbs"], 4)},

@@ -7,7 +7,7 @@ from __future__ import annotations
 
 import ctypes as C
 from dataclasses import dataclass
-from typing import List, Sequence, Tuple
+from typing import List, Optional, Sequence, Tuple
 
 from .. import build
 
@@ -57,7 +57,7 @@ def _host():
             fn.restype = C.c_int
         lib.gbh_cache_decode_rows.restype = C.c_int
         lib.gbh_cache_decode_rows.argtypes = [C.c_void_p, C.POINTER(C.c_int64), C.c_int, C.c_int] + [C.c_void_p] * 2 + \
-                                             [C.c_void_p, C.c_int, C.c_void_p, C.c_int]
+                                             [C.c_void_p, C.c_int, C.c_void_p, C.c_int, C.POINTER(C.c_int32)]
         lib.gbh_cache_max_len.restype = C.c_int
         lib.gbh_cache_max_len.argtypes = [C.c_void_p, C.POINTER(C.c_int64), C.c_int]
         lib.gbh_cache_max_pages.restype = C.c_int
@@ -189,14 +189,17 @@ class CacheManager:
         return n
 
     def decode_rows(self, seq_ids: Sequence[int], stride: int, pos_ptr: int, state_ptr: int, rows_ptr: int,
-                    rows_gap: int, tables_ptr: int, tables_gap: int) -> None:
+                    rows_gap: int, tables_ptr: int, tables_gap: int, ahead: Optional[Sequence[int]] = None) -> None:
         """For requests that bring one token each, writes into the caller's int32 arrays (given as addresses, for
         instance of a pinned buffer): each request's length and state slot, and per group the cache row of the new
         token ([group][request], ``rows_gap`` entries between groups) and the block table padded with -1 to
-        ``stride`` entries ([group][request][stride], ``tables_gap`` entries between groups)."""
+        ``stride`` entries ([group][request][stride], ``tables_gap`` entries between groups).  ``ahead[i]``: tokens
+        of request i that an earlier step brought and that are not committed yet; the new token lies that far beyond
+        the request's length."""
         ids = (C.c_int64 * max(1, len(seq_ids)))(*seq_ids)
+        far = (C.c_int32 * max(1, len(seq_ids)))(*ahead) if ahead is not None else None
         rc = self._lib.gbh_cache_decode_rows(self._h, ids, len(seq_ids), stride, pos_ptr, state_ptr, rows_ptr,
-                                             rows_gap, tables_ptr, tables_gap)
+                                             rows_gap, tables_ptr, tables_gap, far)
         if rc:
             raise CacheError({-1: "unknown request", -2: f"a block table is longer than {stride} pages",
                               -3: "the page of a new token is not reserved"}.get(rc, f"error {rc}"))

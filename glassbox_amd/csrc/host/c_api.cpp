@@ -55,13 +55,17 @@ int gbh_cache_table(void* h, int64_t id, int group, int32_t* out, int cap) {
 // block table, padded with -1 to `stride` entries.  rows and tables are laid out [group][request] and
 // [group][request][stride], with `group_gap` entries from one group's array to the next.  Returns 0; -1 for an
 // unknown request; -2 if a table is longer than stride; -3 if the page of the new position is not reserved.
+// ahead (may be null): tokens of request i that an earlier step has brought and that are not committed yet; the
+// new token's position lies that many beyond the request's length (a step launched before the one before it
+// has been accounted for).
 int gbh_cache_decode_rows(void* h, const int64_t* ids, int n, int stride, int32_t* pos, int32_t* state_slot,
-                          int32_t* rows, int rows_gap, int32_t* tables, int tables_gap) {
+                          int32_t* rows, int rows_gap, int32_t* tables, int tables_gap, const int32_t* ahead) {
   auto* cm = (CacheManager*)h;
   const int page = cm->page_size(), groups = cm->num_groups();
   for (int i = 0; i < n; ++i) {
     int len = cm->seq_len(ids[i]);
     if (len < 0) return -1;
+    if (ahead) len += ahead[i];
     pos[i] = len;
     state_slot[i] = cm->state_slot(ids[i]);
     for (int g = 0; g < groups; ++g) {

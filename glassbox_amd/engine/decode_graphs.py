@@ -24,10 +24,11 @@ import contextlib
 import gc
 import weakref
 from collections import OrderedDict
-from typing import List, Sequence, Tuple
+from typing import List, Optional, Sequence, Tuple
 
 import torch
 
+from ..sampling.pending import PendingToken, place_pending
 from .context import StepContext, Workspace
 
 BUCKET = 1024
@@ -132,14 +133,16 @@ class DecodeGraphs:
             raise RuntimeError("the engine of these graphs is gone")
         return eng
 
-    def run(self, entries: Sequence[Tuple[int, List[int], List[int]]]) -> torch.Tensor:
+    def run(self, entries: Sequence[Tuple[int, List[int], List[int]]], ahead: Optional[Sequence[int]] = None) -> torch.Tensor:
+        """``ahead[i]``: tokens that request i brought in a step before this one and that the cache manager has not
+        been told of yet (that step is still running, its pages are reserved): this step's token lies behind them."""
         eng = self.engine
         cache = eng.cache
         n = len(entries)
         sids = [e[0] for e in entries]
         # the shape's tables must hold the longest table, which pages of an uncommitted reservation (a step that
-        # found no room for a later entry) can make longer than the lengths need
-        longest = max(cache.max_len(sids) + 1, cache.max_pages(sids) * eng.page_size)
+        # found no room for a later entry, a step that runs ahead) can make longer than the lengths need
+        longest = max(cache.max_len(sids) + 1 + (max(ahead) if ahead else 0), cache.max_pages(sids) * eng.page_size)
         key = (padded_rows(n), context_bucket(longest))
         shape = self.shapes.get(key)
         if shape is None:
@@ -152,11 +155,15 @@ class DecodeGraphs:
         shape.copied.synchronize()           # the last copy out of the pinned buffer has run
         hv = shape.host.numpy()
         hv[:] = shape.filler
-        shape.h_tok[:n] = [e[1][0] for e in entries]
+        toks = [e[1][0] for e in entries]
+        late = [(i, t) for i, t in enumerate(toks) if isinstance(t, PendingToken)]   # still on the device
+        shape.h_tok[:n] = [0 if isinstance(t, PendingToken) else t for t in toks] if late else toks
         cache.decode_rows(sids, shape.stride, shape.pos_ptr, shape.state_ptr, shape.rows_ptr, shape.rows,
-                          shape.tables_ptr, shape.tables_gap)
+                          shape.tables_ptr, shape.tables_gap, ahead)
         shape.dev.copy_(shape.host, non_blocking=True)
         shape.copied.record()
+        if late:
+            place_pending(shape.dev, late)   # token ids are the first rows of the layout
         loads = getattr(eng.model, "loads", 0)
         if self.workspace.epoch != self.epoch or loads != self.loads:
             # a buffer was replaced by a larger one, or the weights by another loading of them, since graphs were

@@ -14,12 +14,15 @@ import torch
 from .. import ops
 from ..cache.manager import FULL, CacheManager, GroupSpec, OutOfPages
 from ..parts.base import LayerCache
+from ..sampling.pending import PendingToken, place_pending, token_values
 from ..config import config_from_dir
 from ..weights.loader import build_model, compute_dtype, load_weights
 from .context import StepContext, Workspace
 from .decode_graphs import DecodeGraphs
 
-Entry = Tuple[Hashable, Sequence[int], Sequence[int]]  # (request, its next tokens, wanted places among them)
+# (request, its next tokens, wanted places among them); a token may be a sampling.PendingToken, which the step takes
+# from the device
+Entry = Tuple[Hashable, Sequence[int], Sequence[int]]
 
 
 class EngineError(RuntimeError):
@@ -250,7 +253,11 @@ class Engine:
 
         Reserves pages (raising OutOfPages if the pool is too small), runs, commits.  Returns
         float32 logits [wanted, vocab] in the order of the entries and of their wanted places.
-        The tensor is a view of the engine's workspace: use it before the next step."""
+        The tensor is a view of the engine's workspace: use it before the next step.
+
+        A token may be a ``sampling.PendingToken`` (what ``sampling.greedy_pending`` left on the device): the step is
+        launched with it, and its value is waited for only afterwards, for the cache manager's record of the
+        request's tokens; a decoding loop then keeps the GPU one step behind the host, with no pause between steps."""
         entries = [(r, list(t), list(w)) for r, t, w in entries]
         seen = set()
         for request, _, _ in entries:
@@ -262,7 +269,7 @@ class Engine:
         by_id = [(self._ids[r], t, w) for r, t, w in entries]
         logits = self.run_reserved(by_id, validated=True)
         for sid, tokens, _ in by_id:
-            self.cache.commit(sid, tokens)
+            self.cache.commit(sid, token_values(tokens))   # (pending values: waits for the step before this one)
         return logits
 
     def _validate(self, entries) -> None:
@@ -270,14 +277,19 @@ class Engine:
         for request, tokens, want in entries:
             if not tokens:
                 raise EngineError(f"request {request!r} brings no tokens")
-            if min(tokens) < 0 or max(tokens) >= vocab:
+            known = [t for t in tokens if not isinstance(t, PendingToken)]   # a sampler's tokens lie below the vocabulary
+            if known and (min(known) < 0 or max(known) >= vocab):
                 raise EngineError(f"request {request!r}: token ids must lie in 0..{vocab - 1}")
             if any(w < 0 or w >= len(tokens) for w in want):
                 raise EngineError(f"request {request!r}: wanted places must lie among its {len(tokens)} tokens")
 
-    def run_reserved(self, entries: Sequence[Tuple[int, List[int], List[int]]], validated: bool = False) -> torch.Tensor:
+    def run_reserved(self, entries: Sequence[Tuple[int, List[int], List[int]]], validated: bool = False,
+                     ahead: Optional[Sequence[int]] = None) -> torch.Tensor:
         """The step itself, on the cache manager's own request numbers: pages for the tokens are
-        reserved already and nothing is committed (the scheduler does both around this call)."""
+        reserved already and nothing is committed (the scheduler does both around this call).
+
+        ``ahead`` (see ``runs_ahead``): request i has brought ``ahead[i]`` tokens in a step that is not committed
+        yet; this step's single token lies behind them, and pages up to there are reserved."""
         if not entries:
             return torch.empty((0, self.model.vocab_size), dtype=torch.float32, device=self.device)
         if not validated:
@@ -285,10 +297,20 @@ class Engine:
         self._apply_copies()
         self.steps += 1
         graphs = self.decode_graphs
+        if ahead is not None:
+            if not self.runs_ahead(entries):
+                raise EngineError("only a step of single tokens, replayed from a graph, can run ahead of the step before it")
+            return graphs.run(entries, ahead)
         if graphs is not None and graphs.applies(entries):
             return graphs.run(entries)
         ctx = self._build_context(entries)
         return self.model.forward(ctx, self.layers)
+
+    def runs_ahead(self, entries) -> bool:
+        """Whether this step can be launched before the step before it is committed: one token a request with the
+        logits after it (the steps that graphs replay, whose metadata the cache manager writes for a position beyond
+        the committed length), and no state of a request's own that a step launched in vain would leave changed."""
+        return self.decode_graphs is not None and not self.has_state and self.decode_graphs.applies(entries)
 
     def reset_state(self, sid: int) -> None:
         """Sets the state slot of a request that starts (again) from its first token to its initial value."""
@@ -333,8 +355,13 @@ class Engine:
             stride = need   # a request holds more pages than its tokens need
         hv = staged.numpy()
         tok = hv[:n]
+        late = []   # (row, pending token): placed on the device after the copy
         for s, ei in enumerate(order):
-            tok[q_start[s]:q_start[s] + q_len[s]] = entries[ei][1]
+            toks = entries[ei][1]
+            if any(isinstance(t, PendingToken) for t in toks):
+                late += [(q_start[s] + j, t) for j, t in enumerate(toks) if isinstance(t, PendingToken)]
+                toks = [0 if isinstance(t, PendingToken) else t for t in toks]
+            tok[q_start[s]:q_start[s] + q_len[s]] = toks
         hv[3 * n + S:3 * n + 2 * S] = q_len
         hv[3 * n + 4 * S:o_rows] = want_rows
         state_slots = hv[3 * n + 3 * S:3 * n + 4 * S].tolist()
@@ -342,6 +369,8 @@ class Engine:
             self._meta_dev = torch.empty(max(total * 2, 4096), dtype=torch.int32, device=self.device)
         dev = self._meta_dev
         dev[:total].copy_(staged, non_blocking=True)
+        if late:
+            place_pending(dev, late)
         cut = lambda off, count: dev[off:off + count]
         slots = [cut(o_rows + g * n, n) for g in range(G)]
         tables = [cut(o_rows + G * n + g * S * stride, S * stride).view(S, stride) for g in range(G)]

@@ -12,7 +12,8 @@ from typing import List, Optional, Sequence, Union
 
 import torch
 
-from ..sampling.sampler import Sampler, SamplerConfig, sample_rows
+from ..sampling.pending import token_values
+from ..sampling.sampler import SamplerConfig, greedy_pending
 from .engine import Engine
 from .scheduler import Scheduler, SchedulerConfig
 
@@ -27,10 +28,11 @@ class Generator:
         engine.add_request(name)
 
     def feed(self, tokens: Sequence[int]) -> torch.Tensor:
-        """Appends tokens and returns the logits after the last one (float32 [vocab] on the GPU)."""
+        """Appends tokens and returns the logits after the last one (float32 [vocab] on the GPU).  A token may be
+        one that a sampler left on the device (``sampling.PendingToken``)."""
         toks = list(tokens)
         logits = self.engine.step([(self.name, toks, [len(toks) - 1])])
-        self.tokens.extend(toks)
+        self.tokens.extend(token_values(toks))   # (the step has read pending values back already)
         return logits[0]
 
     def truncate(self, length: int) -> None:
@@ -50,13 +52,13 @@ def greedy(engine: Engine, prompt: Sequence[int], n: int) -> List[int]:
     g = Generator(engine, name=("greedy", id(prompt), len(prompt)))
     try:
         logits = g.feed(prompt)
-        out: List[int] = []
-        greedy_cfg = [SamplerConfig()]
+        out = []
         for _ in range(n):
-            toks, _ = sample_rows(logits.reshape(1, -1), greedy_cfg, [0.0])
-            out.append(toks[0])
-            logits = g.feed([toks[0]])
-        return out
+            # the token stays on the device for the next step; its value is read while that step runs
+            token = greedy_pending(logits.reshape(1, -1))[0]
+            out.append(token)
+            logits = g.feed([token])
+        return token_values(out)
     finally:
         g.close()
 

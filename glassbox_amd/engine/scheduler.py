@@ -17,7 +17,9 @@ from dataclasses import dataclass, field
 from typing import Dict, List, Optional, Sequence, Tuple
 
 from .. import build
-from ..sampling.sampler import SamplerConfig, sample_rows
+from ..cache.manager import OutOfPages
+from ..sampling.pending import PendingToken, PendingTokens, token_values
+from ..sampling.sampler import SamplerConfig, greedy_pending, sample_rows
 
 STOP, LENGTH, ABORTED = 0, 1, 2
 FINISH_NAMES = {STOP: "stop", LENGTH: "length", ABORTED: "aborted"}
@@ -64,6 +66,8 @@ class SchedulerConfig:
     """scheduler.rs:54-74.  The number of pages is the engine's (its ``max_tokens``)."""
     token_budget: int = 256
     max_seqs: int = 32
+    #: launch the step that is bound to follow a greedy decoding step before this one's tokens are read (``Scheduler.step``)
+    run_ahead: bool = True
 
 
 @dataclass
@@ -85,6 +89,16 @@ class StepRecord:
     kv_used: int
 
 
+@dataclass
+class _Ahead:
+    """A step launched before the step before it was accounted for: the request of each row, the position and the
+    (pending) token it ran with, and what it sampled."""
+    row_of: Dict[int, int]
+    positions: List[int]
+    inputs: List[PendingToken]
+    sampled: PendingTokens
+
+
 class Scheduler:
     def __init__(self, engine, config: Optional[SchedulerConfig] = None, trace: bool = False, sample_fn=None):
         self.engine = engine
@@ -97,6 +111,11 @@ class Scheduler:
         max_pos = getattr(engine.model.config, "max_position_embeddings", 1 << 30)
         self._h = C.c_void_p(self._lib.gbh_sched_create(engine.cache.handle, self.config.token_budget,
                                                         self.config.max_seqs, max_pos))
+        self._max_pos = max_pos
+        self._ahead: Optional[_Ahead] = None
+        #: rows launched ahead of their plan, and how many of them a plan then took
+        self.ahead_rows = {"launched": 0, "served": 0}
+        self._limits: Dict[int, Tuple[int, int]] = {}    # request -> (tokens it may generate, tokens of its prompt)
         self.outputs: Dict[int, RequestOutput] = {}
         self.trace: Optional[List[StepRecord]] = [] if trace else None
         self._steps = 0
@@ -131,6 +150,7 @@ class Scheduler:
         rid = self._lib.gbh_sched_submit(self._h, p, len(prompt), max_tokens, s.temperature, s.top_k, s.top_p,
                                          s.min_p, s.repetition_penalty, s.seed, st, len(stop))
         self.outputs[rid] = RequestOutput(prompt_tokens=len(prompt))
+        self._limits[rid] = (max_tokens, len(prompt))
         self._arrival[rid] = time.perf_counter() if arrival is None else arrival
         return rid
 
@@ -149,9 +169,22 @@ class Scheduler:
 
     # ---------------------------------------------------------------------- step
     def step(self) -> bool:
-        """One batch through the model.  False when there was nothing to do (scheduler.rs:239)."""
+        """One batch through the model.  False when there was nothing to do (scheduler.rs:239).
+
+        The host library knows a step's sampled tokens only when ``finish`` is told them, and plans the next step
+        from them; with nothing else done, the GPU would wait between steps for the read-back, the bookkeeping, the
+        plan and the launch.  So when every live request decodes greedily, the step that is bound to follow (one
+        token for each request that goes on, the token taken from the device: ``sampling.PendingToken``) is
+        launched *before* this step's tokens are read, beyond the pages and positions of this step
+        (``Engine.run_reserved(..., ahead=...)``).  The next call plans as ever and finds the rows it needs already
+        computed: an entry is served by a row that ran ahead if it is the same request at the same position with the
+        same token; what the plan holds besides (a new request's prompt) runs as a launch of its own, and rows
+        that ran ahead for nothing (the request stopped, was aborted or preempted) are dropped.  Every request's
+        tokens are those of the plain sequence; where the pool is nearly full a waiting request may be admitted a step
+        later than there, because the pages of the rows that ran ahead are taken before the plan looks for room."""
         t0 = time.perf_counter()
         lib, h = self._lib, self._h
+        before, self._ahead = self._ahead, None
         rc = lib.gbh_sched_plan(h)
         if rc != 1:
             finished = self._drain_events()
@@ -166,50 +199,119 @@ class Scheduler:
                                meta[3].ctypes.data, flat.ctypes.data)
         ids, (starts, counts, wants, decodes), flat = ids.tolist(), meta.tolist(), flat.tolist()
         entries, batch_desc, at = [], [], 0
+        served: Dict[int, int] = {}      # entry -> row of the step that ran ahead
         for i in range(n):
-            if starts[i] == 0:
+            toks = flat[at:at + counts[i]]
+            j = before.row_of.get(ids[i]) if before is not None else None
+            if (j is not None and counts[i] == 1 and wants[i] and starts[i] == before.positions[j]
+                    and toks[0] == before.inputs[j].value()):
+                served[i] = j
+            elif starts[i] == 0:
                 self.engine.reset_state(ids[i])
-            entries.append((ids[i], flat[at:at + counts[i]], [counts[i] - 1] if wants[i] else []))
+            entries.append((ids[i], toks, [counts[i] - 1] if wants[i] else []))
             batch_desc.append((ids[i], "decode" if decodes[i] else "prefill", counts[i]))
             at += counts[i]
         # prompt ids were checked when the request was submitted and sampled ids lie below the vocabulary by construction
-        logits = self.engine.run_reserved(entries, validated=True)
-        rows = logits.shape[0]
+        self.ahead_rows["served"] += len(served)
+        rest = [e for i, e in enumerate(entries) if i not in served]
+        logits = self.engine.run_reserved(rest, validated=True)
+        wanted = [i for i in range(n) if wants[i]]                  # the entry of every row
+        rest_rows = [r for r, i in enumerate(wanted) if i not in served]
+        rows = len(wanted)
         # sampling parameters of every wanted row: temperature, top_p, min_p, penalty, uniform | top_k, skip
         fl, it = np.empty((5, max(1, rows)), np.float32), np.empty((2, max(1, rows)), np.int32)
         lib.gbh_sched_rows_params(h, rows, fl[0].ctypes.data, it[0].ctypes.data, fl[1].ctypes.data, fl[2].ctypes.data,
                                   fl[3].ctypes.data, fl[4].ctypes.data, it[1].ctypes.data)
         temp, top_p, min_p, penalty, uniforms = (a[:rows] for a in fl.tolist())
         top_k = it[0].tolist()[:rows]
-        if self.sample_fn is sample_rows and rows and max(temp) <= 0.0 and all(p == 1.0 for p in penalty):
-            configs, more = self._greedy[:rows] if rows <= len(self._greedy) else [SamplerConfig()] * rows, ()
-        else:
-            configs = [SamplerConfig(temp[j], top_k[j], top_p[j], min_p[j], penalty[j]) for j in range(rows)]
-            if self.sample_fn is sample_rows:
-                # the native scheduler keeps count of every such request's tokens: (row, token, occurrences, penalty)
-                m = lib.gbh_sched_penalty_pairs(h, None, None, None, None, 0) if any(p != 1.0 for p in penalty) else 0
-                pairs = np.empty((4, m), np.int32)
-                if m:
-                    lib.gbh_sched_penalty_pairs(h, pairs[0].ctypes.data, pairs[1].ctypes.data, pairs[2].ctypes.data,
-                                                pairs[3].ctypes.data, m)
-                more = (None, pairs)
+        greedy = bool(rows) and max(temp) <= 0.0 and all(p == 1.0 for p in penalty)
+        tokens: List = [None] * rows      # ints, or tokens still on the device
+        cands = [1] * rows
+        for r, i in enumerate(wanted):
+            if i in served:
+                tokens[r] = before.sampled[served[i]]
+        if rest_rows:
+            pick = lambda a: [a[r] for r in rest_rows]
+            if self.sample_fn is sample_rows and greedy:
+                got, more = greedy_pending(logits), None
+            elif self.sample_fn is sample_rows and max(pick(temp)) <= 0.0 and all(p == 1.0 for p in pick(penalty)):
+                k = len(rest_rows)
+                got, more = self.sample_fn(logits, self._greedy[:k] if k <= len(self._greedy) else [SamplerConfig()] * k,
+                                           pick(uniforms)), ()
             else:
-                contexts = []
-                for j in range(rows):
-                    if penalty[j] != 1.0:
-                        m = lib.gbh_sched_row_context(h, j, None, 0)
-                        cb = (C.c_int32 * max(1, m))()
-                        lib.gbh_sched_row_context(h, j, cb, m)
-                        contexts.append(list(cb[:m]))
-                    else:
-                        contexts.append([])
-                more = (contexts,)
-        tokens, cands = self.sample_fn(logits, configs, uniforms, *more) if rows else ([], [])
+                configs = [SamplerConfig(temp[r], top_k[r], top_p[r], min_p[r], penalty[r]) for r in rest_rows]
+                if self.sample_fn is sample_rows:
+                    # the native scheduler keeps count of every such request's tokens: (row, token, occurrences, penalty)
+                    m = lib.gbh_sched_penalty_pairs(h, None, None, None, None, 0) if any(p != 1.0 for p in penalty) else 0
+                    pairs = np.empty((4, m), np.int32)
+                    if m:
+                        lib.gbh_sched_penalty_pairs(h, pairs[0].ctypes.data, pairs[1].ctypes.data, pairs[2].ctypes.data,
+                                                    pairs[3].ctypes.data, m)
+                        if len(rest_rows) != rows:    # rows are numbered among those of this launch
+                            number = {r: q for q, r in enumerate(rest_rows)}
+                            pairs = pairs[:, [c for c in range(m) if int(pairs[0, c]) in number]]
+                            pairs[0] = [number[int(r)] for r in pairs[0]]
+                    more = (None, pairs)
+                else:
+                    contexts = []
+                    for r in rest_rows:
+                        if penalty[r] != 1.0:
+                            m = lib.gbh_sched_row_context(h, r, None, 0)
+                            cb = (C.c_int32 * max(1, m))()
+                            lib.gbh_sched_row_context(h, r, cb, m)
+                            contexts.append(list(cb[:m]))
+                        else:
+                            contexts.append([])
+                    more = (contexts,)
+                got = self.sample_fn(logits, configs, pick(uniforms), *more)
+            if more is None:
+                for q, r in enumerate(rest_rows):
+                    tokens[r] = got[q]
+            else:
+                for q, r in enumerate(rest_rows):
+                    tokens[r], cands[r] = got[0][q], got[1][q]
+        if greedy and self.sample_fn is sample_rows:
+            self._run_ahead(ids, starts, counts, wanted, tokens)     # the step that follows, before this one is read
+        tokens = token_values(tokens)                                # (waits for this step)
         lib.gbh_sched_finish(h, (C.c_int32 * max(1, rows))(*tokens), (C.c_int32 * max(1, rows))(*cands), rows)
         finished = self._drain_events()
         self._steps += 1
         self._record(t0, batch_desc, finished)
         return True
+
+    def _run_ahead(self, ids, starts, counts, wanted, tokens) -> None:
+        """Launches the step that follows a step in which every live request has just sampled greedily: one token for
+        each request that its length lets go on.  Nothing is launched when a live request is still in its prompt
+        (the next step then brings portions too, and would read the weights twice if it were cut in two), when the
+        engine cannot (``Engine.runs_ahead``), or when the pages do not suffice; the next plan is made as ever and
+        takes from here what fits it.  A request that the next plan admits runs its first portion in a launch of
+        its own, beside the rows computed ahead."""
+        eng, lib, h = self.engine, self._lib, self._h
+        if not self.config.run_ahead or len(wanted) != lib.gbh_sched_running(h):
+            return
+        entries, far, positions, inputs = [], [], [], []
+        for r, i in enumerate(wanted):
+            rid = ids[i]
+            out, limit = self.outputs[rid], self._limits.get(rid)
+            if limit is None or not isinstance(tokens[r], PendingToken):
+                return
+            generated = len(out.tokens) + 1
+            if generated >= limit[0] or limit[1] + generated >= self._max_pos:
+                continue                                             # ends with this token whatever it is
+            entries.append((rid, [tokens[r]], [0]))
+            far.append(counts[i])
+            positions.append(starts[i] + counts[i])
+            inputs.append(tokens[r])
+        if not entries or not eng.runs_ahead(entries):
+            return
+        try:
+            for (rid, _, _), k in zip(entries, far):
+                eng.cache.reserve(rid, k + 1)                        # this step's tokens and the next one
+        except OutOfPages:
+            return                                                   # (pages taken so far are the requests' own: the plan wants them too)
+        logits = eng.run_reserved(entries, validated=True, ahead=far)
+        self.ahead_rows["launched"] += len(entries)
+        self._ahead = _Ahead({e[0]: j for j, e in enumerate(entries)}, positions, inputs, greedy_pending(logits))
 
     def run(self, max_steps: int = 1 << 30) -> None:
         steps = 0
@@ -237,6 +339,7 @@ class Scheduler:
                 else:
                     out.finish = FINISH_NAMES[vals[i]]
                     finished.append(ids[i])
+                    self._limits.pop(ids[i], None)
                     self._arrival.pop(ids[i], None)
                     self._last_token.pop(ids[i], None)
             if n <= cap:

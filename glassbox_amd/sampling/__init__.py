@@ -1,3 +1,4 @@
-from .sampler import Rng, Sampler, SamplerConfig, host_sample, sample_rows
+from .pending import PendingToken, PendingTokens
+from .sampler import Rng, Sampler, SamplerConfig, greedy_pending, host_sample, sample_rows
 
-__all__ = ["Rng", "Sampler", "SamplerConfig", "host_sample", "sample_rows"]
+__all__ = ["PendingToken", "PendingTokens", "Rng", "Sampler", "SamplerConfig", "greedy_pending", "host_sample", "sample_rows"]

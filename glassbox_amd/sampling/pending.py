@@ -1,0 +1,77 @@
+"""Tokens that a sampler has left on the device.
+
+A step's sampled tokens are the next step's input.  Read back first, they leave the GPU idle while the host
+fetches them, prepares the next step's metadata and launches it.  ``PendingTokens`` lets the next step take
+them from device memory instead: ``Engine.step`` accepts a ``PendingToken`` wherever a request brings one
+token, launches the step, and only then asks for the value (the cache manager keeps every request's tokens),
+which has arrived by the time the step before has ended.  So the host runs one step ahead of the GPU, and the
+GPU goes from one step into the next.  Greedy rows only: a drawn token's generator advances or not with the
+number of candidates, which the host would know a step late.
+"""
+from __future__ import annotations
+
+from typing import List, Optional
+
+import torch
+
+
+class PendingTokens:
+    """One sampled token per row, int32 on the device, on their way into pinned host memory."""
+
+    def __init__(self, tensor: torch.Tensor):
+        if tensor.dtype != torch.int32 or tensor.dim() != 1 or not tensor.is_cuda:
+            raise ValueError("pending tokens are a one-dimensional int32 tensor on the GPU")
+        self.tensor = tensor
+        self._host = torch.empty(tensor.shape[0], dtype=torch.int32, pin_memory=True)
+        self._host.copy_(tensor, non_blocking=True)
+        self._arrived = torch.cuda.Event()
+        self._arrived.record()
+        self._values: Optional[List[int]] = None
+
+    def __len__(self) -> int:
+        return self.tensor.shape[0]
+
+    def __getitem__(self, row: int) -> "PendingToken":
+        if not 0 <= row < len(self):
+            raise IndexError(row)
+        return PendingToken(self, row)
+
+    def tolist(self) -> List[int]:
+        """The values; waits until the kernels that made them have run."""
+        if self._values is None:
+            self._arrived.synchronize()
+            self._values = self._host.tolist()
+        return self._values
+
+
+class PendingToken:
+    """Row ``row`` of ``source``: a token id that a step can take from the device before the host knows it."""
+    __slots__ = ("source", "row")
+
+    def __init__(self, source: PendingTokens, row: int):
+        self.source, self.row = source, row
+
+    def value(self) -> int:
+        return self.source.tolist()[self.row]
+
+
+def token_values(tokens) -> List[int]:
+    """The ids of a request's tokens, pending ones read back."""
+    return [t.value() if isinstance(t, PendingToken) else t for t in tokens]
+
+
+def place_pending(dst: torch.Tensor, items) -> None:
+    """Writes pending tokens into ``dst`` (int32 token ids of a step, on the device): ``items`` are
+    (row of dst, PendingToken).  Runs of neighbouring rows from neighbouring rows of one source are one copy."""
+    by_source = {}
+    for row, tok in items:
+        by_source.setdefault(id(tok.source), (tok.source, []))[1].append((row, tok.row))
+    for source, pairs in by_source.values():
+        at = 0
+        while at < len(pairs):
+            end = at + 1
+            while end < len(pairs) and pairs[end][0] == pairs[end - 1][0] + 1 and pairs[end][1] == pairs[end - 1][1] + 1:
+                end += 1
+            (d0, s0), k = pairs[at], end - at
+            dst[d0:d0 + k].copy_(source.tensor[s0:s0 + k], non_blocking=True)
+            at = end

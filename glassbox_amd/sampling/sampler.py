@@ -18,6 +18,7 @@ import numpy as np
 import torch
 
 from .. import build, ops
+from .pending import PendingTokens
 
 _MASK = (1 << 64) - 1
 
@@ -110,6 +111,15 @@ def sample_rows(logits: torch.Tensor, configs: Sequence[SamplerConfig], uniforms
     ops.sample(logits, fl[0], par[4], fl[1], fl[2], fl[3], out[0], out[1])
     both = out.tolist()
     return both[0], both[1]
+
+
+def greedy_pending(logits: torch.Tensor) -> PendingTokens:
+    """The largest logit of every row, left on the device: the next step can take the tokens from there
+    (``Engine.step`` accepts them) while the host still waits for their values."""
+    out = torch.empty(logits.shape[0], dtype=torch.int32, device=logits.device)
+    if logits.shape[0]:
+        ops.argmax(logits, out)
+    return PendingTokens(out)
 
 
 class Sampler:

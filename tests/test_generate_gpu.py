@@ -196,6 +196,57 @@ def assert_greedy(folder, prompts, outs, steps, dtype, what):
     assert compared >= 0.6 * steps * len(prompts), f"{what}, {dtype}: the comparison ended early too often"
 
 
+@pytest.mark.parametrize("dtype,graphs", [("bfloat16", True), ("bfloat16", False), ("float32", True)])
+def test_a_step_takes_sampled_tokens_from_the_device(model_dirs, dtype, graphs):
+    """``greedy_pending`` leaves a step's tokens on the device and ``Engine.step`` takes them from there (the host reads
+    their values after the launch): the same logits, bit for bit, as with tokens read back first.  Rows in another
+    order than the sampler left them, a request that sits a step out, a pending token beside another request's
+    prompt portion (the general path), and the cache manager's record of the tokens, which a later request with the
+    same beginning finds."""
+    from glassbox_amd.engine import Engine
+    from glassbox_amd.sampling import PendingToken, greedy_pending
+    folder = model_dirs.get("B")
+    vocab = helpers.TINY["B"]["vocab_size"]
+    prompts = {r: helpers.random_tokens(vocab, n, seed=80 + i) for i, (r, n) in enumerate({"a": 30, "b": 17, "c": 44}.items())}
+    late, first = (Engine(folder, dtype=dtype, max_tokens=1024, max_seqs=8, graph_decode=graphs, prefix_caching=True)
+                   for _ in range(2))
+    wants = [(r, p, [len(p) - 1]) for r, p in prompts.items()]
+    order = ["a", "b", "c"]
+    sampled = greedy_pending(late.step(wants))
+    tok_late = {r: sampled[i] for i, r in enumerate(order)}               # each request's newest token: on the device
+    tok_first = dict(zip(order, first.step(wants).argmax(-1).tolist()))   # and read back
+    history = {r: [] for r in order}
+    schedule = [["a", "b", "c"], ["c", "a", "b"], ["b", "c"], ["b", "c"], ["c", "b"]] + [["c", "b"]] * 20
+    for step, live in enumerate(schedule):
+        e_late = [(r, [tok_late[r]], [0]) for r in live]
+        e_first = [(r, [tok_first[r]], [0]) for r in live]
+        if step == 3:     # request a comes back with a prompt portion beside the others' pending tokens
+            extra = helpers.random_tokens(vocab, 9, seed=99)
+            e_late.insert(0, ("a", [tok_late["a"]] + extra, [9]))
+            e_first.insert(0, ("a", [tok_first["a"]] + extra, [9]))
+            live = ["a"] + live
+        assert all(isinstance(toks[0], PendingToken) for _, toks, _ in e_late)
+        for r, toks, _ in e_first:
+            history[r] += toks
+        l_late, l_first = late.step(e_late), first.step(e_first)
+        assert torch.equal(l_late, l_first), f"step {step}: logits differ with tokens taken from the device"
+        sampled = greedy_pending(l_late)
+        tok_first.update(zip(live, l_first.argmax(-1).tolist()))
+        tok_late.update({r: sampled[i] for i, r in enumerate(live)})
+        assert sampled.tolist() == [tok_first[r] for r in live]
+    if graphs:
+        assert late.decode_graphs.replays >= 15
+    # what the cache manager recorded are the values: a request with the same beginning finds the pages
+    for eng in (late, first):
+        eng.cache.check_invariants()
+        whole = prompts["c"] + history["c"]
+        assert eng.request_len("c") == len(whole)
+        assert eng.add_request("again", whole) == (len(whole) - 1) // 16 * 16
+        for r in ("a", "b", "c", "again"):
+            eng.end_request(r)
+        assert eng.cache.used_pages() == 0
+
+
 @pytest.mark.parametrize("name", ["A", "B", "D"])
 def test_greedy_generation_through_the_entry_point(model_dirs, name):
     """generate() against the plain implementation's greedy decoding: the first tiny configuration with its

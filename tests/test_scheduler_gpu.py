@@ -31,14 +31,16 @@ def serve(eng, prompts, max_tokens, samplers=None, budget=16, max_seqs=4, abort_
     records = []
     inner = eng.run_reserved
 
-    def spy(entries, validated=False):
-        at = [eng.cache.seq_len(sid) for sid, _, _ in entries]
-        logits = inner(entries, validated)
+    early = []   # rows of steps launched ahead of their plan: kept if the request got as far as their position
+
+    def spy(entries, validated=False, ahead=None):
+        at = [eng.cache.seq_len(sid) + (ahead[j] if ahead else 0) for j, (sid, _, _) in enumerate(entries)]
+        logits = inner(entries, validated, ahead)
         rows = logits.float().cpu().numpy()
         row = 0
         for (sid, toks, want), first in zip(entries, at):
             for w in want:
-                records.append((index[sid], first + w, rows[row].copy()))
+                (early if ahead else records).append((index[sid], first + w, rows[row].copy()))
                 row += 1
         assert row == rows.shape[0]
         return logits
@@ -62,7 +64,10 @@ def serve(eng, prompts, max_tokens, samplers=None, budget=16, max_seqs=4, abort_
                     eng.cache.check_invariants()
     finally:
         del eng.run_reserved
-    return [sched.outputs[i].tokens for i in ids], sched, records
+    replies = [sched.outputs[i].tokens for i in ids]
+    # a row that ran ahead for a request that then stopped or was aborted stands for no position of its reply
+    records += [r for r in early if r[1] < len(prompts[r[0]]) + len(replies[r[0]])]
+    return replies, sched, records
 
 
 def check_records(folder, prompts, replies, records, dtype, tol, what):

@@ -187,6 +187,67 @@ def test_stop_tokens_end_replies_on_the_device(model_dirs, dtype):
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("name", ["B", "D"])
+def test_steps_launched_ahead_of_their_plan_change_nothing(model_dirs, bf16_bound, name, dtype):
+    """When every live request decodes greedily the scheduler launches the next step before it has read this one's
+    tokens (``SchedulerConfig.run_ahead``).  Replies and finish reasons are those of a scheduler that
+    does not; rows that ran ahead were used (most of them) and dropped (a request stopped by a stop token, one
+    aborted, requests preempted in a pool of few pages, a request that arrives in the middle and whose prompt runs
+    beside rows computed ahead); every row of logits, also of the steps that ran ahead, is the plain
+    implementation's; requests that sample with a temperature keep their steps from running ahead."""
+    from glassbox_amd.engine import Engine, Scheduler, SchedulerConfig
+    from glassbox_amd.sampling import SamplerConfig
+    folder = model_dirs.get(name)
+    vocab = helpers.TINY[name]["vocab_size"]
+    prompts = [helpers.random_tokens(vocab, n, seed=200 + n) for n in (9, 40, 70, 3, 25, 17)]
+    # free replies first, to find a stop token that the first reply reaches in its middle
+    eng = Engine(folder, dtype=dtype, max_tokens=9 * 16, max_seqs=6, prefix_caching=True, graph_decode=True)
+    free, _, _ = serve(eng, prompts, max_tokens=20, budget=16, max_seqs=6)
+    full = {f"r{i}": p + r for i, (p, r) in enumerate(zip(prompts, free))}
+    tol = helpers.TOL_F32 if dtype == "float32" else bf16_bound.get(folder, full)
+    first = free[0]
+    at = next((i for i in range(4, 20) if first[i] not in first[:i]), None)
+    stop = [first[at]] if at is not None else []
+
+    def run(ahead):
+        sched = Scheduler(eng, SchedulerConfig(token_budget=16, max_seqs=6, run_ahead=ahead))
+        ids = [sched.submit(p, 20, stop=stop) for p in prompts[:5]]
+        steps = 0
+        while not sched.is_idle():
+            sched.step()
+            eng.cache.check_invariants()
+            steps += 1
+            if steps == 9:
+                ids.append(sched.submit(prompts[5], 20, stop=stop))     # arrives while the others decode
+            if steps == 14:
+                sched.abort(ids[1])
+        outs = [(sched.outputs[i].tokens, sched.outputs[i].finish) for i in ids]
+        assert eng.cache.used_pages() == 0
+        return outs, sched
+
+    plain_outs, plain_sched = run(False)
+    ahead_outs, ahead_sched = run(True)
+    assert ahead_outs == plain_outs
+    assert plain_sched.ahead_rows == {"launched": 0, "served": 0}
+    rows = ahead_sched.ahead_rows
+    assert rows["launched"] >= rows["served"] >= 20, rows    # (launched in vain: for a request that then stopped or was aborted)
+    # (the number of steps may differ by a few where the pool is nearly full: the pages of rows that run ahead are
+    # taken before the plan looks for room to admit a waiting request, not after)
+    for key in ("requests_finished", "generated_tokens"):
+        assert ahead_sched.metrics[key] == plain_sched.metrics[key], key
+    assert any(f == "stop" for _, f in ahead_outs) or not stop
+    assert ahead_outs[1][1] == "aborted"
+    # at the level of logits, rows that ran ahead included (serve records them when the reply got that far)
+    replies, sched, records = serve(eng, prompts, max_tokens=20, budget=16, max_seqs=6)
+    assert replies == free and sched.ahead_rows["served"] >= 20 and sched.metrics["preemptions"] > 0
+    check_records(folder, prompts, replies, records, dtype, tol, f"{name}: steps launched ahead")
+    # requests that draw: every step waits for its tokens (whether a draw took place decides the next random number)
+    drawn = [SamplerConfig(temperature=0.8, seed=3 + i) for i in range(6)]
+    _, sched, _ = serve(eng, prompts, max_tokens=6, samplers=drawn, budget=64, max_seqs=6)
+    assert sched.ahead_rows["launched"] == 0
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 @pytest.mark.parametrize("name,count", [("E", 72), ("M", 96)])
 def test_more_than_sixty_four_requests_decode_together(model_dirs, bf16_bound, name, count, dtype):
     """Seventy-two and ninety-six requests whose last twelve tokens are decoded in the same steps: a graph of more
