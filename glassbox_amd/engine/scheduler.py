@@ -13,13 +13,14 @@ import ctypes as C
 import time
 
 import numpy as np
+import torch
 from dataclasses import dataclass, field
 from typing import Dict, List, Optional, Sequence, Tuple
 
 from .. import build
 from ..cache.manager import OutOfPages
-from ..sampling.pending import PendingToken, PendingTokens, token_values
-from ..sampling.sampler import SamplerConfig, greedy_pending, sample_rows
+from ..sampling.pending import PendingToken, token_values
+from ..sampling.sampler import SamplerConfig, sample_rows, sample_rows_pending
 
 STOP, LENGTH, ABORTED = 0, 1, 2
 FINISH_NAMES = {STOP: "stop", LENGTH: "length", ABORTED: "aborted"}
@@ -66,7 +67,7 @@ class SchedulerConfig:
     """scheduler.rs:54-74.  The number of pages is the engine's (its ``max_tokens``)."""
     token_budget: int = 256
     max_seqs: int = 32
-    #: launch the step that is bound to follow a greedy decoding step before this one's tokens are read (``Scheduler.step``)
+    #: launch the step that is bound to follow a decoding step before this one's tokens are read (``Scheduler.step``)
     run_ahead: bool = True
 
 
@@ -92,11 +93,12 @@ class StepRecord:
 @dataclass
 class _Ahead:
     """A step launched before the step before it was accounted for: the request of each row, the position and the
-    (pending) token it ran with, and what it sampled."""
+    (pending) token it ran with, and its logits (a view of the engine's buffers: sampled at the next call, before
+    anything else is launched)."""
     row_of: Dict[int, int]
     positions: List[int]
     inputs: List[PendingToken]
-    sampled: PendingTokens
+    logits: "torch.Tensor"
 
 
 class Scheduler:
@@ -173,13 +175,14 @@ class Scheduler:
 
         The host library knows a step's sampled tokens only when ``finish`` is told them, and plans the next step
         from them; with nothing else done, the GPU would wait between steps for the read-back, the bookkeeping, the
-        plan and the launch.  So when every live request decodes greedily, the step that is bound to follow (one
-        token for each request that goes on, the token taken from the device: ``sampling.PendingToken``) is
-        launched *before* this step's tokens are read, beyond the pages and positions of this step
-        (``Engine.run_reserved(..., ahead=...)``).  The next call plans as ever and finds the rows it needs already
-        computed: an entry is served by a row that ran ahead if it is the same request at the same position with the
-        same token; what the plan holds besides (a new request's prompt) runs as a launch of its own, and rows
-        that ran ahead for nothing (the request stopped, was aborted or preempted) are dropped.  Every request's
+        plan and the launch.  So when every live request has just sampled, the step that is bound to follow (one
+        token for each request that its length lets go on, the token taken from the device:
+        ``sampling.PendingToken``) is launched *before* this step's tokens are read, beyond the pages and positions
+        of this step (``Engine.run_reserved(..., ahead=...)``).  The next call plans as ever and finds the rows it
+        needs already computed: an entry is served by a row that ran ahead if it is the same request at the same
+        position with the same token.  Such rows are sampled now, with the parameters and random numbers that the plan
+        gives, like any other; what the plan holds besides (a new request's prompt) runs as a launch of its own, and
+        rows that ran ahead for nothing (the request stopped, was aborted or preempted) are dropped.  Every request's
         tokens are those of the plain sequence; where the pool is nearly full a waiting request may be admitted a step
         later than there, because the pages of the rows that ran ahead are taken before the plan looks for room."""
         t0 = time.perf_counter()
@@ -211,83 +214,94 @@ class Scheduler:
             entries.append((ids[i], toks, [counts[i] - 1] if wants[i] else []))
             batch_desc.append((ids[i], "decode" if decodes[i] else "prefill", counts[i]))
             at += counts[i]
-        # prompt ids were checked when the request was submitted and sampled ids lie below the vocabulary by construction
         self.ahead_rows["served"] += len(served)
-        rest = [e for i, e in enumerate(entries) if i not in served]
-        logits = self.engine.run_reserved(rest, validated=True)
-        wanted = [i for i in range(n) if wants[i]]                  # the entry of every row
-        rest_rows = [r for r, i in enumerate(wanted) if i not in served]
+        wanted = [i for i in range(n) if wants[i]]                  # the entry of every row of logits
         rows = len(wanted)
         # sampling parameters of every wanted row: temperature, top_p, min_p, penalty, uniform | top_k, skip
         fl, it = np.empty((5, max(1, rows)), np.float32), np.empty((2, max(1, rows)), np.int32)
         lib.gbh_sched_rows_params(h, rows, fl[0].ctypes.data, it[0].ctypes.data, fl[1].ctypes.data, fl[2].ctypes.data,
                                   fl[3].ctypes.data, fl[4].ctypes.data, it[1].ctypes.data)
-        temp, top_p, min_p, penalty, uniforms = (a[:rows] for a in fl.tolist())
-        top_k = it[0].tolist()[:rows]
-        greedy = bool(rows) and max(temp) <= 0.0 and all(p == 1.0 for p in penalty)
+        params = [a[:rows] for a in fl.tolist()] + [it[0].tolist()[:rows]]
         tokens: List = [None] * rows      # ints, or tokens still on the device
-        cands = [1] * rows
-        for r, i in enumerate(wanted):
-            if i in served:
-                tokens[r] = before.sampled[served[i]]
-        if rest_rows:
-            pick = lambda a: [a[r] for r in rest_rows]
-            if self.sample_fn is sample_rows and greedy:
-                got, more = greedy_pending(logits), None
-            elif self.sample_fn is sample_rows and max(pick(temp)) <= 0.0 and all(p == 1.0 for p in pick(penalty)):
-                k = len(rest_rows)
-                got, more = self.sample_fn(logits, self._greedy[:k] if k <= len(self._greedy) else [SamplerConfig()] * k,
-                                           pick(uniforms)), ()
-            else:
-                configs = [SamplerConfig(temp[r], top_k[r], top_p[r], min_p[r], penalty[r]) for r in rest_rows]
-                if self.sample_fn is sample_rows:
-                    # the native scheduler keeps count of every such request's tokens: (row, token, occurrences, penalty)
-                    m = lib.gbh_sched_penalty_pairs(h, None, None, None, None, 0) if any(p != 1.0 for p in penalty) else 0
-                    pairs = np.empty((4, m), np.int32)
-                    if m:
-                        lib.gbh_sched_penalty_pairs(h, pairs[0].ctypes.data, pairs[1].ctypes.data, pairs[2].ctypes.data,
-                                                    pairs[3].ctypes.data, m)
-                        if len(rest_rows) != rows:    # rows are numbered among those of this launch
-                            number = {r: q for q, r in enumerate(rest_rows)}
-                            pairs = pairs[:, [c for c in range(m) if int(pairs[0, c]) in number]]
-                            pairs[0] = [number[int(r)] for r in pairs[0]]
-                    more = (None, pairs)
-                else:
-                    contexts = []
-                    for r in rest_rows:
-                        if penalty[r] != 1.0:
-                            m = lib.gbh_sched_row_context(h, r, None, 0)
-                            cb = (C.c_int32 * max(1, m))()
-                            lib.gbh_sched_row_context(h, r, cb, m)
-                            contexts.append(list(cb[:m]))
-                        else:
-                            contexts.append([])
-                    more = (contexts,)
-                got = self.sample_fn(logits, configs, pick(uniforms), *more)
-            if more is None:
-                for q, r in enumerate(rest_rows):
-                    tokens[r] = got[q]
-            else:
-                for q, r in enumerate(rest_rows):
-                    tokens[r], cands[r] = got[0][q], got[1][q]
-        if greedy and self.sample_fn is sample_rows:
-            self._run_ahead(ids, starts, counts, wanted, tokens)     # the step that follows, before this one is read
-        tokens = token_values(tokens)                                # (waits for this step)
+        cands: List = [1] * rows
+        # the rows that ran ahead first: the launch below may write where their logits lie
+        mine = [(r, served[i]) for r, i in enumerate(wanted) if i in served]
+        if mine:
+            js = [j for _, j in mine]
+            logits = before.logits
+            if js != list(range(logits.shape[0])):     # some of its rows only (through pinned memory: no wait for the stream)
+                pick = torch.tensor(js, dtype=torch.int64).pin_memory().to(logits.device, non_blocking=True)
+                logits = logits.index_select(0, pick)
+            self._sample(logits, [r for r, _ in mine], params, tokens, cands)
+        # prompt ids were checked when the request was submitted and sampled ids lie below the vocabulary by construction
+        rest = [e for i, e in enumerate(entries) if i not in served]
+        if rest:
+            logits = self.engine.run_reserved(rest, validated=True)
+            self._sample(logits, [r for r, i in enumerate(wanted) if i not in served], params, tokens, cands)
+        self._run_ahead(ids, starts, counts, wanted, tokens)         # the step that follows, before this one is read
+        tokens, cands = token_values(tokens), token_values(cands)   # (waits for this step)
         lib.gbh_sched_finish(h, (C.c_int32 * max(1, rows))(*tokens), (C.c_int32 * max(1, rows))(*cands), rows)
         finished = self._drain_events()
         self._steps += 1
         self._record(t0, batch_desc, finished)
         return True
 
+    def _sample(self, logits, rows: List[int], params, tokens: List, cands: List) -> None:
+        """Samples the rows of ``logits``, which are rows ``rows`` of the plan, into ``tokens`` and ``cands``: values, or
+        with the device sampler what it left on the device."""
+        if not rows:
+            return
+        lib, h = self._lib, self._h
+        temp, top_p, min_p, penalty, uniforms, top_k = ([a[r] for r in rows] for a in params)
+        device = self.sample_fn is sample_rows
+        if device and max(temp) <= 0.0 and all(p == 1.0 for p in penalty):
+            k = len(rows)
+            configs, more = self._greedy[:k] if k <= len(self._greedy) else [SamplerConfig()] * k, ()
+        else:
+            configs = [SamplerConfig(temp[q], top_k[q], top_p[q], min_p[q], penalty[q]) for q in range(len(rows))]
+            if device:
+                # the native scheduler keeps count of every such request's tokens: (row, token, occurrences, penalty)
+                m = lib.gbh_sched_penalty_pairs(h, None, None, None, None, 0) if any(p != 1.0 for p in penalty) else 0
+                pairs = np.empty((4, m), np.int32)
+                if m:
+                    lib.gbh_sched_penalty_pairs(h, pairs[0].ctypes.data, pairs[1].ctypes.data, pairs[2].ctypes.data,
+                                                pairs[3].ctypes.data, m)
+                    number = {r: q for q, r in enumerate(rows)}       # rows are numbered among those of these logits
+                    if list(number) != list(range(len(params[0]))):
+                        pairs = pairs[:, [c for c in range(m) if int(pairs[0, c]) in number]]
+                        pairs[0] = [number[int(r)] for r in pairs[0]]
+                more = (None, pairs)
+            else:
+                contexts = []
+                for q, r in enumerate(rows):
+                    if penalty[q] != 1.0:
+                        m = lib.gbh_sched_row_context(h, r, None, 0)
+                        cb = (C.c_int32 * max(1, m))()
+                        lib.gbh_sched_row_context(h, r, cb, m)
+                        contexts.append(list(cb[:m]))
+                    else:
+                        contexts.append([])
+                more = (contexts,)
+        if device and self.config.run_ahead:
+            got, many = sample_rows_pending(logits, configs, uniforms, *more)
+            for q, r in enumerate(rows):
+                tokens[r] = got[q]
+                if many is not None:
+                    cands[r] = many[q]
+        else:
+            got, many = self.sample_fn(logits, configs, uniforms, *more)
+            for q, r in enumerate(rows):
+                tokens[r], cands[r] = got[q], many[q]
+
     def _run_ahead(self, ids, starts, counts, wanted, tokens) -> None:
-        """Launches the step that follows a step in which every live request has just sampled greedily: one token for
-        each request that its length lets go on.  Nothing is launched when a live request is still in its prompt
+        """Launches the step that follows a step in which every live request has just sampled: one token for each
+        request that its length lets go on.  Nothing is launched when a live request is still in its prompt
         (the next step then brings portions too, and would read the weights twice if it were cut in two), when the
-        engine cannot (``Engine.runs_ahead``), or when the pages do not suffice; the next plan is made as ever and
-        takes from here what fits it.  A request that the next plan admits runs its first portion in a launch of
-        its own, beside the rows computed ahead."""
+        sampler is not the device's, when the engine cannot (``Engine.runs_ahead``), or when the pages do not suffice;
+        the next plan is made as ever and takes from here what fits it.  A request that the next plan admits runs
+        its first portion in a launch of its own, beside the rows computed ahead."""
         eng, lib, h = self.engine, self._lib, self._h
-        if not self.config.run_ahead or len(wanted) != lib.gbh_sched_running(h):
+        if not self.config.run_ahead or not wanted or len(wanted) != lib.gbh_sched_running(h):
             return
         entries, far, positions, inputs = [], [], [], []
         for r, i in enumerate(wanted):
@@ -311,7 +325,7 @@ class Scheduler:
             return                                                   # (pages taken so far are the requests' own: the plan wants them too)
         logits = eng.run_reserved(entries, validated=True, ahead=far)
         self.ahead_rows["launched"] += len(entries)
-        self._ahead = _Ahead({e[0]: j for j, e in enumerate(entries)}, positions, inputs, greedy_pending(logits))
+        self._ahead = _Ahead({e[0]: j for j, e in enumerate(entries)}, positions, inputs, logits)
 
     def run(self, max_steps: int = 1 << 30) -> None:
         steps = 0

@@ -5,8 +5,10 @@ fetches them, prepares the next step's metadata and launches it.  ``PendingToken
 them from device memory instead: ``Engine.step`` accepts a ``PendingToken`` wherever a request brings one
 token, launches the step, and only then asks for the value (the cache manager keeps every request's tokens),
 which has arrived by the time the step before has ended.  So the host runs one step ahead of the GPU, and the
-GPU goes from one step into the next.  Greedy rows only: a drawn token's generator advances or not with the
-number of candidates, which the host would know a step late.
+GPU goes from one step into the next.  ``greedy_pending`` and ``sample_rows_pending`` leave their results so; a
+draw also leaves its number of candidates, which decides whether the request's generator advances: a caller
+that draws needs it before it can name the next random number, so it samples a step's rows only when it has
+read the step before (``Scheduler.step`` does: it launches the next step ahead and samples it a call later).
 """
 from __future__ import annotations
 

@@ -76,6 +76,38 @@ def penalty_pairs(configs: Sequence[SamplerConfig], contexts: Optional[Sequence[
     return parts[0] if len(parts) == 1 else np.concatenate(parts, axis=1)
 
 
+def _to_device(array: np.ndarray, dev) -> torch.Tensor:
+    """A small host array on the device, through pinned memory: a copy out of pageable memory would make the host
+    wait for everything the stream still has to do."""
+    return torch.from_numpy(np.ascontiguousarray(array)).pin_memory().to(dev, non_blocking=True)
+
+
+def _sample_on_device(logits: torch.Tensor, configs: Sequence[SamplerConfig], uniforms: Sequence[float],
+                      contexts, pairs) -> Tuple[torch.Tensor, bool]:
+    """The launches of ``sample_rows``.  Returns (int32 [2, rows] on the device: tokens, candidates; whether the
+    second row was written: greedy rows have one candidate each)."""
+    rows, dev = logits.shape[0], logits.device
+    # the repetition penalty, once per occurrence of a token in the row's context
+    if pairs is None:
+        pairs = penalty_pairs(configs, contexts)
+    if pairs is not None and pairs.shape[1]:
+        p = _to_device(np.asarray(pairs, np.int32), dev)                         # one copy for the four columns
+        ops.penalize(logits, p[0], p[1], p[2], p[3].view(torch.float32))
+    out = torch.empty(2, rows, dtype=torch.int32, device=dev)
+    if all(cfg.temperature <= 0.0 for cfg in configs):
+        ops.argmax(logits, out[0])
+        return out, False
+    # temperature, top_p, min_p, the uniform number and top_k of every row: one copy, the numbers as their bits
+    host = np.empty((5, rows), np.int32)
+    host[:4].view(np.float32)[:] = ([c.temperature for c in configs], [c.top_p for c in configs],
+                                    [c.min_p for c in configs], list(uniforms))
+    host[4] = [c.top_k for c in configs]
+    par = _to_device(host, dev)
+    fl = par[:4].view(torch.float32)
+    ops.sample(logits, fl[0], par[4], fl[1], fl[2], fl[3], out[0], out[1])
+    return out, True
+
+
 def sample_rows(logits: torch.Tensor, configs: Sequence[SamplerConfig], uniforms: Sequence[float],
                 contexts: Optional[Sequence[Sequence[int]]] = None,
                 pairs: Optional[np.ndarray] = None) -> Tuple[List[int], List[int]]:
@@ -88,29 +120,26 @@ def sample_rows(logits: torch.Tensor, configs: Sequence[SamplerConfig], uniforms
     among; the caller advances the row's generator only if that is more than one, as the
     reference draws no number when a single candidate is left (sampler.rs:152-155)."""
     rows = logits.shape[0]
-    dev = logits.device
     if rows == 0:
         return [], []
-    # the repetition penalty, once per occurrence of a token in the row's context
-    if pairs is None:
-        pairs = penalty_pairs(configs, contexts)
-    if pairs is not None and pairs.shape[1]:
-        p = torch.from_numpy(np.ascontiguousarray(pairs, np.int32)).to(dev)      # one copy for the four columns
-        ops.penalize(logits, p[0], p[1], p[2], p[3].view(torch.float32))
-    out = torch.empty(2, rows, dtype=torch.int32, device=dev)
-    if all(cfg.temperature <= 0.0 for cfg in configs):
-        ops.argmax(logits, out[0])
+    out, drawn = _sample_on_device(logits, configs, uniforms, contexts, pairs)
+    if not drawn:
         return out[0].tolist(), [1] * rows
-    # temperature, top_p, min_p, the uniform number and top_k of every row: one copy, the numbers as their bits
-    host = np.empty((5, rows), np.int32)
-    host[:4].view(np.float32)[:] = ([c.temperature for c in configs], [c.top_p for c in configs],
-                                    [c.min_p for c in configs], list(uniforms))
-    host[4] = [c.top_k for c in configs]
-    par = torch.from_numpy(host).to(dev)
-    fl = par[:4].view(torch.float32)
-    ops.sample(logits, fl[0], par[4], fl[1], fl[2], fl[3], out[0], out[1])
     both = out.tolist()
     return both[0], both[1]
+
+
+def sample_rows_pending(logits: torch.Tensor, configs: Sequence[SamplerConfig], uniforms: Sequence[float],
+                        contexts: Optional[Sequence[Sequence[int]]] = None,
+                        pairs: Optional[np.ndarray] = None) -> Tuple[PendingTokens, Optional[PendingTokens]]:
+    """``sample_rows`` whose results stay on the device (``sampling.pending``): the tokens, which a next step can take
+    from there, and the candidates of every draw (None for rows that are all greedy: one each).  The host reads both
+    when it needs them."""
+    if logits.shape[0] == 0:
+        empty = torch.empty(0, dtype=torch.int32, device=logits.device)
+        return PendingTokens(empty), None
+    out, drawn = _sample_on_device(logits, configs, uniforms, contexts, pairs)
+    return PendingTokens(out[0]), (PendingTokens(out[1]) if drawn else None)
 
 
 def greedy_pending(logits: torch.Tensor) -> PendingTokens:

@@ -194,7 +194,7 @@ def test_steps_launched_ahead_of_their_plan_change_nothing(model_dirs, bf16_boun
     does not; rows that ran ahead were used (most of them) and dropped (a request stopped by a stop token, one
     aborted, requests preempted in a pool of few pages, a request that arrives in the middle and whose prompt runs
     beside rows computed ahead); every row of logits, also of the steps that ran ahead, is the plain
-    implementation's; requests that sample with a temperature keep their steps from running ahead."""
+    implementation's; requests that draw with a temperature and a penalty run ahead as well, with the same tokens."""
     from glassbox_amd.engine import Engine, Scheduler, SchedulerConfig
     from glassbox_amd.sampling import SamplerConfig
     folder = model_dirs.get(name)
@@ -241,10 +241,26 @@ def test_steps_launched_ahead_of_their_plan_change_nothing(model_dirs, bf16_boun
     replies, sched, records = serve(eng, prompts, max_tokens=20, budget=16, max_seqs=6)
     assert replies == free and sched.ahead_rows["served"] >= 20 and sched.metrics["preemptions"] > 0
     check_records(folder, prompts, replies, records, dtype, tol, f"{name}: steps launched ahead")
-    # requests that draw: every step waits for its tokens (whether a draw took place decides the next random number)
-    drawn = [SamplerConfig(temperature=0.8, seed=3 + i) for i in range(6)]
-    _, sched, _ = serve(eng, prompts, max_tokens=6, samplers=drawn, budget=64, max_seqs=6)
-    assert sched.ahead_rows["launched"] == 0
+    # requests that draw, some with a penalty: their steps run ahead too (a row that ran ahead is sampled once the plan
+    # has said with which random number), and a seeded run gives the tokens of a scheduler that launches nothing ahead
+    drawn = [SamplerConfig(temperature=0.8, top_k=(0, 40)[i % 2], top_p=(1.0, 0.9)[i % 3 == 0],
+                           repetition_penalty=(1.0, 1.3)[i % 2], seed=3 + i) for i in range(6)]
+
+    def draw(ahead):
+        sched = Scheduler(eng, SchedulerConfig(token_budget=64, max_seqs=6, run_ahead=ahead))
+        ids = [sched.submit(p, 14, s) for p, s in zip(prompts, drawn)]
+        sched.run()
+        assert eng.cache.used_pages() == 0
+        return [sched.outputs[i].tokens for i in ids], sched.ahead_rows
+
+    with_ahead, rows = draw(True)
+    without, none = draw(False)
+    assert rows["served"] >= 20 and none["launched"] == 0, (rows, none)
+    assert len({tuple(t) for t in with_ahead}) > 1
+    if dtype == "float32":    # (in bfloat16 a row's rounding depends on what else is in its launch, and a draw may tip)
+        assert with_ahead == without
+    else:
+        assert [len(t) for t in with_ahead] == [len(t) for t in without]
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
