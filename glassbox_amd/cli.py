@@ -141,7 +141,7 @@ def cmd_bench_single(a) -> int:
     import statistics
     import torch
     from .engine import Engine, Generator
-    from .sampling import SamplerConfig, sample_rows
+    from .sampling import greedy_pending
     pp, tg, reps = 512, 128, 3
     eng = Engine(a.model, dtype=a.dtype, max_tokens=pp + tg + 64, max_seqs=2)
     vocab = eng.model.vocab_size
@@ -158,7 +158,7 @@ def cmd_bench_single(a) -> int:
         tok = 1
         for _ in range(tg):
             logits = g.feed([tok])
-            tok = sample_rows(logits.reshape(1, -1), [SamplerConfig()], [0.0])[0][0]
+            tok = greedy_pending(logits.reshape(1, -1))[0]   # stays on the device for the next step (as in greedy())
         torch.cuda.synchronize(); d = tg / (time.time() - t)
         g.close()
         if rep > 0:
