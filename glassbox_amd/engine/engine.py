@@ -14,14 +14,14 @@ import torch
 from .. import ops
 from ..cache.manager import FULL, CacheManager, GroupSpec, OutOfPages
 from ..parts.base import LayerCache
-from ..sampling.pending import PendingToken, place_pending, token_values
+from ..sampling.pending import PendingToken, entry_values, place_pending
 from ..config import config_from_dir
 from ..weights.loader import build_model, compute_dtype, load_weights
 from .context import StepContext, Workspace
 from .decode_graphs import DecodeGraphs
 
-# (request, its next tokens, wanted places among them); a token may be a sampling.PendingToken, which the step takes
-# from the device
+# (request, its next tokens, wanted places among them); the first token may be a sampling.PendingToken, which the step
+# takes from the device
 Entry = Tuple[Hashable, Sequence[int], Sequence[int]]
 
 
@@ -255,7 +255,7 @@ class Engine:
         float32 logits [wanted, vocab] in the order of the entries and of their wanted places.
         The tensor is a view of the engine's workspace: use it before the next step.
 
-        A token may be a ``sampling.PendingToken`` (what ``sampling.greedy_pending`` left on the device): the step is
+        A request's first token may be a ``sampling.PendingToken`` (what ``sampling.greedy_pending`` left on the device): the step is
         launched with it, and its value is waited for only afterwards, for the cache manager's record of the
         request's tokens; a decoding loop then keeps the GPU one step behind the host, with no pause between steps."""
         entries = [(r, list(t), list(w)) for r, t, w in entries]
@@ -269,7 +269,7 @@ class Engine:
         by_id = [(self._ids[r], t, w) for r, t, w in entries]
         logits = self.run_reserved(by_id, validated=True)
         for sid, tokens, _ in by_id:
-            self.cache.commit(sid, token_values(tokens))   # (pending values: waits for the step before this one)
+            self.cache.commit(sid, entry_values(tokens))   # (a pending value: waits for the step before this one)
         return logits
 
     def _validate(self, entries) -> None:
@@ -277,8 +277,13 @@ class Engine:
         for request, tokens, want in entries:
             if not tokens:
                 raise EngineError(f"request {request!r} brings no tokens")
-            known = [t for t in tokens if not isinstance(t, PendingToken)]   # a sampler's tokens lie below the vocabulary
-            if known and (min(known) < 0 or max(known) >= vocab):
+            known = tokens[1:] if isinstance(tokens[0], PendingToken) else tokens   # a sampler's tokens lie below the vocabulary
+            try:
+                bad = bool(known) and (min(known) < 0 or max(known) >= vocab)
+            except TypeError:   # something in the list is no number
+                raise EngineError(f"request {request!r}: token ids must be integers (only the first may still lie on the "
+                                  f"device)") from None
+            if bad:
                 raise EngineError(f"request {request!r}: token ids must lie in 0..{vocab - 1}")
             if any(w < 0 or w >= len(tokens) for w in want):
                 raise EngineError(f"request {request!r}: wanted places must lie among its {len(tokens)} tokens")
@@ -358,9 +363,9 @@ class Engine:
         late = []   # (row, pending token): placed on the device after the copy
         for s, ei in enumerate(order):
             toks = entries[ei][1]
-            if any(isinstance(t, PendingToken) for t in toks):
-                late += [(q_start[s] + j, t) for j, t in enumerate(toks) if isinstance(t, PendingToken)]
-                toks = [0 if isinstance(t, PendingToken) else t for t in toks]
+            if isinstance(toks[0], PendingToken):
+                late.append((q_start[s], toks[0]))
+                toks = [0] + toks[1:]
             tok[q_start[s]:q_start[s] + q_len[s]] = toks
         hv[3 * n + S:3 * n + 2 * S] = q_len
         hv[3 * n + 4 * S:o_rows] = want_rows

@@ -12,7 +12,7 @@ from typing import List, Optional, Sequence, Union
 
 import torch
 
-from ..sampling.pending import token_values
+from ..sampling.pending import entry_values, token_values
 from ..sampling.sampler import SamplerConfig, greedy_pending
 from .engine import Engine
 from .scheduler import Scheduler, SchedulerConfig
@@ -28,11 +28,11 @@ class Generator:
         engine.add_request(name)
 
     def feed(self, tokens: Sequence[int]) -> torch.Tensor:
-        """Appends tokens and returns the logits after the last one (float32 [vocab] on the GPU).  A token may be
-        one that a sampler left on the device (``sampling.PendingToken``)."""
+        """Appends tokens and returns the logits after the last one (float32 [vocab] on the GPU).  The first token
+        may be one that a sampler left on the device (``sampling.PendingToken``)."""
         toks = list(tokens)
         logits = self.engine.step([(self.name, toks, [len(toks) - 1])])
-        self.tokens.extend(token_values(toks))   # (the step has read pending values back already)
+        self.tokens.extend(entry_values(toks))   # (the step has read a pending value back already)
         return logits[0]
 
     def truncate(self, length: int) -> None:

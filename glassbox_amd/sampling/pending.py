@@ -2,8 +2,8 @@
 
 A step's sampled tokens are the next step's input.  Read back first, they leave the GPU idle while the host
 fetches them, prepares the next step's metadata and launches it.  ``PendingTokens`` lets the next step take
-them from device memory instead: ``Engine.step`` accepts a ``PendingToken`` wherever a request brings one
-token, launches the step, and only then asks for the value (the cache manager keeps every request's tokens),
+them from device memory instead: ``Engine.step`` accepts a ``PendingToken`` as the first token that a request
+brings (alone, or ahead of tokens that the host knows), launches the step, and only then asks for the value (the cache manager keeps every request's tokens),
 which has arrived by the time the step before has ended.  So the host runs one step ahead of the GPU, and the
 GPU goes from one step into the next.  ``greedy_pending`` and ``sample_rows_pending`` leave their results so; a
 draw also leaves its number of candidates, which decides whether the request's generator advances: a caller
@@ -58,8 +58,16 @@ class PendingToken:
 
 
 def token_values(tokens) -> List[int]:
-    """The ids of a request's tokens, pending ones read back."""
+    """The values of a list in which any element may be pending."""
     return [t.value() if isinstance(t, PendingToken) else t for t in tokens]
+
+
+def entry_values(tokens) -> List[int]:
+    """The ids of the tokens a request brings to a step: only the first may be pending (what the step before
+    sampled), so that a long prompt portion is not searched."""
+    if tokens and isinstance(tokens[0], PendingToken):
+        return [tokens[0].value()] + list(tokens[1:])
+    return tokens
 
 
 def place_pending(dst: torch.Tensor, items) -> None:

@@ -236,6 +236,8 @@ def test_a_step_takes_sampled_tokens_from_the_device(model_dirs, dtype, graphs):
         assert sampled.tolist() == [tok_first[r] for r in live]
     if graphs:
         assert late.decode_graphs.replays >= 15
+    with pytest.raises(Exception, match="only the first"):
+        late.step([("b", [5, tok_late["b"]], [1])])
     # what the cache manager recorded are the values: a request with the same beginning finds the pages
     for eng in (late, first):
         eng.cache.check_invariants()
