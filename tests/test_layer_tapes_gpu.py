@@ -136,6 +136,27 @@ def test_layers_of_two_kinds_are_recorded_apart_and_a_block_named_twice_is_repla
         assert bad is None, f"request {r} ({len(toks)} tokens): first wrong position {bad[0]}, error {bad[1]:.3e}"
     longest = requests["r2"]
     assert np.abs(plain_two_kinds(longest) - plain_two_kinds(longest, windows=False))[8:].max() > 1e-3
+    # The scheduler launches steps ahead of their plan over windowed layers too (the pages that a window has passed go
+    # back when a step is committed, which is after the step that follows was launched: it reads none of them):
+    # the replies of a scheduler that launches nothing ahead, and the plain model's greedy ones.
+    from glassbox_amd.engine import Scheduler, SchedulerConfig
+    prompts, outs = list(requests.values()), {}
+    for ahead in (False, True):
+        eng = Engine(folder, dtype="float32", max_tokens=256, max_seqs=3, graph_decode=True)
+        sched = Scheduler(eng, SchedulerConfig(token_budget=16, max_seqs=3, run_ahead=ahead))
+        ids = [sched.submit(p, 30) for p in prompts]
+        while not sched.is_idle():
+            sched.step()
+            eng.cache.check_invariants()
+        outs[ahead] = [sched.outputs[i].tokens for i in ids]
+        assert eng.cache.used_pages(0) == 0 and eng.cache.used_pages(1) == 0
+        assert (sched.ahead_rows["served"] >= 60) == ahead, sched.ahead_rows
+    assert outs[True] == outs[False]
+    for p, out in zip(prompts, outs[True]):
+        toks = list(p)
+        for t in out[:12]:
+            assert int(plain_two_kinds(toks)[-1].argmax()) == t
+            toks.append(t)
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
