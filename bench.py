@@ -12,7 +12,8 @@ portions of 2,048 tokens) so that the last timed step reaches the context length
 times in a row, each time between synchronisations; ``ms_per_step`` and ``value`` are the mean over the
 repetitions and ``reps`` holds their spread; the batch 1 and 64 points are repeated as often, with their spread
 beside them (``points.decode_b1_sd``).  ``points.decode_b<batch>_scheduler`` is the same workload as
-requests under ``Scheduler.step`` (plan, step, sample, finish).  Prints one JSON line.  One GPU only: for
+requests under ``Scheduler.step`` (plan, step, sample, finish), ``points.decode_b<batch>_read_back_first`` the
+same steps with the tokens read back before each launch.  Prints one JSON line.  One GPU only: for
 --gpus > 1 it says so and exits with 2.
 """
 import argparse
@@ -146,7 +147,7 @@ def main() -> int:
                    "frac": round(pf_flops / pf / (peak * 1e12), 4)}
 
     # ---- decode: Engine.step and the device sampler, tokens fed back
-    def decode_run(batch, steps, warmup, reps):
+    def decode_run(batch, steps, warmup, reps, read_back_first=a.read_back_first):
         start = a.context - reps * steps - warmup
         names = [f"d{batch}_{i}" for i in range(batch)]
         prompts = [torch.randint(0, vocab, (start,), generator=g).tolist() for _ in names]
@@ -161,7 +162,7 @@ def main() -> int:
             # the sampled tokens stay on the device for the next step, which is launched before the host has their
             # values; Engine.step waits for them after the launch (the cache manager keeps every request's tokens)
             logits = eng.step([(name, [t], [0]) for name, t in zip(names, tokens)])
-            if a.read_back_first:
+            if read_back_first:
                 tokens, _ = sample_rows(logits, [SamplerConfig()] * batch, [0.0] * batch)
             else:
                 tokens = greedy_pending(logits)
@@ -215,6 +216,12 @@ def main() -> int:
         sdt = scheduler_run(a.batch, a.steps, a.warmup)
         points[f"decode_b{a.batch}_scheduler"] = round(a.batch * a.steps / sdt, 1)
     if not a.no_points:
+        if not a.read_back_first:
+            # the same steps with every step's tokens read back before the next is launched, as a caller must that
+            # looks at a token before it feeds it
+            k = max(8, min(a.steps, 32))
+            pts, _ = decode_run(a.batch, k, min(a.warmup, 4), 1, read_back_first=True)
+            points[f"decode_b{a.batch}_read_back_first"] = round(a.batch * k / pts[0], 1)
         for b in (1, 64):
             if b == a.batch:
                 points[f"decode_b{b}"] = round(value, 1)
