@@ -177,11 +177,11 @@ def compile_library(name: str, quiet: bool = False) -> str:
 def build_all(force: bool = True, names: Optional[List[str]] = None, jobs: int = 8) -> None:
     """Compile every library (or ``names``).  With ``force`` also those that are current."""
     todo = [n for n in (names or list(LIBRARIES)) if force or not is_current(n)]
-    if not todo:
-        return
-    with ThreadPoolExecutor(max_workers=max(1, min(jobs, len(todo)))) as pool:
-        list(pool.map(compile_library, todo))
-    _stamp_version()
+    if todo:
+        with ThreadPoolExecutor(max_workers=max(1, min(jobs, len(todo)))) as pool:
+            list(pool.map(compile_library, todo))
+    if names is None:
+        _stamp_version()   # also when nothing had to be compiled: the commit names the Python beside the libraries too
 
 
 def _git_commit() -> Optional[str]:
