@@ -119,6 +119,14 @@ def test_sampling_kernel_agrees_with_the_plain_sampler(vocab, spread):
     toks, cands = sample_rows(logits.to(DEV), cfgs, us, ctxs)
     for r in range(rows):
         check_sampled(logits[r].tolist(), ctxs[r], cfgs[r], us[r], toks[r], cands[r])
+    # the same left on the device (what a step launched ahead takes its tokens from), drawn and greedy rows
+    from glassbox_amd.sampling import sample_rows_pending
+    late_toks, late_cands = sample_rows_pending(logits.to(DEV), cfgs, us, ctxs)
+    assert late_toks.tolist() == toks and late_cands.tolist() == cands and late_toks[3].value() == toks[3]
+    greedy = [SamplerConfig(repetition_penalty=c.repetition_penalty) for c in cfgs]
+    want, _ = sample_rows(logits.to(DEV), greedy, us, ctxs)
+    late_toks, late_cands = sample_rows_pending(logits.to(DEV), greedy, us, ctxs)
+    assert late_toks.tolist() == want and late_cands is None
 
 
 def test_sampling_kernel_on_rows_of_ties_and_edge_settings():
