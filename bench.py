@@ -4,10 +4,11 @@
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--batch 8] [--context 4096] [--layers 24]
                     [--shapes smollm2-1.7b|smollm2-360m|llama-3-8b] [--reps 3]
 
-A step is one decode step of the whole batch through the path that greedy generation uses: ``Engine.step`` (which
-replays steps of single tokens from HIP graphs) and the device sampler (``sampling.greedy_pending``), the sampled
-tokens fed back as the next step's input: the step takes them from the device and the host reads every one of
-them while it runs (``--read-back-first`` reads them before the next step is launched, as a sampler that draws does).  The batch is first prefilled (through the same step function, in
+A step is one decode step of the whole batch through the path that greedy generation uses: ``Engine.step``
+(which replays steps of single tokens from HIP graphs) and the device sampler (``sampling.greedy_pending``), the
+sampled tokens fed back as the next step's input: the step takes them from the device and the host reads every
+one of them while it runs (``--read-back-first`` reads them before the next step is launched, as a caller must
+that looks at a token before it feeds it).  The batch is first prefilled (through the same step function, in
 portions of 2,048 tokens) so that the last timed step reaches the context length.  K steps are timed ``--reps``
 times in a row, each time between synchronisations; ``ms_per_step`` and ``value`` are the mean over the
 repetitions and ``reps`` holds their spread; the batch 1 and 64 points are repeated as often, with their spread

@@ -255,9 +255,10 @@ class Engine:
         float32 logits [wanted, vocab] in the order of the entries and of their wanted places.
         The tensor is a view of the engine's workspace: use it before the next step.
 
-        A request's first token may be a ``sampling.PendingToken`` (what ``sampling.greedy_pending`` left on the device): the step is
-        launched with it, and its value is waited for only afterwards, for the cache manager's record of the
-        request's tokens; a decoding loop then keeps the GPU one step behind the host, with no pause between steps."""
+        A request's first token may be a ``sampling.PendingToken`` (what ``sampling.greedy_pending`` left on the
+        device): the step is launched with it, and its value is waited for only afterwards, for the cache manager's
+        record of the request's tokens; a decoding loop then keeps the GPU one step behind the host, with no pause
+        between steps."""
         entries = [(r, list(t), list(w)) for r, t, w in entries]
         seen = set()
         for request, _, _ in entries:
@@ -277,7 +278,8 @@ class Engine:
         for request, tokens, want in entries:
             if not tokens:
                 raise EngineError(f"request {request!r} brings no tokens")
-            known = tokens[1:] if isinstance(tokens[0], PendingToken) else tokens   # a sampler's tokens lie below the vocabulary
+            # (a sampler's token lies below the vocabulary)
+            known = tokens[1:] if isinstance(tokens[0], PendingToken) else tokens
             try:
                 bad = bool(known) and (min(known) < 0 or max(known) >= vocab)
             except TypeError:   # something in the list is no number

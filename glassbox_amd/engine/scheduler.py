@@ -322,7 +322,7 @@ class Scheduler:
             for (rid, _, _), k in zip(entries, far):
                 eng.cache.reserve(rid, k + 1)                        # this step's tokens and the next one
         except OutOfPages:
-            return                                                   # (pages taken so far are the requests' own: the plan wants them too)
+            return     # (the pages taken so far are the requests' own: the plan wants them too)
         logits = eng.run_reserved(entries, validated=True, ahead=far)
         self.ahead_rows["launched"] += len(entries)
         self._ahead = _Ahead({e[0]: j for j, e in enumerate(entries)}, positions, inputs, logits)

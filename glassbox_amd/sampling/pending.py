@@ -3,12 +3,14 @@
 A step's sampled tokens are the next step's input.  Read back first, they leave the GPU idle while the host
 fetches them, prepares the next step's metadata and launches it.  ``PendingTokens`` lets the next step take
 them from device memory instead: ``Engine.step`` accepts a ``PendingToken`` as the first token that a request
-brings (alone, or ahead of tokens that the host knows), launches the step, and only then asks for the value (the cache manager keeps every request's tokens),
-which has arrived by the time the step before has ended.  So the host runs one step ahead of the GPU, and the
-GPU goes from one step into the next.  ``greedy_pending`` and ``sample_rows_pending`` leave their results so; a
-draw also leaves its number of candidates, which decides whether the request's generator advances: a caller
-that draws needs it before it can name the next random number, so it samples a step's rows only when it has
-read the step before (``Scheduler.step`` does: it launches the next step ahead and samples it a call later).
+brings (alone, or ahead of tokens that the host knows), launches the step, and only then asks for the value
+(the cache manager keeps every request's tokens), which has arrived by the time the step before has ended.
+So the host runs one step ahead of the GPU, and the GPU goes from one step into the next.
+
+``greedy_pending`` and ``sample_rows_pending`` leave their results so; a draw also leaves its number of
+candidates, which decides whether the request's generator advances: a caller that draws needs it before it can
+name the next random number, so it samples a step's rows only when it has read the step before
+(``Scheduler.step`` does: it launches the next step ahead and samples it a call later).
 """
 from __future__ import annotations
 
